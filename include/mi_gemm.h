@@ -1,0 +1,186 @@
+/* mi_gemm.h — C ABI of libmigemm.so, the gfx950 (MI355X) training-GEMM library.
+ *
+ * This is the drop-in boundary for vkgrad's matmul path.  The reference has no
+ * FFI of its own for this path (it drives Vulkan through ctypes), so each entry
+ * point below names the reference interface it replaces, as file:line under
+ * /root/reference/.
+ *
+ * Conventions
+ *   - every function returns int: 0 (MG_OK) on success, an MG_ERR_* code otherwise;
+ *     mg_last_error() then holds a message for the calling thread.
+ *   - no torch types, no C++ types, no exceptions cross this boundary.
+ *   - all device work of a context runs on one in-order HIP stream owned by the
+ *     context (the reference separates every dispatch by a full barrier on a
+ *     single queue: vk.py:834-851, 1317-1323).  A context is not thread-safe.
+ *   - argument validation happens before any HIP call (mg_gemm_check is the same
+ *     code mg_gemm runs first), so it can be exercised on a machine without a GPU.
+ *   - matrices are dense row-major; leading dimensions are in elements.
+ *       A is stored (M,K) [lda >= K], or (K,M) [lda >= M] in layout TN
+ *       B is stored (K,N) [ldb >= N], or (N,K) [ldb >= K] in layout NT
+ *       C is (M,N) float32 [ldc >= N]                 (kernels.py:42-43)
+ *     M, N, K are arbitrary positive integers (no tile-multiple requirement,
+ *     unlike kernels.py:265-276); operands need only 2-byte alignment, but
+ *     16-byte-aligned bases with ld % 8 == 0 take the fast path.
+ */
+#ifndef MI_GEMM_H
+#define MI_GEMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct mg_ctx mg_ctx;
+typedef struct mg_graph mg_graph;
+
+enum {
+    MG_OK = 0,
+    MG_ERR_ARG = 1,     /* bad argument; nothing was launched */
+    MG_ERR_HIP = 2,     /* a HIP runtime call failed */
+    MG_ERR_STATE = 3,   /* call not legal in the current state (graph capture etc.) */
+    MG_ERR_NOMEM = 4,
+    MG_ERR_NODEVICE = 5
+};
+
+/* operand layouts: the (trans_a, trans_b) pairs of kernels.py:32-33.  (T,T) is
+ * never used by any call site (autograd.py:186-228, transformer.py:89-104,
+ * 326-330, 362-371) and is not provided. */
+enum { MG_NN = 0, MG_NT = 1, MG_TN = 2 };
+/* input element types; accumulation and C are always float32 */
+enum { MG_F16 = 0, MG_BF16 = 1 };
+/* memory kinds of vk.py:1161-1175 */
+enum { MG_DEVICE = 0, MG_SHARED = 1, MG_CACHED = 2, MG_BAR = 3 };
+/* activations for the companion elementwise kernels */
+enum { MG_ACT_NONE = 0, MG_ACT_GELU = 1, MG_ACT_RELU = 2 };
+
+typedef struct {
+    int32_t struct_size;   /* sizeof(mg_gemm_args), checked */
+    int32_t layout;        /* MG_NN / MG_NT / MG_TN */
+    int32_t dtype;         /* MG_F16 / MG_BF16 */
+    int32_t beta;          /* 0: C is overwritten; 1: C += result (dW accumulation) */
+    int64_t m, n, k;
+    const void *a;  int64_t lda;
+    const void *b;  int64_t ldb;
+    float *c;       int64_t ldc;
+    const float *bias;     /* NULL, or N floats added to every row of the result */
+    int32_t nbatch;        /* >= 1; batch z uses a + z*sa, b + z*sb, c + z*sc (elements) */
+    int32_t tile;          /* tile id from mg_tile_info, or -1 for the built-in picker */
+    int64_t sa, sb, sc;
+    int32_t split_k;       /* 0 = picker decides, 1 = none, >1 = that many K slices */
+    int32_t group_m;       /* 0 = picker decides; else row-blocks per rasterisation band */
+} mg_gemm_args;
+
+typedef struct {
+    int32_t id;
+    int32_t bm, bn, bk;        /* block tile */
+    int32_t waves_m, waves_n;  /* 64-lane wavefronts per workgroup along M and N */
+    int32_t threads;
+    int32_t lds_bytes;         /* for the NT layout; other layouts differ by padding */
+    int32_t min_m;             /* informational: smallest M this tile is meant for */
+    char name[48];
+} mg_tile;
+
+typedef struct {
+    char name[128];
+    char arch[64];
+    int32_t compute_units;
+    int32_t clock_khz;
+    int32_t mem_clock_khz;
+    int32_t mem_bus_bits;
+    int32_t l2_bytes;
+    int32_t lds_bytes_per_cu;
+    int32_t wavefront;
+    int32_t reserved;
+    int64_t total_mem;
+} mg_device_info;
+
+/* ---- runtime: replaces vk.Device / vk.Buffer (vk.py:892-1357, 507-617) ---- */
+
+/* Device() — vk.py:892.  Fails with MG_ERR_NODEVICE when no HIP device exists. */
+int mg_init(int device_index, mg_ctx **out);
+/* Device.destroy — vk.py:1343 */
+int mg_destroy(mg_ctx *ctx);
+/* Device.name / shader_core_props — vk.py:1225-1240 */
+int mg_get_device_info(mg_ctx *ctx, mg_device_info *out);
+/* Device.buffer(size, kind) — vk.py:1251, 507-582.  *host_ptr is the CPU mapping of the
+ * same bytes for host-visible kinds (shared/cached/bar -> pinned, device-accessible
+ * host memory), NULL for MG_DEVICE. */
+int mg_alloc(mg_ctx *ctx, size_t nbytes, int kind, void **dev_ptr, void **host_ptr);
+/* Buffer.destroy — vk.py:607-617 */
+int mg_free(mg_ctx *ctx, void *dev_ptr, int kind);
+/* Device.copy(src, dst, size) — vk.py:1267-1293; any mix of device / host-visible
+ * pointers; returns after the copy has completed. */
+int mg_copy(mg_ctx *ctx, void *dst, const void *src, size_t nbytes);
+/* staged upload/download between ordinary host memory and a buffer */
+int mg_upload(mg_ctx *ctx, void *dst_dev, const void *src_host, size_t nbytes);
+int mg_download(mg_ctx *ctx, void *dst_host, const void *src_dev, size_t nbytes);
+/* fence wait — vk.py:1335; Buffer.flush/invalidate (vk.py:592-605) map to this */
+int mg_sync(mg_ctx *ctx);
+/* message for the last failing call on this thread — VkError text, vk.py:128-134 */
+const char *mg_last_error(void);
+
+/* ---- GEMM: replaces kernels.Matmul (kernels.py:232-315) ---- */
+
+/* Matmul.fits + the argument errors of kernels.py:274-276, vk.py:778-790; pure. */
+int mg_gemm_check(const mg_gemm_args *args);
+/* Matmul.__call__ — kernels.py:269-297 (eager: enqueue, do not wait). */
+int mg_gemm(mg_ctx *ctx, const mg_gemm_args *args);
+/* Device.run(kernel, ..., repeat) timing — vk.py:1295-1340, but timed with HIP
+ * events on the context's stream instead of host wall clock.  Launches the GEMM
+ * `repeat` times back to back, waits, and returns the total seconds. */
+int mg_gemm_time(mg_ctx *ctx, const mg_gemm_args *args, int repeat, double *seconds);
+/* CONFIGS — kernels.py:326-331: the tile table the tuner walks. */
+int mg_tile_count(void);
+int mg_tile_info(int id, mg_tile *out);
+/* Matmul.fits for one tile: 1 if tile `id` can run `args`, else 0. */
+int mg_tile_fits(int id, const mg_gemm_args *args);
+/* pick_config — autograd.py:22-41: heuristic choice without benchmarking; pure.
+ * Writes tile id, split_k and group_m it would use for `args` on a device with
+ * `compute_units` CUs. */
+int mg_pick(const mg_gemm_args *args, int compute_units, int *tile, int *split_k, int *group_m);
+
+/* ---- record / replay: replaces vk.Graph (vk.py:807-889) ---- */
+
+/* Graph.__init__: start capturing the context's stream; launches enqueue nothing
+ * until mg_graph_end. */
+int mg_graph_begin(mg_ctx *ctx);
+/* Graph.finish — vk.py:869-875 */
+int mg_graph_end(mg_ctx *ctx, mg_graph **out);
+/* Graph.submit — vk.py:877-889: replay and wait; *seconds = host wall time. */
+int mg_graph_launch(mg_ctx *ctx, mg_graph *g, double *seconds);
+int mg_graph_destroy(mg_ctx *ctx, mg_graph *g);
+
+/* ---- companion elementwise kernels: kernels.make_kernels (kernels.py:699-862) ----
+ * `dtype` is the 16-bit type of the narrowed outputs / mirrors (MG_F16 or MG_BF16). */
+
+/* bias_gelu / bias (kernels.py:709-718, 742-749): z = acc + bias[i % ncol];
+ * y16 = narrow(act(z)).  z and y16 may each be NULL; bias may be NULL (the GEMM's
+ * fused bias epilogue already added it). */
+int mg_ew_bias_act(mg_ctx *ctx, const float *acc, const float *bias, float *z, void *y16,
+                   int64_t n, int64_t ncol, int act, int dtype);
+/* bias_gelu_bwd (kernels.py:721-739): g = dy * act'(z); dz16 = narrow(g); dz32 = g (may be NULL). */
+int mg_ew_act_bwd(mg_ctx *ctx, const float *dy, const float *z, void *dz16, float *dz32,
+                  int64_t n, int act, int dtype);
+/* col_sum (kernels.py:753-761): sums[c] = sum_r g[r*ncol + c]; accumulate != 0 adds
+ * to the existing sums[c] instead (bias gradients over micro-batches). */
+int mg_ew_col_sum(mg_ctx *ctx, const float *g, float *sums, int64_t ncol, int64_t nrow, int accumulate);
+/* softmax_ce (kernels.py:766-791): per-row loss, gradient (p - onehot)/nrows in both
+ * precisions, classes >= ncls masked to zero. */
+int mg_ew_softmax_ce(mg_ctx *ctx, const float *logits, const uint32_t *labels, void *dl16,
+                     float *dl32, float *loss, int64_t nrows, int64_t stride, int64_t ncls, int dtype);
+/* adamw (kernels.py:832-851): hp = {lr, b1, b2, bc1, bc2, eps} read from memory. */
+int mg_ew_adamw(mg_ctx *ctx, float *w, const float *g, float *m, float *v, void *w16,
+                const float *hp, int64_t n, float wd, int dtype);
+/* zero (kernels.py:853-854) */
+int mg_ew_zero(mg_ctx *ctx, float *dst, int64_t n);
+/* cast16 (kernels.py:857-860) */
+int mg_ew_cast16(mg_ctx *ctx, const float *src, void *dst, int64_t n, int dtype);
+/* grad_add (dataparallel.py:54-58): dst[i] += src[i] */
+int mg_ew_grad_add(mg_ctx *ctx, float *dst, const float *src, int64_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI_GEMM_H */

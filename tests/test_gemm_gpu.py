@@ -1,0 +1,120 @@
+"""GPU parity: the HIP GEMM path against the oracle, through the C ABI.
+
+Cases and tolerances follow the reference's own kernel tests
+(/root/reference/test_kernels.py:10-95: five NN shapes and the two transposes at
+256^3 with max-abs/max-abs < 2e-3, and the ones-exact K=1024 case), tightened to
+the bar of this build: relative Frobenius error <= 1e-3 and elementwise
+rtol 1e-2 (with the absolute floor oracle.ref_gemm.elementwise_ok documents).
+Integer-valued inputs must match bit for bit in every accumulation order.
+"""
+
+import numpy as np
+import pytest
+
+from oracle import ref_gemm as O
+from tests.util import check_case, run_gemm
+
+pytestmark = pytest.mark.gpu
+
+LAYOUTS = {"NN": (False, False), "NT": (False, True), "TN": (True, False)}
+FRO_TOL = 1e-3
+MAXREL_TOL = 2e-3   # test_kernels.py:36
+
+
+def _assert_close(r, label):
+    assert r["finite"], f"{label}: non-finite output"
+    assert r["fro"] <= FRO_TOL, f"{label}: rel Frobenius {r['fro']:.3e}"
+    assert r["maxrel"] < MAXREL_TOL, f"{label}: max rel {r['maxrel']:.3e}"
+    assert r["elem_ok"], f"{label}: elementwise rtol 1e-2 violated"
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 256), (128, 128, 128), (512, 256, 128),
+                                    (256, 512, 256), (64, 64, 512)])
+def test_reference_shapes_nn(dev, m, n, k):
+    """test_kernels.py:48-59."""
+    r, _, _ = check_case(dev, m, n, k, seed=0)
+    _assert_close(r, f"NN {m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("layout", ["TN", "NT"])
+def test_reference_transposes(dev, layout):
+    """test_kernels.py:62-66."""
+    ta, tb = LAYOUTS[layout]
+    r, _, _ = check_case(dev, 256, 256, 256, ta, tb, seed=0)
+    _assert_close(r, f"{layout} 256^3")
+
+
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_ones_exact(dev, layout, dtype):
+    """test_kernels.py:69-95: K=1024 products of 1.0 sum to exactly 1024.0 only
+    with float32 accumulation."""
+    ta, tb = LAYOUTS[layout]
+    m = n = 64
+    k = 1024
+    one = np.float16(1.0) if dtype == "f16" else np.uint16(0x3F80)
+    a = np.full((k, m) if ta else (m, k), one)
+    b = np.full((n, k) if tb else (k, n), one)
+    got = run_gemm(dev, a, b, m, n, k, ta, tb, dtype)
+    assert np.all(got == float(k)), f"min {got.min()} max {got.max()}"
+
+
+def test_every_tile_every_layout_exact(dev):
+    """Integer inputs: exact in any summation order, so every tile, layout and
+    dtype must reproduce the oracle bit for bit on a ragged shape."""
+    from vkgrad_amd.kernels import CONFIGS
+    m, n, k = 300, 520, 200
+    for layout, (ta, tb) in LAYOUTS.items():
+        for dtype in ("f16", "bf16"):
+            for t in CONFIGS:
+                r, got, ref = check_case(dev, m, n, k, ta, tb, dtype, seed=3, tile=t["id"], integer=True,
+                                         bias=True, accumulate=True)
+                assert r["exact"], f"{layout} {dtype} tile {t['name']}: max diff {np.abs(got - ref).max()}"
+
+
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+def test_ragged_small_exact(dev, layout):
+    """Odd shapes (unaligned rows, K tails of every residue) through the
+    general-alignment kernels, bit exact on integer data."""
+    ta, tb = LAYOUTS[layout]
+    for m, n, k in [(1, 1, 1), (7, 5, 3), (33, 31, 17), (63, 96, 129), (129, 65, 67), (100, 257, 250),
+                    (31, 33, 1025)]:
+        r, got, ref = check_case(dev, m, n, k, ta, tb, "f16", seed=m + n + k, integer=True, bias=True)
+        assert r["exact"], f"{layout} {m}x{n}x{k}: max diff {np.abs(got - ref).max()}"
+
+
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+def test_split_k_exact_and_close(dev, layout):
+    ta, tb = LAYOUTS[layout]
+    for split in (2, 3, 8):
+        r, got, ref = check_case(dev, 192, 320, 2048, ta, tb, "bf16", seed=5, integer=True, split_k=split,
+                                 bias=True, accumulate=True, tile=3)
+        assert r["exact"], f"{layout} split {split}: max diff {np.abs(got - ref).max()}"
+        r, _, _ = check_case(dev, 192, 320, 2048, ta, tb, "bf16", seed=6, split_k=split, tile=3)
+        _assert_close(r, f"{layout} split {split}")
+
+
+def test_beta0_overwrites_nan(dev):
+    """dW with beta=0 doubles as the zeroing of a stale gradient
+    (transformer.py:367-370): a NaN-poisoned C must come back clean."""
+    for split in (1, 4):
+        r, _, _ = check_case(dev, 256, 256, 1024, True, False, "f16", seed=2, split_k=split)
+        _assert_close(r, f"TN poisoned split {split}")
+
+
+def test_wrong_layout_fails(dev):
+    """Negative control (idea: test_hf_gpt2.py:129-136): a square operand read
+    with the wrong layout passes every shape check and must fail on values."""
+    m = n = k = 256
+    a, b = O.make_operands(m, n, k, False, True, "f16", seed=9)       # B stored (n, k)
+    got_wrong = run_gemm(dev, a, b, m, n, k, False, False, "f16")      # read as (k, n)
+    ref = O.ref_gemm(a, b, False, True, "f16")
+    assert O.err_fro(got_wrong, ref) > 0.5
+
+
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_medium_random(dev, layout, dtype):
+    ta, tb = LAYOUTS[layout]
+    r, _, _ = check_case(dev, 1024, 768, 1536, ta, tb, dtype, seed=11, bias=True)
+    _assert_close(r, f"{layout} {dtype} 1024x768x1536")

@@ -1,0 +1,63 @@
+"""Shared helpers for the parity tests: run one GEMM through the library's
+Python surface (which goes through the C ABI) and build the oracle's answer."""
+
+import numpy as np
+
+from oracle import ref_gemm as O
+
+
+def stored_shapes(m, n, k, trans_a, trans_b):
+    return ((k, m) if trans_a else (m, k)), ((n, k) if trans_b else (k, n))
+
+
+def np16(dtype):
+    return np.float16 if dtype == "f16" else np.uint16
+
+
+def run_gemm(dev, a, b, m, n, k, trans_a=False, trans_b=False, dtype="f16", bias=None,
+             c_in=None, tile=None, split_k=0, group_m=0, kind="device", poison=True):
+    """a, b: stored operands (f16 arrays or bf16 bit patterns).  Returns C (m,n) f32."""
+    from vkgrad_amd.kernels import Matmul
+    ba = dev.buffer(max(a.nbytes, 2), kind)
+    bb = dev.buffer(max(b.nbytes, 2), kind)
+    bc = dev.buffer(m * n * 4, kind)
+    bbias = None
+    mm = Matmul(dev, trans_a=trans_a, trans_b=trans_b, tile=tile, dtype=dtype, split_k=split_k,
+                group_m=group_m)
+    try:
+        ba.upload(a)
+        bb.upload(b)
+        if c_in is not None:
+            bc.upload(np.ascontiguousarray(c_in, np.float32))
+        elif poison:
+            bc.upload(np.full((m, n), np.nan, np.float32))   # beta=0 must overwrite
+        if bias is not None:
+            bbias = dev.buffer(n * 4, kind)
+            bbias.upload(np.ascontiguousarray(bias, np.float32))
+        mm(ba, bb, bc, m, n, k, bias=bbias, accumulate=c_in is not None)
+        return bc.download(np.float32, (m, n))
+    finally:
+        mm.destroy()
+        for x in (ba, bb, bc, bbias):
+            if x is not None:
+                x.destroy()
+
+
+def check_case(dev, m, n, k, trans_a=False, trans_b=False, dtype="f16", seed=0, bias=False,
+               accumulate=False, tile=None, split_k=0, integer=False, group_m=0):
+    """Run one seeded case and compare with the oracle.  Returns metrics dict."""
+    a, b = O.make_operands(m, n, k, trans_a, trans_b, dtype, seed, integer=integer)
+    rng = np.random.default_rng(seed + 1000)
+    if integer:
+        bias_v = rng.integers(-8, 9, n).astype(np.float32) if bias else None
+        c_in = rng.integers(-8, 9, (m, n)).astype(np.float32) if accumulate else None
+    else:
+        # per-column-distinct, non-zero biases: a skipped bias add must show
+        bias_v = (rng.standard_normal(n) * 3 + np.arange(n) % 7 + 1).astype(np.float32) if bias else None
+        c_in = rng.standard_normal((m, n)).astype(np.float32) * 5 if accumulate else None
+    got = run_gemm(dev, a, b, m, n, k, trans_a, trans_b, dtype, bias_v, c_in, tile, split_k, group_m)
+    ref = O.ref_gemm(a, b, trans_a, trans_b, dtype, bias_v, c_in)
+    out = dict(maxrel=O.err_maxrel(got, ref), fro=O.err_fro(got, ref),
+               exact=bool(np.array_equal(got, ref)), finite=bool(np.isfinite(got).all()),
+               elem_ok=O.elementwise_ok(got, ref, k))
+    return out, got, ref

@@ -1,0 +1,327 @@
+"""Tape autograd call sites of the GEMM path: Ctx, Param, Linear, MLP, AdamW, TrainStep.
+
+Same classes, arguments and tensor semantics as the reference
+(/root/reference/autograd.py:22-41 pick_config, 44-108 Ctx, 111-156 Param,
+159-228 Linear, 231-301 MLP, 304-343 AdamW, 346-366 TrainStep).  Three GEMMs
+per Linear, in the reference's storage convention (W is in_f x out_f):
+
+    forward  acc = x @ W           (F,F)  m=batch, n=out_f, k=in_f
+    dW       g32 = x^T @ dz        (T,F)  m=in_f,  n=out_f, k=batch
+    dX       dx  = dz @ W^T        (F,T)  m=batch, n=in_f,  k=out_f
+
+Extensions (all off by default keep the reference's exact kernel sequence):
+    Ctx(dtype="bf16")        16-bit type of activations and weight mirrors
+    Ctx(fuse_bias=True)      bias added in the forward GEMM's epilogue
+    MLP(activation="relu")   ReLU instead of GELU in hidden layers
+    Linear.backward(accumulate=True)   dW += (beta=1 epilogue), db +=
+"""
+
+import os
+import zlib
+
+import numpy as np
+
+from .kernels import CONFIGS, Matmul, autotune_matmul, lookup_tuned, make_kernels
+from .vk import VkError
+
+
+def pick_config(m, n, k, trans_a=False, trans_b=False, min_groups=256):
+    """Tile chosen without benchmarking (autograd.py:22-41): the largest tile
+    area that still gives min_groups workgroups (one per CU of an MI355X),
+    else the most workgroups.  Returns the tile id.  The library's own picker
+    (mg_pick) refines this with padding waste and K splits; this restatement
+    exists for callers that used the reference function directly."""
+    best = None
+    for t in CONFIGS:
+        groups = -(-m // t["bm"]) * -(-n // t["bn"])
+        score = (groups >= min_groups, t["bm"] * t["bn"], groups)
+        if best is None or score > best[0]:
+            best = (score, t["id"])
+    if best is None:
+        raise VkError(f"no matmul tile fits {m}x{n}x{k}")
+    return best[1]
+
+
+class Ctx:
+    """Owns the device, the elementwise kernels and a matmul cache keyed by shape."""
+
+    def __init__(self, dev, tune=False, scalar_only=None, *, dtype="f16", fuse_bias=False):
+        if scalar_only:
+            raise VkError("there is no scalar GEMM path on MI355X: MFMA is always present")
+        self.dev = dev
+        self.dtype = dtype
+        self.fuse_bias = fuse_bias
+        self.K = make_kernels(dev, dtype)
+        self.tune = tune
+        self.scalar_only = False
+        self._mm = {}
+        self._owned = []
+
+    def matmul(self, m, n, k, trans_a=False, trans_b=False, batched=False, nbatch=1):
+        key = (m, n, k, trans_a, trans_b, batched, nbatch)
+        if key not in self._mm:
+            if self.tune:
+                mm, _ = autotune_matmul(self.dev, m, n, k, trans_a, trans_b, batched=batched,
+                                        nbatch=nbatch, dtype=self.dtype)
+            else:
+                e = lookup_tuned(self.dev.name, m, n, k, trans_a, trans_b, self.dtype, batched, nbatch)
+                if e is not None:
+                    mm = Matmul(self.dev, trans_a=trans_a, trans_b=trans_b, batched=batched,
+                                tile=e["tile_id"], dtype=self.dtype, split_k=e.get("split_k", 0),
+                                group_m=e.get("group_m", 0))
+                else:
+                    mm = Matmul(self.dev, trans_a=trans_a, trans_b=trans_b, batched=batched,
+                                dtype=self.dtype)
+            self._mm[key] = mm
+        return self._mm[key]
+
+    def buf(self, nbytes, kind="device"):
+        b = self.dev.buffer(nbytes, kind)
+        self._owned.append(b)
+        return b
+
+    def zeros(self, n_floats):
+        b = self.buf(n_floats * 4, "device")
+        self.K["zero"]([b], n_floats)
+        return b
+
+    def destroy(self):
+        for m in self._mm.values():
+            m.destroy()
+        for k in self.K.values():
+            k.destroy()
+        for b in self._owned:
+            b.destroy()
+        self._mm.clear()
+        self._owned.clear()
+
+
+class Param:
+    """f32 master, 16-bit mirror for the matmul, f32 grad, Adam moments."""
+
+    def __init__(self, ctx, shape, init=None, name="", no_decay=False):
+        self.ctx = ctx
+        self.shape = shape
+        self.n = int(np.prod(shape))
+        self.name = name
+        self.no_decay = no_decay
+        self.w32 = ctx.buf(self.n * 4, "cached")
+        self.w16 = ctx.buf(self.n * 2, "device")
+        self.g32 = ctx.buf(self.n * 4, "device")
+        self.m = ctx.zeros(self.n)
+        self.v = ctx.zeros(self.n)
+        w = self.w32.array(np.float32, shape)
+        w[:] = 0 if init is None else init
+        self.w32.flush()
+        self.sync16()
+
+    def sync16(self):
+        self.ctx.K["cast16"]([self.w32, self.w16], self.n)
+
+    def numpy(self):
+        self.w32.invalidate()
+        return self.w32.array(np.float32, self.shape)
+
+    def set(self, arr):
+        self.w32.array(np.float32, self.shape)[:] = arr
+        self.w32.flush()
+        self.sync16()
+
+    def grad_numpy(self):
+        """Copy the gradient back for checking."""
+        return self.g32.download(np.float32, self.shape)
+
+
+def _seed(name):
+    # the reference seeds from hash(name), which Python randomises per process
+    # (autograd.py:172); crc32 is stable
+    return zlib.crc32(name.encode()) & 0xFFFFFFFF
+
+
+class Linear:
+    """y = act(x @ W + b), or the same without the activation."""
+
+    def __init__(self, ctx, batch, in_f, out_f, activation=True, need_dx=True, name="", act="gelu"):
+        self.ctx, self.name = ctx, name
+        self.batch, self.in_f, self.out_f = batch, in_f, out_f
+        self.activation = activation
+        if act not in ("gelu", "relu"):
+            raise VkError(f"unknown activation {act!r}")
+        self.act = act
+        self.need_dx = need_dx
+        rng = np.random.default_rng(_seed(name))
+        w = (rng.standard_normal((in_f, out_f)) * np.sqrt(2.0 / in_f)).astype(np.float32)
+        self.W = Param(ctx, (in_f, out_f), w, name + ".W")
+        self.b = Param(ctx, (out_f,), np.zeros(out_f, np.float32), name + ".b", no_decay=True)
+
+        self.acc = ctx.buf(batch * out_f * 4)
+        self.z = ctx.buf(batch * out_f * 4)
+        self.y16 = ctx.buf(batch * out_f * 2)
+        self.dz16 = ctx.buf(batch * out_f * 2)
+        self.dz32 = ctx.buf(batch * out_f * 4)
+        self.dx32 = ctx.buf(batch * in_f * 4) if need_dx else None
+        self.x16 = None
+
+    def forward(self, x16, tape, graph=None):
+        c, K = self.ctx, self.ctx.K
+        self.x16 = x16
+        n = self.batch * self.out_f
+        mm = c.matmul(self.batch, self.out_f, self.in_f)
+        if c.fuse_bias:
+            # z = x @ W + b straight out of the GEMM epilogue
+            mm(x16, self.W.w16, self.z, self.batch, self.out_f, self.in_f, graph=graph, bias=self.b.w32)
+            if self.activation:
+                K[self.act + "16"]([self.z, self.y16], n, graph=graph)
+                out = self.y16
+            else:
+                out = self.z
+        else:
+            mm(x16, self.W.w16, self.acc, self.batch, self.out_f, self.in_f, graph=graph)
+            if self.activation:
+                K["bias_" + self.act]([self.acc, self.b.w32, self.z, self.y16], n, self.out_f, graph=graph)
+                out = self.y16
+            else:
+                K["bias"]([self.acc, self.b.w32, self.z], n, self.out_f, graph=graph)
+                out = self.z
+        tape.append(self.backward)
+        return out
+
+    def backward(self, dout16, dout32, graph=None, accumulate=False):
+        c, K = self.ctx, self.ctx.K
+        n = self.batch * self.out_f
+        if self.activation:
+            K["bias_" + self.act + "_bwd"]([dout32, self.z, self.dz16, self.dz32], n, graph=graph)
+            g16, g32 = self.dz16, self.dz32
+        else:
+            g16, g32 = dout16, dout32
+
+        # dW = X^T @ dZ.  X is stored batch x in_f, which is K x M: trans_a.
+        c.matmul(self.in_f, self.out_f, self.batch, trans_a=True)(
+            self.x16, g16, self.W.g32, self.in_f, self.out_f, self.batch, graph=graph,
+            accumulate=accumulate)
+        K["col_sum_acc" if accumulate else "col_sum"]([g32, self.b.g32], self.out_f, self.batch, graph=graph)
+
+        if not self.need_dx:
+            return None, None
+        # dX = dZ @ W^T.  W is stored in_f x out_f, which is N x K: trans_b.
+        c.matmul(self.batch, self.in_f, self.out_f, trans_b=True)(
+            g16, self.W.w16, self.dx32, self.batch, self.in_f, self.out_f, graph=graph)
+        return None, self.dx32
+
+
+class MLP:
+    """Hidden layers use the activation; the head is linear and feeds softmax + CE.
+    Classes beyond n_classes (padding) are masked inside the softmax kernel.  The
+    reference pads the class count to a tile multiple (autograd.py:234-240);
+    ragged N is legal here, so pad_classes may equal n_classes."""
+
+    def __init__(self, ctx, batch, sizes, n_classes, pad_classes=16, activation="gelu"):
+        if pad_classes < n_classes:
+            raise VkError(f"pad_classes {pad_classes} < n_classes {n_classes}")
+        self.ctx, self.batch = ctx, batch
+        self.n_classes, self.pad = n_classes, pad_classes
+        self.layers = []
+        for i in range(len(sizes) - 1):
+            self.layers.append(Linear(ctx, batch, sizes[i], sizes[i + 1], activation=True,
+                                      need_dx=(i > 0), name=f"fc{i}", act=activation))
+        self.layers.append(Linear(ctx, batch, sizes[-1], pad_classes, activation=False,
+                                  need_dx=True, name="head", act=activation))
+        self.dlog16 = ctx.buf(batch * pad_classes * 2)
+        self.dlog32 = ctx.buf(batch * pad_classes * 4)
+        self.loss = ctx.buf(batch * 4, "cached")
+
+    def params(self):
+        for l in self.layers:
+            yield l.W
+            yield l.b
+
+    def logits(self, x16, tape=None, graph=None):
+        h = x16
+        for l in self.layers:
+            h = l.forward(h, tape if tape is not None else [], graph=graph)
+        return h
+
+    def record(self, x16, labels_buf, graph, accumulate=False):
+        K = self.ctx.K
+        tape = []
+        logits = self.logits(x16, tape, graph=graph)
+        K["softmax_ce"]([logits, labels_buf, self.dlog16, self.dlog32, self.loss],
+                        self.batch, self.pad, self.n_classes, graph=graph)
+        g16, g32 = self.dlog16, self.dlog32
+        for fn in reversed(tape):
+            g16, g32 = fn(g16, g32, graph=graph, accumulate=accumulate)
+
+    def read_loss(self):
+        self.loss.invalidate()
+        return float(self.loss.array(np.float32, (self.batch,)).mean())
+
+    def forward_backward(self, x16, labels_buf, accumulate=False):
+        """Eager: one synchronous launch per kernel."""
+        K = self.ctx.K
+        tape = []
+        logits = self.logits(x16, tape)
+        K["softmax_ce"]([logits, labels_buf, self.dlog16, self.dlog32, self.loss],
+                        self.batch, self.pad, self.n_classes)
+        loss = self.read_loss()
+        g16, g32 = self.dlog16, self.dlog32
+        for fn in reversed(tape):
+            g16, g32 = fn(g16, g32, accumulate=accumulate)
+        return loss
+
+    def predict(self, x16):
+        logits = self.logits(x16)
+        out = logits.download(np.float32, (self.batch, self.pad))[:, :self.n_classes]
+        return out.argmax(1).copy()
+
+
+class AdamW:
+    """One fused kernel per parameter (autograd.py:304-343); step-varying
+    scalars live in a mapped buffer so a recorded step stays valid."""
+
+    def __init__(self, ctx, params, lr=1e-3, b1=0.9, b2=0.999, eps=1e-8, wd=0.01):
+        self.ctx, self.params = ctx, list(params)
+        self.lr, self.b1, self.b2, self.eps, self.wd = lr, b1, b2, eps, wd
+        self.t = 0
+        self.hp = ctx.buf(8 * 4, "shared")
+        self.hpv = self.hp.array(np.float32)
+        self._set_hp(lr)
+
+    def _set_hp(self, lr):
+        bc1 = 1 - self.b1 ** max(self.t, 1)
+        bc2 = 1 - self.b2 ** max(self.t, 1)
+        self.hpv[:6] = [lr, self.b1, self.b2, bc1, bc2, self.eps]
+        self.hp.flush()
+
+    def advance(self, lr=None):
+        self.t += 1
+        self._set_hp(self.lr if lr is None else lr)
+
+    def record(self, graph):
+        k = self.ctx.K["adamw"]
+        for p in self.params:
+            wd = 0.0 if p.no_decay else self.wd
+            k([p.w32, p.g32, p.m, p.v, p.w16, self.hp], p.n, wd, graph=graph)
+
+    def step(self, lr=None):
+        self.advance(lr)
+        k = self.ctx.K["adamw"]
+        for p in self.params:
+            wd = 0.0 if p.no_decay else self.wd
+            k([p.w32, p.g32, p.m, p.v, p.w16, self.hp], p.n, wd)
+
+
+class TrainStep:
+    """The whole step recorded once and replayed (autograd.py:346-366)."""
+
+    def __init__(self, model, opt, xbuf, ybuf):
+        self.model, self.opt = model, opt
+        self.graph = model.ctx.dev.graph("train_step")
+        model.record(xbuf, ybuf, self.graph)
+        opt.record(self.graph)
+        self.graph.finish()
+        self.n_dispatch = self.graph.n_dispatch
+
+    def __call__(self, lr=None):
+        self.opt.advance(lr)
+        dt = self.graph.submit()
+        return self.model.read_loss(), dt

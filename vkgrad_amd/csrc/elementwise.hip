@@ -1,0 +1,204 @@
+// Companion elementwise kernels of the training step (reference: kernels.py:699-862,
+// dataparallel.py:54-58).  One thread per element (or per row / column where the
+// reference does that); they exist so a whole MLP train step can run on the
+// device around the GEMMs, and are not tuned beyond coalesced access.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mi_gemm.h"
+
+struct mg_ctx;
+namespace mg {
+hipStream_t ctx_stream(mg_ctx *ctx);
+int ctx_fail(int code, const char *msg);
+int ctx_hip_fail(hipError_t e, const char *what);
+
+__device__ __forceinline__ uint16_t narrow16(float x, int dtype) {
+    if (dtype == MG_F16) {
+        _Float16 h = (_Float16)x;   // round to nearest even
+        return __builtin_bit_cast(uint16_t, h);
+    }
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;   // NaN
+    u += 0x7fffu + ((u >> 16) & 1u);                        // round to nearest even
+    return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float gelu_f(float x) {
+    const float c = 0.7978845608028654f;   // sqrt(2/pi), kernels.py:625-629
+    const float x3 = x * x * x;
+    return 0.5f * x * (1.0f + tanhf(c * (x + 0.044715f * x3)));
+}
+__device__ __forceinline__ float dgelu_f(float x) {
+    const float c = 0.7978845608028654f;   // kernels.py:630-635
+    const float x3 = x * x * x;
+    const float t = tanhf(c * (x + 0.044715f * x3));
+    const float sech2 = 1.0f - t * t;
+    return 0.5f * (1.0f + t) + 0.5f * x * sech2 * c * (1.0f + 3.0f * 0.044715f * x * x);
+}
+__device__ __forceinline__ float act_f(float x, int act) {
+    return act == MG_ACT_GELU ? gelu_f(x) : (act == MG_ACT_RELU ? fmaxf(x, 0.f) : x);
+}
+__device__ __forceinline__ float dact_f(float x, int act) {
+    return act == MG_ACT_GELU ? dgelu_f(x) : (act == MG_ACT_RELU ? (x > 0.f ? 1.f : 0.f) : 1.f);
+}
+
+__global__ void k_bias_act(const float *acc, const float *bias, float *z, uint16_t *y16, int64_t n,
+                           int64_t ncol, int act, int dtype) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float v = bias ? acc[i] + bias[i % ncol] : acc[i];
+    if (z) z[i] = v;
+    if (y16) y16[i] = narrow16(act_f(v, act), dtype);
+}
+
+__global__ void k_act_bwd(const float *dy, const float *z, uint16_t *dz16, float *dz32, int64_t n, int act,
+                          int dtype) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float g = dy[i] * dact_f(z[i], act);
+    if (dz16) dz16[i] = narrow16(g, dtype);
+    if (dz32) dz32[i] = g;
+}
+
+__global__ void k_col_sum(const float *g, float *sums, int64_t ncol, int64_t nrow, int accumulate) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= ncol) return;
+    float s = 0.f;
+    for (int64_t r = 0; r < nrow; ++r) s += g[r * ncol + c];
+    sums[c] = accumulate ? sums[c] + s : s;
+}
+
+__global__ void k_softmax_ce(const float *logits, const uint32_t *labels, uint16_t *dl16, float *dl32, float *loss,
+                             int64_t nrows, int64_t stride, int64_t ncls, int dtype) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= nrows) return;
+    const float *row = logits + i * stride;
+    float mx = -1e30f;
+    for (int64_t c = 0; c < ncls; ++c) mx = fmaxf(mx, row[c]);
+    float s = 0.f;
+    for (int64_t c = 0; c < ncls; ++c) s += expf(row[c] - mx);
+    const float logZ = mx + logf(s);
+    const uint32_t y = labels[i];
+    loss[i] = logZ - row[y];
+    const float inv = 1.0f / (float)nrows;
+    for (int64_t c = 0; c < stride; ++c) {
+        float gv = 0.f;
+        if (c < ncls) gv = (expf(row[c] - logZ) - (c == (int64_t)y ? 1.f : 0.f)) * inv;
+        if (dl16) dl16[i * stride + c] = narrow16(gv, dtype);
+        if (dl32) dl32[i * stride + c] = gv;
+    }
+}
+
+__global__ void k_adamw(float *w, const float *g, float *m, float *v, uint16_t *w16, const float *hp, int64_t n,
+                        float wd, int dtype) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float lr = hp[0], b1 = hp[1], b2 = hp[2], bc1 = hp[3], bc2 = hp[4], eps = hp[5];
+    const float gi = g[i];
+    const float mi = b1 * m[i] + (1.0f - b1) * gi;
+    const float vi = b2 * v[i] + (1.0f - b2) * gi * gi;
+    m[i] = mi;
+    v[i] = vi;
+    const float mh = mi / bc1;
+    const float vh = vi / bc2;
+    float wi = w[i];
+    wi -= lr * (mh / (sqrtf(vh) + eps) + wd * wi);
+    w[i] = wi;
+    if (w16) w16[i] = narrow16(wi, dtype);
+}
+
+__global__ void k_zero(float *dst, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = 0.f;
+}
+
+__global__ void k_cast16(const float *src, uint16_t *dst, int64_t n, int dtype) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = narrow16(src[i], dtype);
+}
+
+__global__ void k_grad_add(float *dst, const float *src, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] += src[i];
+}
+
+static inline unsigned blocks_for(int64_t n) { return (unsigned)((n + 255) / 256); }
+
+}  // namespace mg
+
+using namespace mg;
+
+#define EW_PRECHECK(name, cond)                                            \
+    if (!ctx) return ctx_fail(MG_ERR_ARG, name ": ctx is NULL");           \
+    if (!(cond)) return ctx_fail(MG_ERR_ARG, name ": bad argument");
+#define EW_POSTCHECK(name)                                                 \
+    do {                                                                   \
+        hipError_t e_ = hipGetLastError();                                 \
+        if (e_ != hipSuccess) return ctx_hip_fail(e_, name);               \
+        return MG_OK;                                                      \
+    } while (0)
+
+static inline bool dtype_ok(int d) { return d == MG_F16 || d == MG_BF16; }
+static inline bool act_ok(int a) { return a >= MG_ACT_NONE && a <= MG_ACT_RELU; }
+static inline bool count_ok(int64_t n) { return n > 0 && n <= (int64_t)0x7fffffff * 256; }
+
+extern "C" {
+
+int mg_ew_bias_act(mg_ctx *ctx, const float *acc, const float *bias, float *z, void *y16, int64_t n, int64_t ncol,
+                   int act, int dtype) {
+    EW_PRECHECK("mg_ew_bias_act", acc && (z || y16) && count_ok(n) && ncol > 0 && act_ok(act) && dtype_ok(dtype));
+    hipLaunchKernelGGL(k_bias_act, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), acc, bias, z, (uint16_t *)y16, n,
+                       ncol, act, dtype);
+    EW_POSTCHECK("mg_ew_bias_act");
+}
+
+int mg_ew_act_bwd(mg_ctx *ctx, const float *dy, const float *z, void *dz16, float *dz32, int64_t n, int act,
+                  int dtype) {
+    EW_PRECHECK("mg_ew_act_bwd", dy && z && (dz16 || dz32) && count_ok(n) && act_ok(act) && dtype_ok(dtype));
+    hipLaunchKernelGGL(k_act_bwd, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), dy, z, (uint16_t *)dz16, dz32, n,
+                       act, dtype);
+    EW_POSTCHECK("mg_ew_act_bwd");
+}
+
+int mg_ew_col_sum(mg_ctx *ctx, const float *g, float *sums, int64_t ncol, int64_t nrow, int accumulate) {
+    EW_PRECHECK("mg_ew_col_sum", g && sums && count_ok(ncol) && nrow > 0);
+    hipLaunchKernelGGL(k_col_sum, dim3(blocks_for(ncol)), dim3(256), 0, ctx_stream(ctx), g, sums, ncol, nrow, accumulate);
+    EW_POSTCHECK("mg_ew_col_sum");
+}
+
+int mg_ew_softmax_ce(mg_ctx *ctx, const float *logits, const uint32_t *labels, void *dl16, float *dl32, float *loss,
+                     int64_t nrows, int64_t stride, int64_t ncls, int dtype) {
+    EW_PRECHECK("mg_ew_softmax_ce", logits && labels && loss && count_ok(nrows) && ncls > 0 && stride >= ncls && dtype_ok(dtype));
+    hipLaunchKernelGGL(k_softmax_ce, dim3(blocks_for(nrows)), dim3(256), 0, ctx_stream(ctx), logits, labels,
+                       (uint16_t *)dl16, dl32, loss, nrows, stride, ncls, dtype);
+    EW_POSTCHECK("mg_ew_softmax_ce");
+}
+
+int mg_ew_adamw(mg_ctx *ctx, float *w, const float *g, float *m, float *v, void *w16, const float *hp, int64_t n,
+                float wd, int dtype) {
+    EW_PRECHECK("mg_ew_adamw", w && g && m && v && hp && count_ok(n) && dtype_ok(dtype));
+    hipLaunchKernelGGL(k_adamw, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), w, g, m, v, (uint16_t *)w16, hp, n,
+                       wd, dtype);
+    EW_POSTCHECK("mg_ew_adamw");
+}
+
+int mg_ew_zero(mg_ctx *ctx, float *dst, int64_t n) {
+    EW_PRECHECK("mg_ew_zero", dst && count_ok(n));
+    hipLaunchKernelGGL(k_zero, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), dst, n);
+    EW_POSTCHECK("mg_ew_zero");
+}
+
+int mg_ew_cast16(mg_ctx *ctx, const float *src, void *dst, int64_t n, int dtype) {
+    EW_PRECHECK("mg_ew_cast16", src && dst && count_ok(n) && dtype_ok(dtype));
+    hipLaunchKernelGGL(k_cast16, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), src, (uint16_t *)dst, n, dtype);
+    EW_POSTCHECK("mg_ew_cast16");
+}
+
+int mg_ew_grad_add(mg_ctx *ctx, float *dst, const float *src, int64_t n) {
+    EW_PRECHECK("mg_ew_grad_add", dst && src && count_ok(n));
+    hipLaunchKernelGGL(k_grad_add, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), dst, src, n);
+    EW_POSTCHECK("mg_ew_grad_add");
+}
+
+}  // extern "C"

@@ -1,0 +1,338 @@
+// MFMA GEMM kernel template for gfx950: C[M,N] (f32) = op(A) op(B) (+bias) (+C).
+//
+// One template covers the three operand layouts of the training path
+// (reference: kernels.py:32-138 generates one GLSL body per (trans_a, trans_b)):
+//   NN  A (M,K) K-contiguous,  B (K,N) N-contiguous
+//   NT  A (M,K) K-contiguous,  B (N,K) K-contiguous
+//   TN  A (K,M) M-contiguous,  B (K,N) N-contiguous
+// A K-contiguous operand is staged in LDS as [row][BK+8] and read back with one
+// 16-byte ds_read per MFMA fragment.  An operand whose contiguous axis is M or N
+// is staged untransposed as [k][B?+32] and transposed on the way out of LDS by
+// ds_read_b64_tr_b16, so no transposed copy ever exists in memory (the reference
+// makes the same point about coopMatLoad layouts, kernels.py:45-48).
+//
+// Each wavefront owns a (BM/WGM) x (BN/WGN) block of 32x32 v_mfma_f32_32x32x16
+// accumulators.  Global loads for K-block t+1 are issued into registers before
+// the MFMAs of block t and written to the other LDS stage afterwards, so there
+// is one workgroup barrier per K-block.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mg {
+
+enum { L_NN = 0, L_NT = 1, L_TN = 2 };
+enum { D_F16 = 0, D_BF16 = 1 };
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+// 16 bytes with only 2-byte alignment promised: the hardware's unaligned access
+// mode serves these as a single dwordx4 load.
+typedef u32x4 __attribute__((aligned(2))) u32x4_u;
+
+struct GemmParams {
+    const uint16_t *A;
+    const uint16_t *B;
+    float *C;
+    const float *bias;
+    int64_t lda, ldb, ldc;
+    int64_t sa, sb, sc;   // batch strides in elements
+    int M, N, K;
+    int beta;             // 1: read C and add
+    int grid_m, grid_n;   // tiles along M and N
+    int group_m;          // rasterisation band height in tiles (>= 1)
+    int split_k;          // number of K slices (gridDim.y)
+    int k_per_split;      // K elements per slice, a multiple of BK
+    int xcd_remap;        // 1: renumber workgroups so neighbours share an XCD
+};
+
+template <int DT>
+__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+    if constexpr (DT == D_F16) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a),
+                                                      __builtin_bit_cast(half8, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8, a),
+                                                       __builtin_bit_cast(bf8, b), c, 0, 0, 0);
+    }
+}
+
+typedef __attribute__((address_space(3))) short4v lds_short4;
+
+// Transposing LDS read: within each group of 16 lanes the 16 x 8-byte pieces
+// addressed by the lanes form a 4 x 16 matrix of 16-bit elements (lane j supplies
+// row j/4, columns 4*(j%4)..+3); lane j receives column j.
+__device__ __forceinline__ u32x2 lds_read_tr(const uint16_t *p) {
+    short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4 *)p);
+    return __builtin_bit_cast(u32x2, v);
+}
+
+// Workgroup -> output tile.  Consecutive hardware workgroup ids land on
+// different XCDs (8 per chip, one L2 each); renumbering them XCD-major keeps
+// tiles that share operand panels behind one L2.  Inside that order, bands of
+// `group_m` row-blocks are walked column by column (the reference's grouped
+// rasterisation, kernels.py:72-94).
+__device__ __forceinline__ void tile_coords(const GemmParams &p, int &pid_m, int &pid_n) {
+    int pid = blockIdx.x;
+    const int total = p.grid_m * p.grid_n;
+    if (p.xcd_remap) {
+        constexpr int NXCD = 8;
+        const int per = total / NXCD;   // host guarantees total % 8 == 0 when xcd_remap
+        pid = (pid % NXCD) * per + pid / NXCD;
+    }
+    const int in_group = p.group_m * p.grid_n;
+    const int gid = pid / in_group;
+    const int first_m = gid * p.group_m;
+    const int gsize = min(p.grid_m - first_m, p.group_m);
+    const int r = pid % in_group;
+    pid_m = first_m + r % gsize;
+    pid_n = r / gsize;
+}
+
+// ---------------------------------------------------------------------------
+// Operand staging.  KC = K-contiguous in memory.
+//   KC:   tile is ROWS x BK,  LDS [ROWS][BK+8],  chunk = 8 consecutive k
+//   !KC:  tile is BK x ROWS,  LDS [BK][ROWS+32], chunk = 8 consecutive rows (m or n)
+// GENERAL=false promises: base 16-byte aligned, ld % 8 == 0, and the contiguous
+// extent (K for KC, the row count otherwise) a multiple of 8, so a chunk is
+// either entirely inside the matrix or entirely outside.
+// ---------------------------------------------------------------------------
+template <bool KC, int ROWS, int BK, int NTHREADS, bool GENERAL>
+struct Stage {
+    static constexpr int PITCH = KC ? (BK + 8) : (ROWS + 32);
+    static constexpr int ELEMS = KC ? ROWS * PITCH : BK * PITCH;
+    static constexpr int CPR = KC ? BK / 8 : ROWS / 8;        // chunks per LDS row
+    static constexpr int NCHUNK = ROWS * BK / 8;
+    static constexpr int PER = (NCHUNK + NTHREADS - 1) / NTHREADS;
+    static_assert(NCHUNK % NTHREADS == 0 || NCHUNK < NTHREADS, "tile/threads mismatch");
+
+    u32x4 reg[PER];
+
+    // row0: first row (m or n) of the tile; nrows: matrix extent along that axis;
+    // k0: first k of this block; kend: one past the last valid k for this slice.
+    __device__ __forceinline__ void load(const uint16_t *base, int64_t ld, int row0, int nrows,
+                                         int k0, int kend, int tid) {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int c = tid + i * NTHREADS;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (NCHUNK >= NTHREADS || c < NCHUNK) {
+                if constexpr (KC) {
+                    const int r = c / CPR, kc = (c % CPR) * 8;
+                    const int row = min(row0 + r, nrows - 1);   // clamp: feeds masked outputs only
+                    const int k = k0 + kc;
+                    const uint16_t *src = base + (int64_t)row * ld + k;
+                    if constexpr (!GENERAL) {
+                        if (k < kend) v = *(const u32x4 *)src;
+                    } else {
+                        if (k + 8 <= kend) {
+                            v = *(const u32x4_u *)src;
+                        } else if (k < kend) {
+                            uint16_t e[8];
+#pragma unroll
+                            for (int j = 0; j < 8; j++) e[j] = (k + j < kend) ? src[j] : (uint16_t)0;
+                            v = u32x4{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
+                                      (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
+                        }
+                    }
+                } else {
+                    const int kr = c / CPR, rc = (c % CPR) * 8;
+                    const int k = k0 + kr;
+                    const int row = row0 + rc;
+                    const uint16_t *src = base + (int64_t)k * ld + row;
+                    if constexpr (!GENERAL) {
+                        if (k < kend && row < nrows) v = *(const u32x4 *)src;
+                    } else {
+                        if (k < kend) {
+                            if (row + 8 <= nrows) {
+                                v = *(const u32x4_u *)src;
+                            } else if (row < nrows) {
+                                uint16_t e[8];
+#pragma unroll
+                                for (int j = 0; j < 8; j++) e[j] = (row + j < nrows) ? src[j] : (uint16_t)0;
+                                v = u32x4{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
+                                          (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
+                            }
+                        }
+                    }
+                }
+            }
+            reg[i] = v;
+        }
+    }
+
+    __device__ __forceinline__ void store(uint16_t *lds, int tid) const {
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int c = tid + i * NTHREADS;
+            if (NCHUNK >= NTHREADS || c < NCHUNK) {
+                const int r = c / CPR, off = (c % CPR) * 8;
+                *(u32x4 *)(lds + r * PITCH + off) = reg[i];
+            }
+        }
+    }
+
+    // One 32-row x 16-k MFMA operand fragment: lane l gets row (l % 32),
+    // k = kk*16 + 8*(l/32) .. +7 of the staged tile.
+    static __device__ __forceinline__ u32x4 frag(const uint16_t *lds, int row_base, int kk, int lane) {
+        if constexpr (KC) {
+            const int row = row_base + (lane & 31);
+            const int k = kk * 16 + (lane >> 5) * 8;
+            return *(const u32x4 *)(lds + row * PITCH + k);
+        } else {
+            const int j = lane & 15, g = lane >> 4;
+            const int k = kk * 16 + (g >> 1) * 8 + (j >> 2);
+            const int row = row_base + (g & 1) * 16 + (j & 3) * 4;
+            const uint16_t *p = lds + k * PITCH + row;
+            const u32x2 lo = lds_read_tr(p);
+            const u32x2 hi = lds_read_tr(p + 4 * PITCH);
+            return u32x4{lo[0], lo[1], hi[0], hi[1]};
+        }
+    }
+};
+
+template <int LAYOUT, int BM, int BN, int BK, int WGM, int WGN>
+struct TileTraits {
+    static constexpr bool A_KC = (LAYOUT != L_TN);
+    static constexpr bool B_KC = (LAYOUT == L_NT);
+    static constexpr int NTHREADS = WGM * WGN * 64;
+    using SA = Stage<A_KC, BM, BK, NTHREADS, false>;
+    using SB = Stage<B_KC, BN, BK, NTHREADS, false>;
+    static constexpr int STAGE_ELEMS = SA::ELEMS + SB::ELEMS;
+    static constexpr int LDS_BYTES = 2 * STAGE_ELEMS * 2;
+};
+
+template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, bool GENERAL>
+__global__ void __launch_bounds__(WGM *WGN * 64)
+gemm_kernel(const GemmParams p) {
+    constexpr bool A_KC = (LAYOUT != L_TN);
+    constexpr bool B_KC = (LAYOUT == L_NT);
+    constexpr int NTHREADS = WGM * WGN * 64;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 16 == 0, "tile shape");
+    using SA = Stage<A_KC, BM, BK, NTHREADS, GENERAL>;
+    using SB = Stage<B_KC, BN, BK, NTHREADS, GENERAL>;
+    constexpr int STAGE_ELEMS = SA::ELEMS + SB::ELEMS;
+
+    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wave_m = wave / WGN, wave_n = wave % WGN;
+
+    int pid_m, pid_n;
+    tile_coords(p, pid_m, pid_n);
+    const int m0 = pid_m * BM, n0 = pid_n * BN;
+
+    const int64_t zb = blockIdx.z;
+    const uint16_t *A = p.A + zb * p.sa;
+    const uint16_t *B = p.B + zb * p.sb;
+    float *C = p.C + zb * p.sc;
+
+    const int kbeg = blockIdx.y * p.k_per_split;
+    const int kend = min(p.K, kbeg + p.k_per_split);
+    const int nkb = (kend - kbeg + BK - 1) / BK;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    SA sa;
+    SB sb;
+    if (nkb > 0) {
+        sa.load(A, p.lda, m0, p.M, kbeg, kend, tid);
+        sb.load(B, p.ldb, n0, p.N, kbeg, kend, tid);
+        sa.store(smem, tid);
+        sb.store(smem + SA::ELEMS, tid);
+    }
+    __syncthreads();
+
+    for (int kb = 0; kb < nkb; kb++) {
+        const uint16_t *As = smem + (kb & 1) * STAGE_ELEMS;
+        const uint16_t *Bs = As + SA::ELEMS;
+        const bool more = kb + 1 < nkb;
+        if (more) {
+            const int k0 = kbeg + (kb + 1) * BK;
+            sa.load(A, p.lda, m0, p.M, k0, kend, tid);
+            sb.load(B, p.ldb, n0, p.N, k0, kend, tid);
+        }
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; kk++) {
+            u32x4 af[TM], bf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++) af[i] = SA::frag(As, wave_m * WTM + i * 32, kk, lane);
+#pragma unroll
+            for (int j = 0; j < TN; j++) bf[j] = SB::frag(Bs, wave_n * WTN + j * 32, kk, lane);
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) acc[i][j] = mfma32<DT>(af[i], bf[j], acc[i][j]);
+        }
+        if (more) {
+            uint16_t *An = smem + ((kb + 1) & 1) * STAGE_ELEMS;
+            sa.store(An, tid);
+            sb.store(An + SA::ELEMS, tid);
+        }
+        __syncthreads();
+    }
+
+    // Epilogue.  Accumulator register r of lane l holds
+    //   row (r/4)*8 + (l/32)*4 + r%4,  column l%32   of its 32x32 tile.
+    const bool atomic = p.split_k > 1;
+    const bool add_bias = p.bias != nullptr && blockIdx.y == 0;
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int col = n0 + wave_n * WTN + j * 32 + (lane & 31);
+        if (col >= p.N) continue;
+        const float bv = add_bias ? p.bias[col] : 0.f;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = m0 + wave_m * WTM + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                if (row < p.M) {
+                    float *dst = C + (int64_t)row * p.ldc + col;
+                    float v = acc[i][j][r] + bv;
+                    if (atomic) {
+                        __hip_atomic_fetch_add(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    } else {
+                        if (p.beta) v = *dst + v;
+                        *dst = v;
+                    }
+                }
+            }
+        }
+    }
+}
+
+typedef hipError_t (*launch_fn)(const GemmParams &, dim3 grid, hipStream_t);
+
+template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, bool GENERAL>
+hipError_t launch_gemm(const GemmParams &p, dim3 grid, hipStream_t stream) {
+    using TT = TileTraits<LAYOUT, BM, BN, BK, WGM, WGN>;
+    auto kern = gemm_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, GENERAL>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        if (TT::LDS_BYTES > 65536) {
+            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               TT::LDS_BYTES);
+            if (e != hipSuccess) return e;
+        }
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(TT::NTHREADS), TT::LDS_BYTES, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace mg

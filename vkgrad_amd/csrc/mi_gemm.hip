@@ -1,0 +1,524 @@
+// C ABI of libmigemm.so: context, buffers, GEMM dispatch, timing, record/replay.
+// Declarations and the reference interfaces they replace are in include/mi_gemm.h.
+#include <hip/hip_runtime.h>
+
+#include <chrono>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "gemm_kernel.h"
+#include "mi_gemm.h"
+#include "tiles.h"
+
+namespace mg {
+extern launch_fn launch_table_nn_f16[MG_NUM_TILES][2];
+extern launch_fn launch_table_nn_bf16[MG_NUM_TILES][2];
+extern launch_fn launch_table_nt_f16[MG_NUM_TILES][2];
+extern launch_fn launch_table_nt_bf16[MG_NUM_TILES][2];
+extern launch_fn launch_table_tn_f16[MG_NUM_TILES][2];
+extern launch_fn launch_table_tn_bf16[MG_NUM_TILES][2];
+
+// ---------------------------------------------------------------------------
+// Pre-pass for split-K with beta == 0: C = 0 (a fill kernel, so the sequence can
+// be captured in a graph).
+// ---------------------------------------------------------------------------
+__global__ void zero_c_kernel(float *C, int64_t ldc, int M, int N, int64_t sc) {
+    float *Cz = C + (int64_t)blockIdx.z * sc;
+    const int col = blockIdx.x * blockDim.x + threadIdx.x;
+    const int row = blockIdx.y;
+    if (col < N && row < M) Cz[(int64_t)row * ldc + col] = 0.f;
+}
+
+struct TileDesc {
+    int id, bm, bn, bk, wgm, wgn;
+};
+#define X(id, bm, bn, bk, wgm, wgn) {id, bm, bn, bk, wgm, wgn},
+static const TileDesc g_tiles[MG_NUM_TILES] = {MG_TILE_LIST(X)};
+#undef X
+
+static thread_local char g_err[512] = "";
+
+static int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+static int hip_fail(hipError_t e, const char *what) {
+    return fail(MG_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                                  \
+    do {                                               \
+        hipError_t e_ = (expr);                        \
+        if (e_ != hipSuccess) return hip_fail(e_, #expr); \
+    } while (0)
+
+static launch_fn (*table_for(int layout, int dtype))[2] {
+    switch (layout * 2 + dtype) {
+        case 0: return launch_table_nn_f16;
+        case 1: return launch_table_nn_bf16;
+        case 2: return launch_table_nt_f16;
+        case 3: return launch_table_nt_bf16;
+        case 4: return launch_table_tn_f16;
+        default: return launch_table_tn_bf16;
+    }
+}
+
+static int lds_bytes_for(const TileDesc &t, int layout) {
+    const bool a_kc = layout != MG_TN, b_kc = layout == MG_NT;
+    const int a = a_kc ? t.bm * (t.bk + 8) : t.bk * (t.bm + 32);
+    const int b = b_kc ? t.bn * (t.bk + 8) : t.bk * (t.bn + 32);
+    return 2 * (a + b) * 2;
+}
+
+// The aligned instantiation may be used when every 16-byte chunk the loader
+// forms is 16-byte aligned and lies entirely inside or outside the matrix.
+static bool operands_aligned(const mg_gemm_args &a) {
+    const bool a_kc = a.layout != MG_TN, b_kc = a.layout == MG_NT;
+    if (((uintptr_t)a.a | (uintptr_t)a.b) & 15) return false;
+    if ((a.lda | a.ldb) & 7) return false;
+    if (a.nbatch > 1 && ((a.sa | a.sb) & 7)) return false;
+    if ((a_kc || b_kc) && (a.k & 7)) return false;
+    if (!a_kc && (a.m & 7)) return false;
+    if (!b_kc && (a.n & 7)) return false;
+    return true;
+}
+
+static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+struct Plan {
+    int tile, split_k, group_m, k_per_split, grid_m, grid_n, xcd_remap;
+};
+
+// Heuristic choice of tile, K split and rasterisation band.  Pure integer
+// arithmetic, so it is testable without a device.
+static void pick_plan(const mg_gemm_args &a, int cus, Plan &pl) {
+    if (cus <= 0) cus = 256;
+    int tile = a.tile;
+    if (tile < 0) {
+        // Largest tile that still yields at least ~one workgroup per CU; tie
+        // break on the least padding waste.
+        double best = -1.0;
+        for (int t = 0; t < MG_NUM_TILES; t++) {
+            const TileDesc &d = g_tiles[t];
+            const int64_t gm = cdiv(a.m, d.bm), gn = cdiv(a.n, d.bn);
+            const double useful = (double)a.m * (double)a.n / ((double)gm * d.bm * (double)gn * d.bn);
+            const int64_t groups = gm * gn * (int64_t)a.nbatch;
+            // per-workgroup efficiency grows with tile area (operand reuse) ...
+            const double area_eff = (double)d.bm * d.bn / (double)(d.bm + d.bn) / 128.0;
+            // ... and whole-chip efficiency with how evenly the grid fills the CUs.
+            const int64_t waves = cdiv(groups, cus);
+            const double fill = (double)groups / (double)(waves * cus);
+            // split-K can recover fill for deep-K problems
+            const double fill_eff = (a.k >= 2048 && fill < 0.5) ? 0.5 + 0.4 * fill : fill;
+            const double score = useful * area_eff * fill_eff;
+            if (score > best) {
+                best = score;
+                tile = t;
+            }
+        }
+    }
+    const TileDesc &d = g_tiles[tile];
+    pl.tile = tile;
+    pl.grid_m = (int)cdiv(a.m, d.bm);
+    pl.grid_n = (int)cdiv(a.n, d.bn);
+    const int64_t groups = (int64_t)pl.grid_m * pl.grid_n * a.nbatch;
+    const int64_t kblocks = cdiv(a.k, d.bk);
+    int split = a.split_k;
+    if (split <= 0) {
+        split = 1;
+        if (groups * 2 <= cus && kblocks >= 8) {
+            split = (int)(cus / groups);
+            // keep at least 4 K-blocks per slice so the pipeline prologue amortises
+            if (split > kblocks / 4) split = (int)(kblocks / 4);
+            if (split < 1) split = 1;
+        }
+    }
+    if (split > kblocks) split = (int)kblocks;
+    if (split < 1) split = 1;
+    int64_t kb_per = cdiv(kblocks, split);
+    split = (int)cdiv(kblocks, kb_per);   // no empty slices
+    pl.split_k = split;
+    pl.k_per_split = (int)(kb_per * d.bk);
+    int gm = a.group_m;
+    if (gm <= 0) gm = 8;
+    if (gm > pl.grid_m) gm = pl.grid_m;
+    pl.group_m = gm;
+    pl.xcd_remap = ((int64_t)pl.grid_m * pl.grid_n) % 8 == 0 ? 1 : 0;
+}
+
+static int check_args(const mg_gemm_args *a) {
+    if (!a) return fail(MG_ERR_ARG, "mg_gemm: args is NULL");
+    if (a->struct_size != (int32_t)sizeof(mg_gemm_args))
+        return fail(MG_ERR_ARG, "mg_gemm: struct_size %d != %d", a->struct_size, (int)sizeof(mg_gemm_args));
+    if (a->layout < MG_NN || a->layout > MG_TN) return fail(MG_ERR_ARG, "mg_gemm: unknown layout %d", a->layout);
+    if (a->dtype != MG_F16 && a->dtype != MG_BF16) return fail(MG_ERR_ARG, "mg_gemm: unknown dtype %d", a->dtype);
+    if (a->beta != 0 && a->beta != 1) return fail(MG_ERR_ARG, "mg_gemm: beta must be 0 or 1, got %d", a->beta);
+    if (a->m <= 0 || a->n <= 0 || a->k <= 0)
+        return fail(MG_ERR_ARG, "mg_gemm: shape %lldx%lldx%lld must be positive", (long long)a->m, (long long)a->n,
+                    (long long)a->k);
+    if (a->m > 0x7fffffffLL - 512 || a->n > 0x7fffffffLL - 512 || a->k > 0x7fffffffLL - 512)
+        return fail(MG_ERR_ARG, "mg_gemm: shape %lldx%lldx%lld exceeds 32-bit indexing", (long long)a->m,
+                    (long long)a->n, (long long)a->k);
+    if (!a->a || !a->b || !a->c) return fail(MG_ERR_ARG, "mg_gemm: NULL operand pointer");
+    if (((uintptr_t)a->a | (uintptr_t)a->b) & 1) return fail(MG_ERR_ARG, "mg_gemm: A and B must be 2-byte aligned");
+    if ((uintptr_t)a->c & 3) return fail(MG_ERR_ARG, "mg_gemm: C must be 4-byte aligned");
+    if (a->bias && ((uintptr_t)a->bias & 3)) return fail(MG_ERR_ARG, "mg_gemm: bias must be 4-byte aligned");
+    const int64_t a_cols = a->layout == MG_TN ? a->m : a->k;
+    const int64_t b_cols = a->layout == MG_NT ? a->k : a->n;
+    if (a->lda < a_cols) return fail(MG_ERR_ARG, "mg_gemm: lda %lld < %lld stored columns of A", (long long)a->lda, (long long)a_cols);
+    if (a->ldb < b_cols) return fail(MG_ERR_ARG, "mg_gemm: ldb %lld < %lld stored columns of B", (long long)a->ldb, (long long)b_cols);
+    if (a->ldc < a->n) return fail(MG_ERR_ARG, "mg_gemm: ldc %lld < N %lld", (long long)a->ldc, (long long)a->n);
+    if (a->nbatch < 1 || a->nbatch > 65535) return fail(MG_ERR_ARG, "mg_gemm: nbatch %d out of range [1, 65535]", a->nbatch);
+    if (a->nbatch > 1 && (a->sa < 0 || a->sb < 0 || a->sc < 0))
+        return fail(MG_ERR_ARG, "mg_gemm: negative batch stride");
+    if (a->nbatch > 1 && a->sc < a->m * a->ldc && a->sc != 0)
+        return fail(MG_ERR_ARG, "mg_gemm: batch stride of C (%lld) overlaps outputs", (long long)a->sc);
+    if (a->nbatch > 1 && a->sc == 0) return fail(MG_ERR_ARG, "mg_gemm: batches would overwrite one another (sc == 0)");
+    if (a->tile < -1 || a->tile >= MG_NUM_TILES) return fail(MG_ERR_ARG, "mg_gemm: unknown tile id %d", a->tile);
+    if (a->split_k < 0 || a->split_k > 65535) return fail(MG_ERR_ARG, "mg_gemm: split_k %d out of range", a->split_k);
+    if (a->group_m < 0) return fail(MG_ERR_ARG, "mg_gemm: group_m %d is negative", a->group_m);
+    return MG_OK;
+}
+
+}  // namespace mg
+
+using namespace mg;
+
+struct mg_ctx {
+    int device;
+    hipStream_t stream;
+    hipEvent_t ev0, ev1;
+    hipDeviceProp_t prop;
+    bool capturing;
+};
+
+struct mg_graph {
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+};
+
+extern "C" {
+
+const char *mg_last_error(void) { return g_err; }
+
+int mg_init(int device_index, mg_ctx **out) {
+    if (!out) return fail(MG_ERR_ARG, "mg_init: out is NULL");
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        return fail(MG_ERR_NODEVICE, "mg_init: no HIP device available (%s)", e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+    }
+    if (device_index < 0 || device_index >= count)
+        return fail(MG_ERR_ARG, "mg_init: device index %d out of range [0, %d)", device_index, count);
+    HIP_TRY(hipSetDevice(device_index));
+    mg_ctx *c = new (std::nothrow) mg_ctx();
+    if (!c) return fail(MG_ERR_NOMEM, "mg_init: out of host memory");
+    c->device = device_index;
+    c->capturing = false;
+    e = hipGetDeviceProperties(&c->prop, device_index);
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreate(&c->ev0);
+    if (e == hipSuccess) e = hipEventCreate(&c->ev1);
+    if (e != hipSuccess) {
+        delete c;
+        return hip_fail(e, "mg_init");
+    }
+    if (strncmp(c->prop.gcnArchName, "gfx950", 6) != 0) {
+        char arch[64];
+        snprintf(arch, sizeof(arch), "%s", c->prop.gcnArchName);
+        (void)hipStreamDestroy(c->stream);
+        delete c;
+        return fail(MG_ERR_NODEVICE, "mg_init: device is %s; this library is built for gfx950 only", arch);
+    }
+    *out = c;
+    return MG_OK;
+}
+
+int mg_destroy(mg_ctx *ctx) {
+    if (!ctx) return MG_OK;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipEventDestroy(ctx->ev0);
+    (void)hipEventDestroy(ctx->ev1);
+    (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return MG_OK;
+}
+
+int mg_get_device_info(mg_ctx *ctx, mg_device_info *out) {
+    if (!ctx || !out) return fail(MG_ERR_ARG, "mg_get_device_info: NULL argument");
+    memset(out, 0, sizeof(*out));
+    snprintf(out->name, sizeof(out->name), "%s", ctx->prop.name[0] ? ctx->prop.name : ctx->prop.gcnArchName);
+    snprintf(out->arch, sizeof(out->arch), "%s", ctx->prop.gcnArchName);
+    out->compute_units = ctx->prop.multiProcessorCount;
+    out->clock_khz = ctx->prop.clockRate;
+    out->mem_clock_khz = ctx->prop.memoryClockRate;
+    out->mem_bus_bits = ctx->prop.memoryBusWidth;
+    out->l2_bytes = ctx->prop.l2CacheSize;
+    out->lds_bytes_per_cu = (int32_t)ctx->prop.maxSharedMemoryPerMultiProcessor;
+    out->wavefront = ctx->prop.warpSize;
+    out->total_mem = (int64_t)ctx->prop.totalGlobalMem;
+    return MG_OK;
+}
+
+int mg_alloc(mg_ctx *ctx, size_t nbytes, int kind, void **dev_ptr, void **host_ptr) {
+    if (!ctx || !dev_ptr || !host_ptr) return fail(MG_ERR_ARG, "mg_alloc: NULL argument");
+    *dev_ptr = *host_ptr = nullptr;
+    if (kind < MG_DEVICE || kind > MG_BAR) return fail(MG_ERR_ARG, "mg_alloc: unknown memory kind %d", kind);
+    if (nbytes == 0) return fail(MG_ERR_ARG, "mg_alloc: size must be positive");
+    if (ctx->capturing) return fail(MG_ERR_STATE, "mg_alloc: not allowed while a graph is being recorded");
+    HIP_TRY(hipSetDevice(ctx->device));
+    if (kind == MG_DEVICE) {
+        void *p = nullptr;
+        hipError_t e = hipMalloc(&p, nbytes);
+        if (e != hipSuccess) return fail(e == hipErrorOutOfMemory ? MG_ERR_NOMEM : MG_ERR_HIP, "mg_alloc: hipMalloc(%zu): %s", nbytes, hipGetErrorString(e));
+        *dev_ptr = p;
+    } else {
+        // Pinned host memory, mapped into the device's address space and
+        // coherent: the CPU pointer and the GPU pointer name the same bytes.
+        void *p = nullptr;
+        hipError_t e = hipHostMalloc(&p, nbytes, hipHostMallocMapped | hipHostMallocCoherent);
+        if (e != hipSuccess) return fail(e == hipErrorOutOfMemory ? MG_ERR_NOMEM : MG_ERR_HIP, "mg_alloc: hipHostMalloc(%zu): %s", nbytes, hipGetErrorString(e));
+        void *d = nullptr;
+        e = hipHostGetDevicePointer(&d, p, 0);
+        if (e != hipSuccess) {
+            (void)hipHostFree(p);
+            return hip_fail(e, "mg_alloc: hipHostGetDevicePointer");
+        }
+        *host_ptr = p;
+        *dev_ptr = d;
+    }
+    return MG_OK;
+}
+
+int mg_free(mg_ctx *ctx, void *dev_ptr, int kind) {
+    if (!ctx) return fail(MG_ERR_ARG, "mg_free: ctx is NULL");
+    if (!dev_ptr) return MG_OK;
+    if (kind < MG_DEVICE || kind > MG_BAR) return fail(MG_ERR_ARG, "mg_free: unknown memory kind %d", kind);
+    if (ctx->capturing) return fail(MG_ERR_STATE, "mg_free: not allowed while a graph is being recorded");
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    if (kind == MG_DEVICE) HIP_TRY(hipFree(dev_ptr));
+    else HIP_TRY(hipHostFree(dev_ptr));
+    return MG_OK;
+}
+
+static int do_copy(mg_ctx *ctx, void *dst, const void *src, size_t nbytes, hipMemcpyKind kind, const char *who) {
+    if (!ctx || !dst || !src) return fail(MG_ERR_ARG, "%s: NULL argument", who);
+    if (nbytes == 0) return MG_OK;
+    if (ctx->capturing) return fail(MG_ERR_STATE, "%s: not allowed while a graph is being recorded", who);
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipMemcpyAsync(dst, src, nbytes, kind, ctx->stream));
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return MG_OK;
+}
+
+int mg_copy(mg_ctx *ctx, void *dst, const void *src, size_t nbytes) {
+    return do_copy(ctx, dst, src, nbytes, hipMemcpyDefault, "mg_copy");
+}
+int mg_upload(mg_ctx *ctx, void *dst_dev, const void *src_host, size_t nbytes) {
+    return do_copy(ctx, dst_dev, src_host, nbytes, hipMemcpyHostToDevice, "mg_upload");
+}
+int mg_download(mg_ctx *ctx, void *dst_host, const void *src_dev, size_t nbytes) {
+    return do_copy(ctx, dst_host, src_dev, nbytes, hipMemcpyDeviceToHost, "mg_download");
+}
+
+int mg_sync(mg_ctx *ctx) {
+    if (!ctx) return fail(MG_ERR_ARG, "mg_sync: ctx is NULL");
+    if (ctx->capturing) return fail(MG_ERR_STATE, "mg_sync: not allowed while a graph is being recorded");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return MG_OK;
+}
+
+int mg_gemm_check(const mg_gemm_args *args) { return check_args(args); }
+
+int mg_tile_count(void) { return MG_NUM_TILES; }
+
+int mg_tile_info(int id, mg_tile *out) {
+    if (!out) return fail(MG_ERR_ARG, "mg_tile_info: out is NULL");
+    if (id < 0 || id >= MG_NUM_TILES) return fail(MG_ERR_ARG, "mg_tile_info: unknown tile id %d", id);
+    const TileDesc &t = g_tiles[id];
+    memset(out, 0, sizeof(*out));
+    out->id = id;
+    out->bm = t.bm;
+    out->bn = t.bn;
+    out->bk = t.bk;
+    out->waves_m = t.wgm;
+    out->waves_n = t.wgn;
+    out->threads = t.wgm * t.wgn * 64;
+    out->lds_bytes = lds_bytes_for(t, MG_NT);
+    out->min_m = 1;
+    snprintf(out->name, sizeof(out->name), "mm_%dx%dx%d_w%dx%d", t.bm, t.bn, t.bk, t.wgm, t.wgn);
+    return MG_OK;
+}
+
+int mg_tile_fits(int id, const mg_gemm_args *args) {
+    if (id < 0 || id >= MG_NUM_TILES) return 0;
+    if (check_args(args) != MG_OK) return 0;
+    // every tile handles ragged shapes; the only limit is the grid size
+    const TileDesc &t = g_tiles[id];
+    const int64_t groups = cdiv(args->m, t.bm) * cdiv(args->n, t.bn);
+    return groups <= 0x7fffffffLL ? 1 : 0;
+}
+
+int mg_pick(const mg_gemm_args *args, int compute_units, int *tile, int *split_k, int *group_m) {
+    int rc = check_args(args);
+    if (rc != MG_OK) return rc;
+    Plan pl;
+    pick_plan(*args, compute_units, pl);
+    if (tile) *tile = pl.tile;
+    if (split_k) *split_k = pl.split_k;
+    if (group_m) *group_m = pl.group_m;
+    return MG_OK;
+}
+
+static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
+    const mg_gemm_args &a = *args;
+    const TileDesc &t = g_tiles[pl.tile];
+    GemmParams p;
+    p.A = (const uint16_t *)a.a;
+    p.B = (const uint16_t *)a.b;
+    p.C = a.c;
+    p.bias = a.bias;
+    p.lda = a.lda;
+    p.ldb = a.ldb;
+    p.ldc = a.ldc;
+    p.sa = a.nbatch > 1 ? a.sa : 0;
+    p.sb = a.nbatch > 1 ? a.sb : 0;
+    p.sc = a.nbatch > 1 ? a.sc : 0;
+    p.M = (int)a.m;
+    p.N = (int)a.n;
+    p.K = (int)a.k;
+    p.beta = a.beta;
+    p.grid_m = pl.grid_m;
+    p.grid_n = pl.grid_n;
+    p.group_m = pl.group_m;
+    p.split_k = pl.split_k;
+    p.k_per_split = pl.k_per_split;
+    p.xcd_remap = pl.xcd_remap;
+    if ((int64_t)pl.grid_m * pl.grid_n > 0x7fffffffLL) return fail(MG_ERR_ARG, "mg_gemm: grid too large");
+    if (lds_bytes_for(t, a.layout) > (int)ctx->prop.maxSharedMemoryPerMultiProcessor)
+        return fail(MG_ERR_ARG, "mg_gemm: tile %d needs %d bytes of LDS", pl.tile, lds_bytes_for(t, a.layout));
+    if (pl.split_k > 1 && a.beta == 0) {
+        dim3 zg((unsigned)cdiv(a.n, 256), (unsigned)a.m, (unsigned)a.nbatch);
+        if (a.m > 65535) {
+            // rows beyond the grid-y limit: fold into several launches
+            for (int64_t r0 = 0; r0 < a.m; r0 += 65535) {
+                const int rows = (int)((a.m - r0) < 65535 ? (a.m - r0) : 65535);
+                dim3 g2((unsigned)cdiv(a.n, 256), (unsigned)rows, (unsigned)a.nbatch);
+                hipLaunchKernelGGL(zero_c_kernel, g2, dim3(256), 0, ctx->stream, a.c + r0 * a.ldc, a.ldc, rows, (int)a.n, p.sc);
+            }
+        } else {
+            hipLaunchKernelGGL(zero_c_kernel, zg, dim3(256), 0, ctx->stream, a.c, a.ldc, (int)a.m, (int)a.n, p.sc);
+        }
+        HIP_TRY(hipGetLastError());
+    }
+    const int general = operands_aligned(a) ? 0 : 1;
+    launch_fn fn = table_for(a.layout, a.dtype)[pl.tile][general];
+    dim3 grid((unsigned)(pl.grid_m * pl.grid_n), (unsigned)pl.split_k, (unsigned)a.nbatch);
+    hipError_t e = fn(p, grid, ctx->stream);
+    if (e != hipSuccess) return hip_fail(e, "mg_gemm: kernel launch");
+    return MG_OK;
+}
+
+int mg_gemm(mg_ctx *ctx, const mg_gemm_args *args) {
+    if (!ctx) return fail(MG_ERR_ARG, "mg_gemm: ctx is NULL");
+    int rc = check_args(args);
+    if (rc != MG_OK) return rc;
+    Plan pl;
+    pick_plan(*args, ctx->prop.multiProcessorCount, pl);
+    return enqueue_gemm(ctx, args, pl);
+}
+
+int mg_gemm_time(mg_ctx *ctx, const mg_gemm_args *args, int repeat, double *seconds) {
+    if (!ctx || !seconds) return fail(MG_ERR_ARG, "mg_gemm_time: NULL argument");
+    if (repeat < 1) return fail(MG_ERR_ARG, "mg_gemm_time: repeat must be >= 1");
+    if (ctx->capturing) return fail(MG_ERR_STATE, "mg_gemm_time: not allowed while a graph is being recorded");
+    int rc = check_args(args);
+    if (rc != MG_OK) return rc;
+    Plan pl;
+    pick_plan(*args, ctx->prop.multiProcessorCount, pl);
+    HIP_TRY(hipEventRecord(ctx->ev0, ctx->stream));
+    for (int i = 0; i < repeat; i++) {
+        rc = enqueue_gemm(ctx, args, pl);
+        if (rc != MG_OK) return rc;
+    }
+    HIP_TRY(hipEventRecord(ctx->ev1, ctx->stream));
+    HIP_TRY(hipEventSynchronize(ctx->ev1));
+    float ms = 0.f;
+    HIP_TRY(hipEventElapsedTime(&ms, ctx->ev0, ctx->ev1));
+    *seconds = (double)ms * 1e-3;
+    return MG_OK;
+}
+
+int mg_graph_begin(mg_ctx *ctx) {
+    if (!ctx) return fail(MG_ERR_ARG, "mg_graph_begin: ctx is NULL");
+    if (ctx->capturing) return fail(MG_ERR_STATE, "mg_graph_begin: a graph is already being recorded");
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->capturing = true;
+    return MG_OK;
+}
+
+int mg_graph_end(mg_ctx *ctx, mg_graph **out) {
+    if (!ctx || !out) return fail(MG_ERR_ARG, "mg_graph_end: NULL argument");
+    *out = nullptr;
+    if (!ctx->capturing) return fail(MG_ERR_STATE, "mg_graph_end: no graph is being recorded");
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &g);
+    ctx->capturing = false;
+    if (e != hipSuccess) return hip_fail(e, "mg_graph_end: hipStreamEndCapture");
+    hipGraphExec_t ex = nullptr;
+    e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(g);
+        return hip_fail(e, "mg_graph_end: hipGraphInstantiate");
+    }
+    mg_graph *r = new (std::nothrow) mg_graph();
+    if (!r) {
+        (void)hipGraphExecDestroy(ex);
+        (void)hipGraphDestroy(g);
+        return fail(MG_ERR_NOMEM, "mg_graph_end: out of host memory");
+    }
+    r->graph = g;
+    r->exec = ex;
+    *out = r;
+    return MG_OK;
+}
+
+int mg_graph_launch(mg_ctx *ctx, mg_graph *g, double *seconds) {
+    if (!ctx || !g) return fail(MG_ERR_ARG, "mg_graph_launch: NULL argument");
+    if (ctx->capturing) return fail(MG_ERR_STATE, "mg_graph_launch: a graph is being recorded");
+    auto t0 = std::chrono::steady_clock::now();
+    HIP_TRY(hipGraphLaunch(g->exec, ctx->stream));
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    auto t1 = std::chrono::steady_clock::now();
+    if (seconds) *seconds = std::chrono::duration<double>(t1 - t0).count();
+    return MG_OK;
+}
+
+int mg_graph_destroy(mg_ctx *ctx, mg_graph *g) {
+    if (!g) return MG_OK;
+    if (ctx) (void)hipStreamSynchronize(ctx->stream);
+    (void)hipGraphExecDestroy(g->exec);
+    (void)hipGraphDestroy(g->graph);
+    delete g;
+    return MG_OK;
+}
+
+}  // extern "C"
+
+// ---- shared with elementwise.hip ----
+namespace mg {
+hipStream_t ctx_stream(mg_ctx *ctx) { return ctx->stream; }
+int ctx_fail(int code, const char *msg) { return fail(code, "%s", msg); }
+int ctx_hip_fail(hipError_t e, const char *what) { return hip_fail(e, what); }
+}  // namespace mg

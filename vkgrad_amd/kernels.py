@@ -1,0 +1,468 @@
+"""GEMM objects, tile table, autotuner and the companion elementwise kernels.
+
+Call surface of the reference's kernels.py (Matmul: /root/reference/kernels.py:232-315,
+CONFIGS: 326-331, warmup: 353-381, autotune_matmul: 450-603, Elementwise and
+make_kernels: 668-862) over libmigemm.so.  Differences a caller can see:
+
+  * any positive M, N, K is legal (the reference refuses non-tile-multiples,
+    kernels.py:271-276);
+  * keyword-only extensions on a Matmul call: bias=, accumulate=, lda/ldb/ldc=;
+    and on its constructor: dtype= ("f16" | "bf16"), tile=, split_k=;
+  * eager calls are timed with HIP events on the device, not host wall clock.
+"""
+
+import ctypes as C
+import json
+import os
+import time
+
+import numpy as np
+
+from . import _lib as L
+from .vk import VkError, _check
+
+TILE = 32  # MFMA accumulator tile edge (v_mfma_f32_32x32x16); the reference's is 16
+
+
+def _tiles():
+    lib = L.load()
+    out = []
+    for i in range(lib.mg_tile_count()):
+        t = L.Tile()
+        _check(lib.mg_tile_info(i, C.byref(t)), "tile table")
+        out.append(dict(id=t.id, bm=t.bm, bn=t.bn, bk=t.bk, waves_m=t.waves_m, waves_n=t.waves_n,
+                        threads=t.threads, lds_bytes=t.lds_bytes, name=t.name.decode()))
+    return out
+
+
+# The tile table the tuner walks; one dict per block tile built into the library.
+CONFIGS = _tiles()
+
+
+def layout_of(trans_a, trans_b):
+    if trans_a and trans_b:
+        raise VkError("the (trans_a, trans_b) = (True, True) layout is not provided: no call site uses it")
+    return L.MG_TN if trans_a else (L.MG_NT if trans_b else L.MG_NN)
+
+
+def _nearest_tile(bm, bn):
+    """Tile of the table closest to a requested bm x bn (log-distance)."""
+    best = min(CONFIGS, key=lambda t: abs(np.log2(t["bm"] / bm)) + abs(np.log2(t["bn"] / bn)))
+    return best["id"]
+
+
+class Matmul:
+    """One GEMM configuration: C[m,n] f32 = op(A) @ op(B), 16-bit inputs.
+
+    Positional arguments follow the reference (sg, wm, wn described a
+    sg*wm*16 x wn*16 block tile there); here they select the nearest tile of the
+    library's table, tile= selects one by id, and with neither the built-in
+    picker chooses per call.
+    """
+
+    def __init__(self, dev, sg=None, wm=None, wn=None, trans_a=False, trans_b=False,
+                 capture_stats=False, lds=True, bk=64, batched=False, acc16=False,
+                 group_m=0, *, tile=None, dtype="f16", split_k=0):
+        if acc16:
+            raise VkError("acc16 (f16 output) is not provided: no call site of the path uses it")
+        if dtype not in L.DTYPES:
+            raise VkError(f"unknown dtype {dtype!r}; use 'f16' or 'bf16'")
+        self.dev = dev
+        self.sg, self.wm, self.wn = sg, wm, wn
+        self.trans_a, self.trans_b = bool(trans_a), bool(trans_b)
+        self.layout = layout_of(trans_a, trans_b)
+        self.lds, self.bk, self.batched = True, bk, bool(batched)
+        self.acc16 = False
+        self.group_m = int(group_m)
+        self.dtype = dtype
+        self.split_k = int(split_k)
+        if tile is None and sg is not None:
+            tile = _nearest_tile(sg * (wm or 1) * 16, (wn or 1) * 16)
+        if tile is not None and not 0 <= tile < len(CONFIGS):
+            raise VkError(f"unknown tile id {tile}")
+        self.tile = -1 if tile is None else int(tile)
+        if self.tile >= 0:
+            t = CONFIGS[self.tile]
+            self.bm, self.bn, self.bk = t["bm"], t["bn"], t["bk"]
+            base = t["name"]
+        else:
+            self.bm = self.bn = None
+            base = "mm_auto"
+        self.name = (f"{base}_{dtype}{'_ta' if trans_a else ''}{'_tb' if trans_b else ''}"
+                     f"{'_bat' if batched else ''}{'_g' + str(group_m) if group_m else ''}"
+                     f"{'_s' + str(split_k) if split_k > 1 else ''}")
+        self._keep = []
+
+    def fits(self, m, n, k):
+        """Every tile handles ragged shapes; only positivity is required."""
+        return m > 0 and n > 0 and k > 0
+
+    def _args(self, a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc):
+        if self.batched:
+            nb = int(nbatch)
+            sa, sb, sc = (int(s) for s in strides)
+        else:
+            nb, sa, sb, sc = 1, 0, 0, 0
+        ga = L.GemmArgs()
+        ga.struct_size = C.sizeof(L.GemmArgs)
+        ga.layout, ga.dtype = self.layout, L.DTYPES[self.dtype]
+        ga.beta = 1 if accumulate else 0
+        ga.m, ga.n, ga.k = int(m), int(n), int(k)
+        ga.a, ga.b, ga.c = a.ptr, b.ptr, c.ptr
+        ga.lda = int(lda) if lda is not None else (m if self.trans_a else k)
+        ga.ldb = int(ldb) if ldb is not None else (k if self.trans_b else n)
+        ga.ldc = int(ldc) if ldc is not None else n
+        ga.bias = bias.ptr if bias is not None else None
+        ga.nbatch, ga.tile = nb, self.tile
+        ga.sa, ga.sb, ga.sc = sa, sb, sc
+        ga.split_k, ga.group_m = self.split_k, self.group_m
+        # buffers must cover what the kernel touches
+        esz = 2
+        a_rows = k if self.trans_a else m
+        b_rows = n if self.trans_b else k
+        a_cols = m if self.trans_a else k
+        b_cols = k if self.trans_b else n
+        need_a = ((nb - 1) * sa + (a_rows - 1) * ga.lda + a_cols) * esz
+        need_b = ((nb - 1) * sb + (b_rows - 1) * ga.ldb + b_cols) * esz
+        need_c = ((nb - 1) * sc + (m - 1) * ga.ldc + n) * 4
+        if m > 0 and n > 0 and k > 0:
+            if need_a > a.size or need_b > b.size or need_c > c.size:
+                raise VkError(f"{self.name}: shape {m}x{n}x{k} (nbatch {nb}) needs {need_a}/{need_b}/{need_c} "
+                              f"bytes but buffers hold {a.size}/{b.size}/{c.size}")
+            if bias is not None and bias.size < n * 4:
+                raise VkError(f"{self.name}: bias buffer of {bias.size} bytes is shorter than N={n} floats")
+        return ga
+
+    def __call__(self, a, b, c, m, n, k, repeat=1, graph=None, nbatch=1, strides=(0, 0, 0),
+                 *, bias=None, accumulate=False, lda=None, ldb=None, ldc=None):
+        lib, ctx = self.dev._lib, self.dev._ctx
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc)
+        if graph is not None:
+            _check(lib.mg_gemm_check(C.byref(ga)), self.name)
+            self._keep.append(ga)
+
+            def launch(ga=ga):
+                _check(lib.mg_gemm(ctx, C.byref(ga)), self.name)
+
+            graph.record(launch, [a, b, c], name=self.name,
+                         bytes_hint=self.traffic_bytes(m, n, k, nbatch))
+            nb_ = nbatch if self.batched else 1
+            graph.mm_split.append((nb_ * 2 * (m * k + k * n), nb_ * m * n * 4))
+            return 0.0
+        dt = C.c_double()
+        _check(lib.mg_gemm_time(ctx, C.byref(ga), int(repeat), C.byref(dt)), self.name)
+        return dt.value
+
+    def enqueue(self, a, b, c, m, n, k, nbatch=1, strides=(0, 0, 0), *, bias=None,
+                accumulate=False, lda=None, ldb=None, ldc=None):
+        """Launch without waiting (the stream keeps order); for pipelined callers."""
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc)
+        _check(self.dev._lib.mg_gemm(self.dev._ctx, C.byref(ga)), self.name)
+
+    def plan(self, m, n, k, nbatch=1):
+        """(tile id, split_k, group_m) the library would use for this shape."""
+        ga = L.GemmArgs()
+        ga.struct_size = C.sizeof(L.GemmArgs)
+        ga.layout, ga.dtype = self.layout, L.DTYPES[self.dtype]
+        ga.m, ga.n, ga.k = int(m), int(n), int(k)
+        ga.a = ga.b = ga.c = 16     # placeholders: the picker never dereferences
+        ga.lda = m if self.trans_a else k
+        ga.ldb = k if self.trans_b else n
+        ga.ldc = n
+        ga.nbatch, ga.tile = (int(nbatch) if self.batched else 1), self.tile
+        ga.sc = m * n
+        ga.split_k, ga.group_m = self.split_k, self.group_m
+        t, s, g = C.c_int(), C.c_int(), C.c_int()
+        _check(self.dev._lib.mg_pick(C.byref(ga), self.dev.compute_units, C.byref(t), C.byref(s), C.byref(g)),
+               self.name)
+        return t.value, s.value, g.value
+
+    def traffic_bytes(self, m, n, k, nbatch=1, bias=False, accumulate=False):
+        """Algorithmic (compulsory) bytes: each operand once.  The reference's
+        upper bound (kernels.py:299-309) counts per-tile re-reads instead; with
+        LDS-staged 256-wide tiles and L2-aware rasterisation those mostly hit
+        cache, so the compulsory figure is the one rooflines are priced on."""
+        nb = nbatch if self.batched else 1
+        return nb * (2 * (m * k + k * n) + 4 * m * n * (2 if accumulate else 1) + (4 * n if bias else 0))
+
+    def flops(self, m, n, k):
+        return 2 * m * n * k
+
+    def destroy(self):
+        self._keep.clear()
+
+
+# --------------------------------------------------------------------------
+# autotuner
+# --------------------------------------------------------------------------
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+# Shipped table of tuned picks for MI355X, consulted read-only after the user cache.
+_SHIPPED_CACHE = os.path.join(_HERE, "tuned_mi355x.json")
+_TUNE_CACHE = os.environ.get("VKGRAD_AMD_TUNE_CACHE", os.path.join(_HERE, ".autotune.json"))
+
+
+def _load_cache(path=None):
+    path = path or _TUNE_CACHE
+    if os.path.exists(path):
+        try:
+            with open(path) as f:
+                return json.load(f)
+        except (OSError, ValueError):
+            return {}
+    return {}
+
+
+def _save_cache(cache, path=None):
+    path = path or _TUNE_CACHE
+    tmp = path + f".{os.getpid()}.tmp"
+    with open(tmp, "w") as f:
+        json.dump(cache, f, indent=1, sort_keys=True)
+    os.replace(tmp, path)
+
+
+def tune_key(dev_name, m, n, k, trans_a, trans_b, dtype="f16", batched=False, nbatch=1,
+             accumulate=False):
+    """Cache key; the reference's shape (kernels.py:459-460) plus dtype and beta."""
+    return (f"{dev_name}|{m}x{n}x{k}|ta{int(trans_a)}tb{int(trans_b)}|{dtype}"
+            f"{'|acc' if accumulate else ''}{'|bat' + str(nbatch) if batched else ''}")
+
+
+def lookup_tuned(dev_name, m, n, k, trans_a, trans_b, dtype="f16", batched=False, nbatch=1,
+                 accumulate=False):
+    """Cached pick for a shape, user cache first, then the shipped table."""
+    key = tune_key(dev_name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate)
+    for path in (_TUNE_CACHE, _SHIPPED_CACHE):
+        e = _load_cache(path).get(key)
+        if e is not None:
+            return e
+    return None
+
+
+_WARMED = set()
+
+
+def warmup(dev, seconds=2.0, force=False):
+    """Sustained GEMM load until clocks settle (kernels.py:353-381).  On MI355X
+    the effect is a power-managed clock under MFMA load rather than an idle
+    ramp, but timing anything before the chip is in its loaded state still
+    biases a comparison."""
+    if not force and id(dev) in _WARMED:
+        return 0.0
+    m = n = k = 2048
+    a = dev.buffer(m * k * 2, "device")
+    b = dev.buffer(k * n * 2, "device")
+    c = dev.buffer(m * n * 4, "device")
+    mm = Matmul(dev)
+    t0 = time.perf_counter()
+    try:
+        while time.perf_counter() - t0 < seconds:
+            mm(a, b, c, m, n, k, repeat=20)
+    finally:
+        mm.destroy()
+        for x in (a, b, c):
+            x.destroy()
+    _WARMED.add(id(dev))
+    return time.perf_counter() - t0
+
+
+_MEASURE_S = 0.02     # GPU time per measurement (kernels.py:424)
+_SUBMIT_CAP_S = 0.2   # one timed batch stays under this (kernels.py:421)
+
+
+def _repeat_for(t_one):
+    """Launches per measurement so every candidate is timed over equal GPU
+    time, not an equal number of launches (kernels.py:433-447)."""
+    return max(1, int(min(_MEASURE_S, _SUBMIT_CAP_S) / max(t_one, 1e-7)))
+
+
+def candidate_space(m, n, k, cus=256, nbatch=1):
+    """(tile, split_k) pairs worth timing for a shape: every tile whose padding
+    waste is tolerable, with K splits that bring an under-filled grid up to
+    about one or two workgroups per CU."""
+    out = []
+    for t in CONFIGS:
+        gm, gn = -(-m // t["bm"]), -(-n // t["bn"])
+        useful = (m * n) / (gm * t["bm"] * gn * t["bn"])
+        if useful < 0.45 and len(CONFIGS) > 1:
+            continue
+        groups = gm * gn * nbatch
+        kblocks = -(-k // t["bk"])
+        splits = {1}
+        if groups < cus and kblocks >= 4:
+            for target in (cus, 2 * cus):
+                s = max(1, min(target // groups, kblocks // 2))
+                splits.add(s)
+                if s > 2:
+                    splits.add(s // 2)
+        for s in sorted(splits):
+            out.append((t["id"], s))
+    if not out:
+        out = [(CONFIGS[0]["id"], 1)]
+    return out
+
+
+def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=False,
+                    use_cache=True, batched=False, nbatch=1, *, dtype="f16", accumulate=False,
+                    timer=None):
+    """Pick the fastest (tile, split_k, group_m) for one shape (kernels.py:450-603).
+
+    Stage one times every candidate round-robin over equal GPU time and keeps
+    the best-of-`reps`; stage two sweeps the rasterisation band on the winner
+    only, re-measuring group_m's default alongside (kernels.py:539-584).
+    `timer(mm, repeat) -> seconds` replaces the device for tests of the logic.
+    Returns (Matmul, best) with best keys config, lds, tflops, ms, tile,
+    evaluated, pruned, group_m, split_k, tile_id.
+    """
+    key = tune_key(dev.name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate)
+    if use_cache:
+        e = lookup_tuned(dev.name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate)
+        if e is not None:
+            return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=e["tile_id"],
+                          dtype=dtype, split_k=e.get("split_k", 0), group_m=e.get("group_m", 0)), e
+
+    nb = nbatch if batched else 1
+    strides = (m * k, k * n, m * n)
+    call = dict(nbatch=nb, strides=strides) if batched else {}
+    bufs = None
+    if timer is None:
+        warmup(dev)
+        bufs = (dev.buffer(nb * m * k * 2, "device"), dev.buffer(nb * k * n * 2, "device"),
+                dev.buffer(nb * m * n * 4, "device"))
+        K = make_kernels(dev)
+        # finite operands: garbage bit patterns may be NaN/denormal and skew timing
+        K["zero"]([bufs[0]], nb * m * k // 2 or 1)
+        K["zero"]([bufs[1]], nb * k * n // 2 or 1)
+
+        def timer(mm, repeat):
+            return mm(bufs[0], bufs[1], bufs[2], m, n, k, repeat=repeat, accumulate=accumulate, **call)
+
+    try:
+        cands = [Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=t, dtype=dtype,
+                        split_k=s, group_m=0)
+                 for t, s in candidate_space(m, n, k, getattr(dev, "compute_units", 256), nb)]
+        if not cands:
+            raise VkError(f"no matmul config fits {m}x{n}x{k}")
+
+        def measure(mms):
+            warm = {id(x): timer(x, 1) for x in mms}
+            best_t = {id(x): float("inf") for x in mms}
+            for _ in range(reps):
+                for x in mms:   # round-robin: drift spreads evenly over candidates
+                    r = _repeat_for(warm[id(x)])
+                    best_t[id(x)] = min(best_t[id(x)], timer(x, r) / r)
+            return best_t
+
+        best_t = measure(cands)
+        results = []
+        for x in cands:
+            t = best_t[id(x)]
+            tf = x.flops(m, n, k) * nb / t / 1e12
+            results.append({"config": [x.bm, x.bn, x.bk], "lds": True, "tflops": tf, "ms": t * 1e3,
+                            "tile": [x.bm, x.bn], "tile_id": x.tile, "split_k": x.split_k})
+            if verbose:
+                print(f"    tile {x.bm:3d}x{x.bn:3d} split_k={x.split_k:2d}  {tf:8.2f} TFLOPS  {t * 1e6:9.1f} us")
+        results.sort(key=lambda r: -r["tflops"])
+        best = dict(results[0])
+
+        variants = [Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=best["tile_id"],
+                           dtype=dtype, split_k=best["split_k"], group_m=g) for g in (0, 1, 2, 4, 16)]
+        gt = measure(variants)
+        scored = sorted(((v.flops(m, n, k) * nb / gt[id(v)] / 1e12, v.group_m) for v in variants), reverse=True)
+        if verbose:
+            for tf, g in scored:
+                print(f"    group_m={g:2d} on winning tile   {tf:8.2f} TFLOPS")
+        tf, g = scored[0]
+        best.update(tflops=tf, ms=2.0 * m * n * k * nb / tf / 1e9, group_m=g)
+        best["pruned"] = len(CONFIGS) * 1 - len({c.tile for c in cands})
+        best["evaluated"] = len(results)
+        if use_cache:
+            cache = _load_cache()
+            cache[key] = best
+            _save_cache(cache)
+        return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=best["tile_id"],
+                      dtype=dtype, split_k=best["split_k"], group_m=best["group_m"]), best
+    finally:
+        if bufs:
+            for x in bufs:
+                x.destroy()
+
+
+# --------------------------------------------------------------------------
+# companion elementwise kernels
+# --------------------------------------------------------------------------
+
+class Elementwise:
+    """One elementwise kernel with the reference's call shape
+    (kernels.py:687-693): k(buffers, n, *args, graph=None)."""
+
+    def __init__(self, dev, name, launch):
+        self.dev, self.name, self._launch = dev, name, launch
+
+    def __call__(self, buffers, n, *args, repeat=1, graph=None):
+        lib, ctx = self.dev._lib, self.dev._ctx
+        ptrs = [b.ptr for b in buffers]
+        if any(p is None for p in ptrs):
+            raise VkError(f"{self.name}: a buffer was destroyed")
+
+        def launch():
+            _check(self._launch(lib, ctx, ptrs, int(n), *args), self.name)
+
+        if graph is not None:
+            graph.record(launch, buffers, name=self.name)
+            return 0.0
+        t0 = time.perf_counter()
+        for _ in range(repeat):
+            launch()
+        _check(lib.mg_sync(ctx), self.name)
+        return time.perf_counter() - t0
+
+    def destroy(self):
+        pass
+
+
+def make_kernels(dev, dtype="f16"):
+    """The elementwise kernels the training loop needs (kernels.py:699-862), by
+    the reference's names.  `dtype` is the 16-bit type of narrowed outputs.
+    bias_relu / bias_relu_bwd are the ReLU counterparts of the GELU pair."""
+    dt = L.DTYPES[dtype]
+    K = {}
+
+    def add(name, fn):
+        K[name] = Elementwise(dev, name, fn)
+
+    # buffers: acc, bias, z, y16 ; args: ncol
+    add("bias_gelu", lambda lib, ctx, p, n, ncol:
+        lib.mg_ew_bias_act(ctx, p[0], p[1], p[2], p[3], n, int(ncol), L.MG_ACT_GELU, dt))
+    add("bias_relu", lambda lib, ctx, p, n, ncol:
+        lib.mg_ew_bias_act(ctx, p[0], p[1], p[2], p[3], n, int(ncol), L.MG_ACT_RELU, dt))
+    # buffers: dy, z, dz16, dz32
+    add("bias_gelu_bwd", lambda lib, ctx, p, n:
+        lib.mg_ew_act_bwd(ctx, p[0], p[1], p[2], p[3], n, L.MG_ACT_GELU, dt))
+    add("bias_relu_bwd", lambda lib, ctx, p, n:
+        lib.mg_ew_act_bwd(ctx, p[0], p[1], p[2], p[3], n, L.MG_ACT_RELU, dt))
+    # buffers: dy, z, dz16
+    add("bias_gelu_bwd16", lambda lib, ctx, p, n:
+        lib.mg_ew_act_bwd(ctx, p[0], p[1], p[2], None, n, L.MG_ACT_GELU, dt))
+    # buffers: acc, bias, z ; args: ncol
+    add("bias", lambda lib, ctx, p, n, ncol:
+        lib.mg_ew_bias_act(ctx, p[0], p[1], p[2], None, n, int(ncol), L.MG_ACT_NONE, dt))
+    # buffers: g, sums ; n = ncol ; args: nrow
+    add("col_sum", lambda lib, ctx, p, n, nrow: lib.mg_ew_col_sum(ctx, p[0], p[1], n, int(nrow), 0))
+    add("col_sum_acc", lambda lib, ctx, p, n, nrow: lib.mg_ew_col_sum(ctx, p[0], p[1], n, int(nrow), 1))
+    # buffers: z, y16 — activation + narrowing of a pre-activation that already holds its bias
+    add("gelu16", lambda lib, ctx, p, n:
+        lib.mg_ew_bias_act(ctx, p[0], None, None, p[1], n, 1, L.MG_ACT_GELU, dt))
+    add("relu16", lambda lib, ctx, p, n:
+        lib.mg_ew_bias_act(ctx, p[0], None, None, p[1], n, 1, L.MG_ACT_RELU, dt))
+    # buffers: logits, labels, dl16, dl32, loss ; n = rows ; args: stride, ncls
+    add("softmax_ce", lambda lib, ctx, p, n, stride, ncls:
+        lib.mg_ew_softmax_ce(ctx, p[0], p[1], p[2], p[3], p[4], n, int(stride), int(ncls), dt))
+    # buffers: w, g, m, v, w16, hp ; args: wd
+    add("adamw", lambda lib, ctx, p, n, wd:
+        lib.mg_ew_adamw(ctx, p[0], p[1], p[2], p[3], p[4], p[5], n, float(wd), dt))
+    add("zero", lambda lib, ctx, p, n: lib.mg_ew_zero(ctx, p[0], n))
+    add("cast16", lambda lib, ctx, p, n: lib.mg_ew_cast16(ctx, p[0], p[1], n, dt))
+    # dataparallel.py:54-58 — buffers: dst, src
+    add("grad_add", lambda lib, ctx, p, n: lib.mg_ew_grad_add(ctx, p[0], p[1], n))
+    return K
