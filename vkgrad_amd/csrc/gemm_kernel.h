@@ -109,9 +109,23 @@ struct Stage {
     static constexpr int CPR = KC ? BK / 8 : ROWS / 8;        // chunks per LDS row
     static constexpr int NCHUNK = ROWS * BK / 8;
     static constexpr int PER = (NCHUNK + NTHREADS - 1) / NTHREADS;
-    static_assert(NCHUNK % NTHREADS == 0 || NCHUNK < NTHREADS, "tile/threads mismatch");
+    static constexpr int RSTEP = NTHREADS / CPR;              // LDS rows between a thread's chunks
+    static_assert(NCHUNK % NTHREADS == 0 && NTHREADS % CPR == 0, "tile/threads mismatch");
 
     u32x4 reg[PER];
+
+    // Unconditional loads for a K-block that lies entirely inside the matrix in
+    // both directions.  `tile` points at the block's first element (uniform over
+    // the workgroup); a thread's chunks are RSTEP*ld apart.
+    __device__ __forceinline__ void load_fast(const uint16_t *tile, int64_t ld, int tid) {
+        const uint16_t *src = tile + (int64_t)(tid / CPR) * ld + (tid % CPR) * 8;
+        const int64_t step = (int64_t)RSTEP * ld;
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            if constexpr (GENERAL) reg[i] = *(const u32x4_u *)(src + i * step);
+            else reg[i] = *(const u32x4 *)(src + i * step);
+        }
+    }
 
     // row0: first row (m or n) of the tile; nrows: matrix extent along that axis;
     // k0: first k of this block; kend: one past the last valid k for this slice.
@@ -121,7 +135,7 @@ struct Stage {
         for (int i = 0; i < PER; i++) {
             const int c = tid + i * NTHREADS;
             u32x4 v = {0u, 0u, 0u, 0u};
-            if (NCHUNK >= NTHREADS || c < NCHUNK) {
+            {
                 if constexpr (KC) {
                     const int r = c / CPR, kc = (c % CPR) * 8;
                     const int row = min(row0 + r, nrows - 1);   // clamp: feeds masked outputs only
@@ -170,7 +184,7 @@ struct Stage {
 #pragma unroll
         for (int i = 0; i < PER; i++) {
             const int c = tid + i * NTHREADS;
-            if (NCHUNK >= NTHREADS || c < NCHUNK) {
+            {
                 const int r = c / CPR, off = (c % CPR) * 8;
                 *(u32x4 *)(lds + r * PITCH + off) = reg[i];
             }
@@ -207,6 +221,32 @@ struct TileTraits {
     static constexpr int LDS_BYTES = 2 * STAGE_ELEMS * 2;
 };
 
+template <int N>
+struct IntC {
+    static constexpr int value = N;
+};
+
+// Pin the instruction mix of one MFMA group for the backend scheduler: the
+// group's LDS reads, LDS writes and global loads are spread evenly between its
+// MFMAs instead of being issued in a burst in front of them.
+template <int I, int NMFMA, int NDSR, int NDSW, int NVMEM>
+__device__ __forceinline__ void interleave_step() {
+    if constexpr (I < NMFMA) {
+        constexpr int r = (I + 1) * NDSR / NMFMA - I * NDSR / NMFMA;
+        constexpr int w = (I + 1) * NDSW / NMFMA - I * NDSW / NMFMA;
+        constexpr int v = (I + 1) * NVMEM / NMFMA - I * NVMEM / NMFMA;
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+        if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);   // LDS reads
+        if constexpr (w > 0) __builtin_amdgcn_sched_group_barrier(0x200, w, 0);   // LDS writes
+        if constexpr (v > 0) __builtin_amdgcn_sched_group_barrier(0x020, v, 0);   // global loads
+        interleave_step<I + 1, NMFMA, NDSR, NDSW, NVMEM>();
+    }
+}
+template <int NMFMA, int NDSR, int NDSW, int NVMEM>
+__device__ __forceinline__ void interleave_group() {
+    interleave_step<0, NMFMA, NDSR, NDSW, NVMEM>();
+}
+
 template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, bool GENERAL>
 __global__ void __launch_bounds__(WGM *WGN * 64)
 gemm_kernel(const GemmParams p) {
@@ -215,10 +255,14 @@ gemm_kernel(const GemmParams p) {
     constexpr int NTHREADS = WGM * WGN * 64;
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 16 == 0, "tile shape");
+    constexpr int KK = BK / 16;
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 32 == 0, "tile shape");
     using SA = Stage<A_KC, BM, BK, NTHREADS, GENERAL>;
     using SB = Stage<B_KC, BN, BK, NTHREADS, GENERAL>;
     constexpr int STAGE_ELEMS = SA::ELEMS + SB::ELEMS;
+    // LDS read instructions per fragment: one b128, or two transposing b64
+    constexpr int NDSR = TM * (A_KC ? 1 : 2) + TN * (B_KC ? 1 : 2);
+    constexpr int NLOAD = SA::PER + SB::PER;
 
     extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
 
@@ -239,6 +283,10 @@ gemm_kernel(const GemmParams p) {
     const int kbeg = blockIdx.y * p.k_per_split;
     const int kend = min(p.K, kbeg + p.k_per_split);
     const int nkb = (kend - kbeg + BK - 1) / BK;
+    // K-blocks that the unconditional loader may fetch: the whole block inside
+    // K, and the tile inside M and N.
+    const bool interior = (m0 + BM <= p.M) && (n0 + BN <= p.N);
+    const int nkb_fast = interior ? (kend - kbeg) / BK : 0;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -250,69 +298,164 @@ gemm_kernel(const GemmParams p) {
 
     SA sa;
     SB sb;
+    u32x4 af[2][TM], bf[2][TN];
+
+    // first element of K-block kb of this tile, per operand
+    auto a_tile = [&](int kb) -> const uint16_t * {
+        const int64_t k0 = kbeg + (int64_t)kb * BK;
+        return A_KC ? A + (int64_t)m0 * p.lda + k0 : A + k0 * p.lda + m0;
+    };
+    auto b_tile = [&](int kb) -> const uint16_t * {
+        const int64_t k0 = kbeg + (int64_t)kb * BK;
+        return B_KC ? B + (int64_t)n0 * p.ldb + k0 : B + k0 * p.ldb + n0;
+    };
+    auto load_block = [&](int kb) {   // uniform branch: fast when the block is interior
+        if (kb < nkb_fast) {
+            sa.load_fast(a_tile(kb), p.lda, tid);
+            sb.load_fast(b_tile(kb), p.ldb, tid);
+        } else {
+            sa.load(A, p.lda, m0, p.M, kbeg + kb * BK, kend, tid);
+            sb.load(B, p.ldb, n0, p.N, kbeg + kb * BK, kend, tid);
+        }
+    };
+    auto read_frags = [&](const uint16_t *As, int kk, int slot) {
+        const uint16_t *Bs = As + SA::ELEMS;
+#pragma unroll
+        for (int i = 0; i < TM; i++) af[slot][i] = SA::frag(As, wave_m * WTM + i * 32, kk, lane);
+#pragma unroll
+        for (int j = 0; j < TN; j++) bf[slot][j] = SB::frag(Bs, wave_n * WTN + j * 32, kk, lane);
+    };
+    auto mfma_group = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) acc[i][j] = mfma32<DT>(af[slot][i], bf[slot][j], acc[i][j]);
+    };
+
+    // Prologue: K-block 0 -> LDS stage 0, K-block 1 -> registers, fragments of
+    // (block 0, kk 0) -> af[0], bf[0].
     if (nkb > 0) {
-        sa.load(A, p.lda, m0, p.M, kbeg, kend, tid);
-        sb.load(B, p.ldb, n0, p.N, kbeg, kend, tid);
+        load_block(0);
         sa.store(smem, tid);
         sb.store(smem + SA::ELEMS, tid);
+        if (nkb > 1) load_block(1);
     }
     __syncthreads();
+    if (nkb > 0) read_frags(smem, 0, 0);
 
-    for (int kb = 0; kb < nkb; kb++) {
+    // One K-block.  MODE 1: blocks kb+1 and kb+2 exist and kb+2 is interior, so
+    // the loop body is straight-line code; MODE 0: generic tail with uniform
+    // branches.  The global loads issued here are consumed one whole K-block
+    // later, by the LDS writes of the next iteration.
+    auto kblock = [&](auto mode, int kb) {
+        constexpr int MODE = decltype(mode)::value;
         const uint16_t *As = smem + (kb & 1) * STAGE_ELEMS;
-        const uint16_t *Bs = As + SA::ELEMS;
-        const bool more = kb + 1 < nkb;
-        if (more) {
-            const int k0 = kbeg + (kb + 1) * BK;
-            sa.load(A, p.lda, m0, p.M, k0, kend, tid);
-            sb.load(B, p.ldb, n0, p.N, k0, kend, tid);
+        uint16_t *An = smem + ((kb + 1) & 1) * STAGE_ELEMS;
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) {
+            const int cur = kk & 1, nxt = cur ^ 1;
+#ifndef EXP_NO_FRAG
+            if (kk < KK - 1) {
+                read_frags(As, kk + 1, nxt);
+            } else if (MODE == 1 || kb + 1 < nkb) {
+                read_frags(An, 0, nxt);   // next stage is complete: the barrier below has passed
+            }
+#endif
+            if (kk == KK - 2) {
+#ifndef EXP_NO_STORE
+                if (MODE == 1 || kb + 1 < nkb) {
+                    sa.store(An, tid);
+                    sb.store(An + SA::ELEMS, tid);
+                }
+#endif
+                if constexpr (MODE == 1) {
+#ifndef EXP_NO_GLOAD
+                    sa.load_fast(a_tile(kb + 2), p.lda, tid);
+                    sb.load_fast(b_tile(kb + 2), p.ldb, tid);
+#endif
+                } else {
+                    if (kb + 2 < nkb) load_block(kb + 2);
+                }
+            }
+            mfma_group(cur);
+            if constexpr (MODE == 1) {
+                if (kk == KK - 2) interleave_group<TM * TN, NDSR, NLOAD, NLOAD>();
+                else interleave_group<TM * TN, NDSR, 0, 0>();
+            }
+#ifndef EXP_NO_BARRIER
+            if (kk == KK - 2) __syncthreads();
+#endif
         }
-#pragma unroll
-        for (int kk = 0; kk < BK / 16; kk++) {
-            u32x4 af[TM], bf[TN];
-#pragma unroll
-            for (int i = 0; i < TM; i++) af[i] = SA::frag(As, wave_m * WTM + i * 32, kk, lane);
-#pragma unroll
-            for (int j = 0; j < TN; j++) bf[j] = SB::frag(Bs, wave_n * WTN + j * 32, kk, lane);
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++) acc[i][j] = mfma32<DT>(af[i], bf[j], acc[i][j]);
-        }
-        if (more) {
-            uint16_t *An = smem + ((kb + 1) & 1) * STAGE_ELEMS;
-            sa.store(An, tid);
-            sb.store(An + SA::ELEMS, tid);
-        }
-        __syncthreads();
-    }
+    };
 
+    int kb = 0;
+#ifdef EXP_NO_MAINLOOP
+    kb = nkb;
+#endif
+    const int n_steady = nkb_fast - 2;   // iterations whose kb+2 prefetch is interior
+    for (; kb < n_steady; kb++) kblock(IntC<1>{}, kb);
+    for (; kb < nkb; kb++) kblock(IntC<0>{}, kb);
+
+#ifdef EXP_NO_EPILOGUE
+    if (p.M > 0) { if (acc[0][0][0] == 123.456f) C[0] = 1.f; return; }
+#endif
     // Epilogue.  Accumulator register r of lane l holds
-    //   row (r/4)*8 + (l/32)*4 + r%4,  column l%32   of its 32x32 tile.
-    const bool atomic = p.split_k > 1;
+    //   row (r/4)*8 + (l/32)*4 + r%4,  column l%32   of its 32x32 tile,
+    // so one store instruction writes two full 128-byte row segments.  The mode
+    // (overwrite / read-add / atomic-add) and the edge test are uniform over the
+    // workgroup and hoisted out of the element loops.
     const bool add_bias = p.bias != nullptr && blockIdx.y == 0;
+    const int row_l = m0 + wave_m * WTM + (lane >> 5) * 4;
+    const int col_l = n0 + wave_n * WTN + (lane & 31);
+    float *cl = C + (int64_t)row_l * p.ldc + col_l;
+    const int64_t ldc = p.ldc;
+    float bv[TN];
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
-        const int col = n0 + wave_n * WTN + j * 32 + (lane & 31);
-        if (col >= p.N) continue;
-        const float bv = add_bias ? p.bias[col] : 0.f;
+    for (int j = 0; j < TN; j++) bv[j] = (add_bias && col_l + j * 32 < p.N) ? p.bias[col_l + j * 32] : 0.f;
+
+    auto write_out = [&](auto mode_c, auto edge_c) {
+        constexpr int MODE = decltype(mode_c)::value;   // 0 overwrite, 1 C += , 2 atomic +=
+        constexpr bool EDGE = decltype(edge_c)::value != 0;
 #pragma unroll
         for (int i = 0; i < TM; i++) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int row = m0 + wave_m * WTM + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-                if (row < p.M) {
-                    float *dst = C + (int64_t)row * p.ldc + col;
-                    float v = acc[i][j][r] + bv;
-                    if (atomic) {
-                        __hip_atomic_fetch_add(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    } else {
-                        if (p.beta) v = *dst + v;
-                        *dst = v;
+            for (int j = 0; j < TN; j++) {
+                float *ct = cl + (int64_t)(i * 32) * ldc + j * 32;
+                const bool col_ok = !EDGE || (col_l + j * 32 < p.N);
+                float old[16];
+                if constexpr (MODE == 1) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int ro = (r >> 2) * 8 + (r & 3);
+                        const bool ok = col_ok && (!EDGE || row_l + i * 32 + ro < p.M);
+                        old[r] = ok ? ct[ro * ldc] : 0.f;
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int ro = (r >> 2) * 8 + (r & 3);
+                    const bool ok = col_ok && (!EDGE || row_l + i * 32 + ro < p.M);
+                    float v = acc[i][j][r] + bv[j];
+                    if constexpr (MODE == 1) v = old[r] + v;
+                    if (ok) {
+                        if constexpr (MODE == 2)
+                            __hip_atomic_fetch_add(ct + ro * ldc, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        else
+                            ct[ro * ldc] = v;
                     }
                 }
             }
         }
+    };
+    const int mode = p.split_k > 1 ? 2 : (p.beta ? 1 : 0);
+    if (interior) {
+        if (mode == 0) write_out(IntC<0>{}, IntC<0>{});
+        else if (mode == 1) write_out(IntC<1>{}, IntC<0>{});
+        else write_out(IntC<2>{}, IntC<0>{});
+    } else {
+        if (mode == 0) write_out(IntC<0>{}, IntC<1>{});
+        else if (mode == 1) write_out(IntC<1>{}, IntC<1>{});
+        else write_out(IntC<2>{}, IntC<1>{});
     }
 }
 
