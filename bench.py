@@ -1,0 +1,243 @@
+#!/usr/bin/env python3
+"""Benchmark of the training-GEMM path on one MI355X.
+
+One step = every GEMM of one GPT-2-small training step (BASELINE.json configs[2]):
+d_model 768, 12 layers, 8 x 1024 = 8192 token rows, per layer QKV 768->2304,
+proj 768->768, MLP 768->3072->768, plus the tied LM head 768->50257; for every
+linear the forward, dX and dW products (147 GEMMs, 6.07 TFLOP), bf16 inputs,
+fp32 accumulate and fp32 outputs, synthetic operands already resident in HBM.
+Weights are stored out x in (the tied-head convention), so the kernel layouts
+are NT forward, NN dX, TN dW.
+
+Prints ONE JSON line: whole-step TFLOP/s, the MFMA roofline of the dominant
+GEMM measured with HIP events on the library's stream, and the numpy oracle
+timed on this machine's host cores over one transformer layer.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = 2500.0     # MI355X dense bf16/fp16 MFMA peak
+ROWS, D, LAYERS, VOCAB = 8192, 768, 12, 50257
+LINEARS = [("qkv", 768, 2304), ("proj", 768, 768), ("fc1", 768, 3072), ("fc2", 3072, 768)]
+DTYPE = "bf16"
+
+
+def gemm_list():
+    """(name, layout, M, N, K, count) for one step.  W is (out, in)."""
+    out = []
+    for name, fin, fout in LINEARS:
+        out.append((name + ".fwd", "NT", ROWS, fout, fin, LAYERS))   # Y  = X  W^T
+        out.append((name + ".dX", "NN", ROWS, fin, fout, LAYERS))    # dX = dY W
+        out.append((name + ".dW", "TN", fout, fin, ROWS, LAYERS))    # dW = dY^T X
+    out.append(("head.fwd", "NT", ROWS, VOCAB, D, 1))
+    out.append(("head.dX", "NN", ROWS, D, VOCAB, 1))
+    out.append(("head.dW", "TN", VOCAB, D, ROWS, 1))
+    return out
+
+
+LAYOUT_FLAGS = {"NN": (False, False), "NT": (False, True), "TN": (True, False)}
+
+
+def fill_bf16(dev, buf, n, rng, scale):
+    """Upload n bf16 values ~N(0, scale) in slabs (keeps host memory small)."""
+    from vkgrad_amd.dtypes import f32_to_bf16_bits
+    slab = 1 << 24
+    tmp = dev.buffer(min(n, slab) * 2, "device")
+    done = 0
+    lib, ctx = dev._lib, dev._ctx
+    while done < n:
+        m = min(slab, n - done)
+        bits = f32_to_bf16_bits((rng.standard_normal(m, dtype=np.float32) * scale))
+        tmp.upload(bits)
+        rc = lib.mg_copy(ctx, buf.ptr + done * 2, tmp.ptr, m * 2)
+        assert rc == 0
+        done += m
+    tmp.destroy()
+
+
+def cpu_baseline():
+    """The oracle (numpy float32 matmul of the rounded operands, reference
+    kernels.py:606-610) over one transformer layer's 12 GEMMs, on this host."""
+    from oracle.ref_gemm import f32_to_bf16_bits, bf16_bits_to_f32
+    rng = np.random.default_rng(1)
+    flops = 0.0
+    secs = 0.0
+    # warm the BLAS thread pool
+    w = rng.standard_normal((512, 512), dtype=np.float32)
+    (w @ w).sum()
+    for name, fin, fout in LINEARS:
+        x = bf16_bits_to_f32(f32_to_bf16_bits(rng.standard_normal((ROWS, fin), dtype=np.float32)))
+        wt = bf16_bits_to_f32(f32_to_bf16_bits(rng.standard_normal((fout, fin), dtype=np.float32) * 0.02))
+        dy = bf16_bits_to_f32(f32_to_bf16_bits(rng.standard_normal((ROWS, fout), dtype=np.float32)))
+        t0 = time.perf_counter()
+        y = x @ wt.T
+        dx = dy @ wt
+        dw = dy.T @ x
+        secs += time.perf_counter() - t0
+        flops += 3 * 2.0 * ROWS * fin * fout
+        del y, dx, dw
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        cores = os.cpu_count() or 1
+    threads = int(os.environ.get("OPENBLAS_NUM_THREADS") or os.environ.get("OMP_NUM_THREADS") or cores)
+    return {"value": round(flops / secs / 1e12, 4), "unit": "TFLOP/s", "cores": min(threads, cores),
+            "kind": "port",
+            "sample": "one transformer layer (12 GEMMs, 348 GFLOP), numpy float32 matmul of bf16-rounded operands, single pass"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--eager", action="store_true", help="enqueue GEMMs one by one instead of replaying a graph")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the path has no multi-GPU part); run with --gpus 1")
+
+    from vkgrad_amd.vk import Device
+    from vkgrad_amd.kernels import Matmul, lookup_tuned
+
+    dev = Device()
+    rng = np.random.default_rng(1)
+
+    # Operands: per linear one activation X, one weight W (out x in) and one
+    # upstream gradient dY; three rotating sets so that consecutive layers never
+    # reuse a buffer that may still sit in the 256 MB last-level cache.
+    NSET = 3
+    sets = []
+    for s in range(NSET):
+        bufs = {}
+        for name, fin, fout in LINEARS:
+            x = dev.buffer(ROWS * fin * 2, "device")
+            w = dev.buffer(fout * fin * 2, "device")
+            dy = dev.buffer(ROWS * fout * 2, "device")
+            fill_bf16(dev, x, ROWS * fin, rng, 1.0)
+            fill_bf16(dev, w, fout * fin, rng, 0.02)
+            fill_bf16(dev, dy, ROWS * fout, rng, 1.0)
+            bufs[name] = dict(x=x, w=w, dy=dy, y=dev.buffer(ROWS * fout * 4, "device"),
+                              dx=dev.buffer(ROWS * fin * 4, "device"), dw=dev.buffer(fout * fin * 4, "device"))
+        sets.append(bufs)
+    head = dict(x=dev.buffer(ROWS * D * 2, "device"), w=dev.buffer(VOCAB * D * 2, "device"),
+                dy=dev.buffer(ROWS * VOCAB * 2, "device"), y=dev.buffer(ROWS * VOCAB * 4, "device"),
+                dx=dev.buffer(ROWS * D * 4, "device"), dw=dev.buffer(VOCAB * D * 4, "device"))
+    fill_bf16(dev, head["x"], ROWS * D, rng, 1.0)
+    fill_bf16(dev, head["w"], VOCAB * D, rng, 0.02)
+    fill_bf16(dev, head["dy"], ROWS * VOCAB, rng, 1.0)
+
+    mms = {}
+
+    def mm_for(layout, m, n, k):
+        key = (layout, m, n, k)
+        if key not in mms:
+            ta, tb = LAYOUT_FLAGS[layout]
+            e = lookup_tuned(dev.name, m, n, k, ta, tb, DTYPE)
+            if e is not None:
+                mms[key] = Matmul(dev, trans_a=ta, trans_b=tb, dtype=DTYPE, tile=e["tile_id"],
+                                  split_k=e.get("split_k", 0), group_m=e.get("group_m", 0))
+            else:
+                mms[key] = Matmul(dev, trans_a=ta, trans_b=tb, dtype=DTYPE)
+        return mms[key]
+
+    def linear_calls(b, fin, fout, rows=ROWS):
+        """The three GEMMs of one linear: (mm, a, b, c, m, n, k)."""
+        return [
+            (mm_for("NT", rows, fout, fin), b["x"], b["w"], b["y"], rows, fout, fin),
+            (mm_for("NN", rows, fin, fout), b["dy"], b["w"], b["dx"], rows, fin, fout),
+            (mm_for("TN", fout, fin, rows), b["dy"], b["x"], b["dw"], fout, fin, rows),
+        ]
+
+    calls = []
+    for layer in range(LAYERS):
+        b = sets[layer % NSET]
+        for name, fin, fout in LINEARS:
+            calls += linear_calls(b[name], fin, fout)
+    calls += linear_calls(head, D, VOCAB)
+    step_flops = sum(2.0 * m * n * k for (_, _, _, _, m, n, k) in calls)
+
+    if args.eager:
+        def run_step():
+            for mm, a, b, c, m, n, k in calls:
+                mm.enqueue(a, b, c, m, n, k)
+    else:
+        graph = dev.graph("gpt2_small_gemms")
+        for mm, a, b, c, m, n, k in calls:
+            mm(a, b, c, m, n, k, graph=graph)
+        graph.finish()
+
+        def run_step():
+            graph.enqueue()
+
+    for _ in range(args.warmup):
+        run_step()
+    dev.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run_step()
+    dev.sync()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    tflops = step_flops / (dt / args.steps) / 1e12
+
+    # Per-shape launch durations with HIP events on the library's stream
+    # (mg_gemm_time): best of 3 batches of back-to-back launches.
+    per_shape = []
+    for name, layout, m, n, k, count in gemm_list():
+        mm = mm_for(layout, m, n, k)
+        b = head if name.startswith("head") else sets[0][name.split(".")[0]]
+        role = name.split(".")[1]
+        a_, b_, c_ = {"fwd": (b["x"], b["w"], b["y"]), "dX": (b["dy"], b["w"], b["dx"]),
+                      "dW": (b["dy"], b["x"], b["dw"])}[role]
+        t1 = mm(a_, b_, c_, m, n, k)
+        rep = max(1, int(0.02 / max(t1, 1e-6)))
+        sec = min(mm(a_, b_, c_, m, n, k, repeat=rep) / rep for _ in range(3))
+        fl = 2.0 * m * n * k
+        by = 2.0 * (m * k + k * n) + 4.0 * m * n
+        tile, split, gm = mm.plan(m, n, k)
+        per_shape.append({"gemm": name, "layout": layout, "m": m, "n": n, "k": k, "count": count,
+                          "us": round(sec * 1e6, 2), "tflops": round(fl / sec / 1e12, 1),
+                          "frac_mfma": round(fl / sec / 1e12 / PEAK_TFLOPS, 4),
+                          "gbps": round(by / sec / 1e9, 1), "tile": tile, "split_k": split})
+    dom = max(per_shape, key=lambda r: r["us"] * r["count"])
+    roofline = {"bound": "mfma", "kernel": f"gemm {dom['gemm']} {dom['layout']} {dom['m']}x{dom['n']}x{dom['k']}",
+                "achieved": dom["tflops"], "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(dom["tflops"] / PEAK_TFLOPS, 4), "traffic": None}
+    events_ms = sum(r["us"] * r["count"] for r in per_shape) / 1e3
+
+    out = {
+        "metric": "GEMM TFLOP/s (fwd+dX+dW) at GPT-2-small shapes, % of fp16 MFMA peak, 1 GPU",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": DTYPE, "data": "synthetic",
+        "config": {"workload": "GPT-2-small training GEMMs: d_model 768, 12 layers, 8192 token rows, "
+                               "QKV/proj/MLP + tied head 50257, fwd+dX+dW, 147 GEMMs, 6.07 TFLOP per step",
+                   "rows": ROWS, "d_model": D, "layers": LAYERS, "vocab": VOCAB,
+                   "launch": "eager" if args.eager else "hip-graph replay"},
+        "frac_of_mfma_peak": round(tflops / PEAK_TFLOPS, 4),
+        "sum_of_event_timed_gemms_ms": round(events_ms, 4),
+        "roofline": roofline,
+        "device": {"name": dev.name, "compute_units": dev.compute_units, "clock_khz": dev.clock_khz,
+                   "derived_peak_tflops": round(dev.compute_units * 4 * 1024 * dev.clock_khz * 1e3 / 1e12, 1)},
+        "per_shape": per_shape,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline()
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+    dev.destroy()
+
+
+if __name__ == "__main__":
+    main()

@@ -79,6 +79,8 @@ typedef struct {
     int32_t threads;
     int32_t lds_bytes;         /* for the NT layout; other layouts differ by padding */
     int32_t min_m;             /* informational: smallest M this tile is meant for */
+    int32_t stages;            /* 0: register-staged kernel (any alignment); >0: direct-to-LDS ring depth */
+    int32_t fallback;          /* tile used instead when a direct-to-LDS tile's preconditions fail */
     char name[48];
 } mg_tile;
 
@@ -150,6 +152,9 @@ int mg_graph_begin(mg_ctx *ctx);
 int mg_graph_end(mg_ctx *ctx, mg_graph **out);
 /* Graph.submit — vk.py:877-889: replay and wait; *seconds = host wall time. */
 int mg_graph_launch(mg_ctx *ctx, mg_graph *g, double *seconds);
+/* Graph.submit without the fence wait (vk.py:1295 `wait=False` is the eager analogue):
+ * replay on the context's stream and return; mg_sync waits for it. */
+int mg_graph_enqueue(mg_ctx *ctx, mg_graph *g);
 int mg_graph_destroy(mg_ctx *ctx, mg_graph *g);
 
 /* ---- companion elementwise kernels: kernels.make_kernels (kernels.py:699-862) ----

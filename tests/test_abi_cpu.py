@@ -1,0 +1,266 @@
+"""CPU-only checks of the C ABI and the host logic: the library loads, exports
+every symbol include/mi_gemm.h declares, validates arguments before touching HIP,
+and the picker / tuner logic behaves.  No compute runs here.
+
+Error cases mirror the ones the reference can raise from the host
+(kernels.py:274-276, 247-248; vk.py:843-844, 878-879, 1184-1185, 586-587;
+autograd.py:39-40)."""
+
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from vkgrad_amd import _lib as L
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return L.load()
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "mi_gemm.h")).read()
+    return sorted(set(re.findall(r"\b(mg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree(lib):
+    names = declared_symbols()
+    assert len(names) >= 25
+    for n in names:
+        assert hasattr(lib, n), f"libmigemm.so does not export {n}"
+        assert n in L.SIGNATURES, f"{n} is declared in the header but not bound"
+    assert set(L.SIGNATURES) == set(names)
+
+
+def test_struct_layouts_match(lib):
+    # the library checks struct_size; a mismatch would make every call fail
+    ga = L.GemmArgs()
+    ga.struct_size = C.sizeof(L.GemmArgs) - 8
+    assert lib.mg_gemm_check(C.byref(ga)) == L.MG_ERR_ARG
+    assert "struct_size" in L.last_error()
+    t = L.Tile()
+    assert lib.mg_tile_info(0, C.byref(t)) == L.MG_OK and t.bm > 0 and t.name
+
+
+def good_args(**kw):
+    ga = L.GemmArgs()
+    ga.struct_size = C.sizeof(L.GemmArgs)
+    ga.layout, ga.dtype, ga.beta = L.MG_NN, L.MG_F16, 0
+    ga.m, ga.n, ga.k = 128, 96, 64
+    ga.a, ga.b, ga.c = 0x1000, 0x2000, 0x3000
+    ga.lda, ga.ldb, ga.ldc = 64, 96, 96
+    ga.nbatch, ga.tile = 1, -1
+    for k, v in kw.items():
+        setattr(ga, k, v)
+    return ga
+
+
+def test_validation_accepts_ragged_shapes(lib):
+    assert lib.mg_gemm_check(C.byref(good_args())) == L.MG_OK
+    # any positive shape is legal (the reference refuses non-tile-multiples)
+    assert lib.mg_gemm_check(C.byref(good_args(m=1, n=7, k=3, lda=3, ldb=7, ldc=7))) == L.MG_OK
+    assert lib.mg_gemm_check(C.byref(good_args(m=4097, n=50257, k=768, lda=768, ldb=50257, ldc=50257))) == L.MG_OK
+
+
+@pytest.mark.parametrize("kw,needle", [
+    (dict(layout=3), "layout"), (dict(dtype=2), "dtype"), (dict(beta=2), "beta"),
+    (dict(m=0), "positive"), (dict(k=-5), "positive"), (dict(a=None), "NULL"), (dict(c=None), "NULL"),
+    (dict(a=0x1001), "2-byte"), (dict(c=0x3002), "4-byte"), (dict(bias=0x4002), "bias"),
+    (dict(lda=63), "lda"), (dict(ldb=95), "ldb"), (dict(ldc=95), "ldc"),
+    (dict(nbatch=0), "nbatch"), (dict(nbatch=2, sc=0), "overwrite"), (dict(nbatch=2, sc=10), "overlap"),
+    (dict(tile=999), "tile"), (dict(split_k=-1), "split_k"), (dict(group_m=-2), "group_m"),
+    (dict(m=2 ** 31), "32-bit"),
+])
+def test_validation_rejects(lib, kw, needle):
+    assert lib.mg_gemm_check(C.byref(good_args(**kw))) == L.MG_ERR_ARG
+    assert needle in L.last_error(), L.last_error()
+
+
+def test_layout_dependent_leading_dimensions(lib):
+    # TN: A is (K, M), so lda >= M; NT: B is (N, K), so ldb >= K
+    assert lib.mg_gemm_check(C.byref(good_args(layout=L.MG_TN, lda=128))) == L.MG_OK
+    assert lib.mg_gemm_check(C.byref(good_args(layout=L.MG_TN, lda=64))) == L.MG_ERR_ARG
+    assert lib.mg_gemm_check(C.byref(good_args(layout=L.MG_NT, ldb=64))) == L.MG_OK
+    assert lib.mg_gemm_check(C.byref(good_args(layout=L.MG_NT, ldb=63))) == L.MG_ERR_ARG
+
+
+def test_null_context_is_an_error_not_a_crash(lib):
+    assert lib.mg_gemm(None, C.byref(good_args())) == L.MG_ERR_ARG
+    assert lib.mg_sync(None) == L.MG_ERR_ARG
+    assert lib.mg_ew_zero(None, 0x1000, 4) == L.MG_ERR_ARG
+    assert lib.mg_destroy(None) == L.MG_OK
+
+
+def test_init_without_gpu_reports_nodevice(lib):
+    import subprocess, sys
+    # in a subprocess: on a GPU box this would create a context we do not want here
+    code = ("import ctypes as C, sys; sys.path.insert(0, %r); from vkgrad_amd import _lib as L; l = L.load(); "
+            "c = C.c_void_p(); rc = l.mg_init(0, C.byref(c)); print(rc, L.last_error()); "
+            "l.mg_destroy(c) if rc == 0 else None" % ROOT)
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120).stdout
+    rc = int(out.split()[0])
+    assert rc in (L.MG_OK, L.MG_ERR_NODEVICE), out
+    if rc == L.MG_ERR_NODEVICE:
+        assert "no HIP device" in out
+
+
+def test_tile_table(lib):
+    n = lib.mg_tile_count()
+    assert n >= 9
+    seen = set()
+    for i in range(n):
+        t = L.Tile()
+        assert lib.mg_tile_info(i, C.byref(t)) == L.MG_OK
+        assert t.id == i and t.threads == t.waves_m * t.waves_n * 64
+        assert t.bm % (32 * t.waves_m) == 0 and t.bn % (32 * t.waves_n) == 0
+        assert t.lds_bytes <= 160 * 1024
+        assert 0 <= t.fallback < n
+        fb = L.Tile()
+        lib.mg_tile_info(t.fallback, C.byref(fb))
+        assert fb.stages == 0 and (fb.bm, fb.bn) == (t.bm, t.bn)
+        seen.add(t.name)
+    assert len(seen) == n
+    assert lib.mg_tile_info(n, C.byref(L.Tile())) == L.MG_ERR_ARG
+    assert lib.mg_tile_fits(0, C.byref(good_args())) == 1
+    assert lib.mg_tile_fits(n, C.byref(good_args())) == 0
+
+
+def pick(lib, cus=256, **kw):
+    t, s, g = C.c_int(), C.c_int(), C.c_int()
+    assert lib.mg_pick(C.byref(good_args(**kw)), cus, C.byref(t), C.byref(s), C.byref(g)) == L.MG_OK
+    info = L.Tile()
+    lib.mg_tile_info(t.value, C.byref(info))
+    return info, s.value, g.value
+
+
+def test_picker_properties(lib):
+    # a big aligned square problem gets a big tile and no K split
+    info, split, gm = pick(lib, m=8192, n=8192, k=8192, lda=8192, ldb=8192, ldc=8192)
+    assert info.bm * info.bn >= 128 * 128 and split == 1 and gm >= 1
+    # deep-K, small-MN (a dW shape) is split along K to fill the chip
+    info, split, _ = pick(lib, layout=L.MG_TN, m=768, n=768, k=8192, lda=768, ldb=768, ldc=768)
+    assert split > 1
+    assert -(-768 // info.bm) * -(-768 // info.bn) * split >= 64
+    # unaligned operands never get a direct-to-LDS tile
+    info, _, _ = pick(lib, m=8192, n=768, k=50257, lda=50257, ldb=768, ldc=768)
+    assert info.stages == 0
+    # an explicit split is honoured, an explicit tile too
+    info, split, _ = pick(lib, m=1024, n=1024, k=4096, lda=4096, ldb=1024, ldc=1024, tile=3, split_k=4)
+    assert info.id == 3 and split == 4
+    # a split never exceeds the number of K blocks
+    _, split, _ = pick(lib, m=128, n=96, k=64, tile=3, split_k=50)
+    assert split == 1
+    # tiny problems still get a plan
+    info, split, _ = pick(lib, m=1, n=1, k=1, lda=1, ldb=1, ldc=1)
+    assert split == 1
+
+
+# ---------------------------------------------------------------------------
+# Python surface
+# ---------------------------------------------------------------------------
+
+class FakeDev:
+    name = "fake-mi355x"
+    compute_units = 256
+
+
+def test_matmul_object_surface():
+    from vkgrad_amd.kernels import CONFIGS, Matmul
+    from vkgrad_amd.vk import VkError
+    mm = Matmul(FakeDev(), 8, 2, 8, trans_b=True)       # reference-style (sg, wm, wn): 256 x 128
+    assert (mm.bm, mm.bn) == (256, 128) and mm.trans_b and not mm.trans_a
+    assert mm.fits(1, 7, 3) and not mm.fits(0, 1, 1)
+    assert mm.flops(2, 3, 4) == 48
+    assert mm.traffic_bytes(4, 8, 16) == 2 * (4 * 16 + 16 * 8) + 4 * 4 * 8
+    assert "tb" in mm.name
+    with pytest.raises(VkError):
+        Matmul(FakeDev(), trans_a=True, trans_b=True)
+    with pytest.raises(VkError):
+        Matmul(FakeDev(), acc16=True)
+    with pytest.raises(VkError):
+        Matmul(FakeDev(), dtype="f32")
+    with pytest.raises(VkError):
+        Matmul(FakeDev(), tile=len(CONFIGS))
+
+
+def test_pick_config_restatement():
+    from vkgrad_amd.autograd import pick_config
+    from vkgrad_amd.kernels import CONFIGS
+    t = CONFIGS[pick_config(8192, 8192, 8192)]
+    assert t["bm"] * t["bn"] == max(c["bm"] * c["bn"] for c in CONFIGS)
+    small = CONFIGS[pick_config(64, 64, 64)]
+    assert small["bm"] * small["bn"] <= 64 * 64      # most workgroups wins when nothing fills the chip
+
+
+def test_autotuner_logic_with_fake_timer(tmp_path, monkeypatch):
+    """Round-robin order, equal-time repeats, best-of-reps, cache reuse
+    (kernels.py:433-447, 462-466, 513-521) — against a deterministic fake clock."""
+    import vkgrad_amd.kernels as K
+    monkeypatch.setattr(K, "_TUNE_CACHE", str(tmp_path / "tune.json"))
+    monkeypatch.setattr(K, "_SHIPPED_CACHE", str(tmp_path / "none.json"))
+    calls = []
+    fast_tile = K.CONFIGS[3]["id"]
+
+    def timer(mm, repeat):
+        calls.append((mm.tile, mm.split_k, mm.group_m, repeat))
+        per = 1e-4 if mm.tile == fast_tile else 5e-4
+        if mm.group_m == 4:
+            per *= 0.9
+        return per * repeat
+
+    mm, best = K.autotune_matmul(FakeDev(), 1024, 1024, 1024, reps=3, timer=timer)
+    assert best["tile_id"] == fast_tile and best["group_m"] == 4 and mm.tile == fast_tile
+    assert best["tflops"] > 0 and best["evaluated"] >= 2 and "pruned" in best and best["lds"] is True
+    # equal GPU time per candidate: slow candidates get proportionally fewer repeats
+    first_stage2 = next(i for i, c in enumerate(calls) if c[2] != 0)
+    stage1 = [c for c in calls[:first_stage2 - 1] if c[3] > 1]
+    reps_fast = {c[3] for c in stage1 if c[0] == fast_tile}
+    reps_slow = {c[3] for c in stage1 if c[0] != fast_tile}
+    assert reps_fast and reps_slow and min(reps_fast) == 5 * max(reps_slow)
+    # round-robin: no candidate is measured twice in a row within stage one
+    timed = [c[:2] for c in stage1]
+    ncand = len(set(timed))
+    assert ncand > 1 and len(timed) == 3 * ncand
+    assert timed[:ncand] == timed[ncand:2 * ncand] == timed[2 * ncand:]
+    # cached pick is reused without timing anything
+    n = len(calls)
+    mm2, e = K.autotune_matmul(FakeDev(), 1024, 1024, 1024, timer=timer)
+    assert len(calls) == n and mm2.tile == fast_tile and e["tile_id"] == fast_tile
+    # a different dtype or layout is a different key
+    assert K.tune_key("d", 1, 2, 3, False, True, "bf16") != K.tune_key("d", 1, 2, 3, False, True, "f16")
+    assert K.tune_key("d", 1, 2, 3, False, True) != K.tune_key("d", 1, 2, 3, True, False)
+
+
+def test_graph_state_errors():
+    from vkgrad_amd.vk import Graph, VkError
+    g = Graph(FakeDev(), "g")
+    with pytest.raises(VkError):
+        g.submit()                      # submit before finish (vk.py:878-879)
+    with pytest.raises(VkError):
+        g.finish()                      # nothing recorded
+    with pytest.raises(VkError):
+        g.record("not callable")
+    g._finished = True
+    with pytest.raises(VkError):
+        g.record(lambda: None)          # record after finish (vk.py:843-844)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(L, "_lib", None)
+    monkeypatch.setattr(L, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(OSError, match="build it"):
+        L.load()
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "vkgrad_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, f"{f} mentions the oracle"
+                assert "_work" not in text

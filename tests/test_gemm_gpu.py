@@ -72,6 +72,34 @@ def test_every_tile_every_layout_exact(dev):
                 assert r["exact"], f"{layout} {dtype} tile {t['name']}: max diff {np.abs(got - ref).max()}"
 
 
+def test_direct_to_lds_tiles_exact(dev):
+    """Aligned shapes that keep the direct-to-LDS kernels eligible (K a multiple
+    of every BK, extents multiples of 8 but not of the tile, so edge clamping
+    runs), every tile x layout x dtype, with bias, beta=1 and a K split."""
+    from vkgrad_amd.kernels import CONFIGS
+    m, n, k = 392, 648, 512
+    for layout, (ta, tb) in LAYOUTS.items():
+        for dtype in ("f16", "bf16"):
+            for t in CONFIGS:
+                if not t["stages"]:
+                    continue
+                for split in (1, 2):
+                    r, got, ref = check_case(dev, m, n, k, ta, tb, dtype, seed=13, tile=t["id"], integer=True,
+                                             bias=True, accumulate=True, split_k=split)
+                    assert r["exact"], (f"{layout} {dtype} tile {t['name']} split {split}: "
+                                        f"max diff {np.abs(got - ref).max()}")
+
+
+def test_direct_to_lds_plan_is_used(dev):
+    """The picker must keep a direct-to-LDS tile when its preconditions hold and
+    fall back to the register-staged sibling when they do not."""
+    from vkgrad_amd.kernels import CONFIGS, Matmul
+    dma = next(t for t in CONFIGS if t["stages"])
+    mm = Matmul(dev, trans_b=True, tile=dma["id"])
+    assert mm.plan(512, 512, 512)[0] == dma["id"]
+    assert mm.plan(512, 512, 500)[0] == dma["fallback"]      # K not a multiple of BK
+
+
 @pytest.mark.parametrize("layout", list(LAYOUTS))
 def test_ragged_small_exact(dev, layout):
     """Odd shapes (unaligned rows, K tails of every residue) through the

@@ -1,0 +1,211 @@
+"""GPU checks of the runtime surface (Device, Buffer, Graph) and the elementwise
+companions, following /root/reference/test_runtime.py (memory kinds :139-149,
+zero-copy round trip :57-75, one MFMA-sized tile :103-136) and test_accum.py
+(accumulation over micro-batches :139-168)."""
+
+import numpy as np
+import pytest
+
+from oracle import ref_gemm as O
+from tests.util import run_gemm
+
+pytestmark = pytest.mark.gpu
+
+
+def test_memory_kinds_round_trip(dev):
+    from vkgrad_amd.vk import VkError
+    for kind in ("device", "shared", "cached", "bar"):
+        b = dev.buffer(1 << 16, kind)
+        try:
+            if b.host_visible:
+                b.array(np.uint32)[:16] = np.arange(16, dtype=np.uint32)
+                assert np.array_equal(b.array(np.uint32)[:16], np.arange(16))
+            else:
+                with pytest.raises(VkError):
+                    b.array(np.uint32)
+                b.upload(np.arange(16, dtype=np.uint32))
+                assert np.array_equal(b.download(np.uint32, (16,)), np.arange(16))
+        finally:
+            b.destroy()
+    with pytest.raises(VkError):
+        dev.buffer(64, "texture")
+    with pytest.raises(VkError):
+        dev.buffer(0, "device")
+
+
+def test_zero_copy_round_trip(dev):
+    """A host-visible tensor is a numpy array and a GPU buffer at once."""
+    from vkgrad_amd.kernels import make_kernels
+    K = make_kernels(dev)
+    n = 4096
+    src = dev.buffer(n * 4, "shared")
+    dst = dev.buffer(n * 4, "shared")
+    x = src.array(np.float32, (n,))
+    x[:] = np.arange(n, dtype=np.float32)
+    d = dst.array(np.float32, (n,))
+    d[:] = 1.0
+    src.flush()
+    K["grad_add"]([dst, src], n)          # dst += src on the device, visible through the view
+    dst.invalidate()
+    assert np.array_equal(d, np.arange(n, dtype=np.float32) + 1.0)
+    src.destroy()
+    dst.destroy()
+
+
+def test_device_copy(dev):
+    a = dev.buffer(1024, "shared")
+    b = dev.buffer(1024, "device")
+    c = dev.buffer(1024, "cached")
+    a.array(np.uint8)[:] = np.arange(1024) % 251
+    dev.copy(a, b)
+    dev.copy(b, c, 512)
+    assert np.array_equal(c.array(np.uint8)[:512], a.array(np.uint8)[:512])
+    for x in (a, b, c):
+        x.destroy()
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_single_mfma_tile(dev, dtype):
+    """32x32x16: one accumulator tile, one K step (test_runtime.py:103-136 does 16^3)."""
+    a, b = O.make_operands(32, 32, 16, False, True, dtype, seed=0)
+    got = run_gemm(dev, a, b, 32, 32, 16, False, True, dtype)
+    ref = O.ref_gemm(a, b, False, True, dtype)
+    assert np.abs(got - ref).max() < 1e-4
+
+
+def test_golden_vectors_through_hip(dev):
+    import os
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "gemm_golden.npz"))
+    LAY = {"NN": (False, False), "NT": (False, True), "TN": (True, False)}
+    names = sorted({k.rsplit("_", 1)[0] for k in z.files})
+    for name in names:
+        layout, dtype = name.split("-")[1:3]
+        ta, tb = LAY[layout]
+        a, b, c = z[name + "_a"], z[name + "_b"], z[name + "_c"]
+        if dtype == "f16":
+            a, b = a.view(np.float16), b.view(np.float16)
+        m, n = c.shape
+        k = a.shape[0] if ta else a.shape[1]
+        bias = z[name + "_bias"] if name + "_bias" in z.files else None
+        c0 = z[name + "_c0"] if name + "_c0" in z.files else None
+        got = run_gemm(dev, a, b, m, n, k, ta, tb, dtype, bias, c0)
+        assert O.err_fro(got, c) <= 1e-5, name
+        assert np.abs(got - c).max() <= 1e-4 * max(1.0, np.abs(c).max()), name
+
+
+@pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
+def test_strided_batched(dev, layout):
+    """z-batched GEMM with element strides (kernels.py:58-62, 98-101), at the
+    attention shapes' pattern: several small matrices per launch."""
+    from vkgrad_amd.kernels import Matmul
+    ta, tb = {"NN": (False, False), "NT": (False, True), "TN": (True, False)}[layout]
+    m, n, k, nb = 96, 64, 40, 5
+    rng = np.random.default_rng(1)
+    a = rng.integers(-3, 4, nb * m * k).astype(np.float16)
+    b = rng.integers(-3, 4, nb * k * n).astype(np.float16)
+    strides = (m * k, k * n, m * n)
+    ba, bb, bc = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), dev.buffer(nb * m * n * 4, "device")
+    ba.upload(a)
+    bb.upload(b)
+    mm = Matmul(dev, trans_a=ta, trans_b=tb, batched=True)
+    mm(ba, bb, bc, m, n, k, nbatch=nb, strides=strides)
+    got = bc.download(np.float32, (nb * m * n,))
+    ref = O.ref_gemm_batched(a, b, m, n, k, nb, strides, ta, tb)
+    assert np.array_equal(got, ref)
+    for x in (ba, bb, bc):
+        x.destroy()
+
+
+def test_dw_accumulation_over_micro_batches(dev):
+    """beta=1 over 4 micro-batches == one GEMM over the concatenated rows, also
+    into a dirty accumulator (test_accum.py:51-58, 149-166)."""
+    from vkgrad_amd.kernels import Matmul
+    m, n, rows, micro = 192, 160, 256, 4
+    parts = [O.make_operands(m, n, rows, True, False, "bf16", seed=20 + i) for i in range(micro)]
+    for start in (0.0, 5.0):
+        bc = dev.buffer(m * n * 4, "device")
+        bc.upload(np.full((m, n), start, np.float32))
+        mm = Matmul(dev, trans_a=True, dtype="bf16")
+        for a, b in parts:
+            ba, bb = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device")
+            ba.upload(a)
+            bb.upload(b)
+            mm(ba, bb, bc, m, n, rows, accumulate=True)
+            ba.destroy()
+            bb.destroy()
+        got = bc.download(np.float32, (m, n))
+        ref = O.ref_gemm_accumulate(parts, True, False, "bf16", np.full((m, n), start, np.float32))
+        big = O.ref_gemm(np.concatenate([p[0] for p in parts]), np.concatenate([p[1] for p in parts]),
+                         True, False, "bf16") + start
+        assert O.err_fro(got, ref) <= 1e-5
+        assert O.err_fro(got, big) <= 2e-5        # measured 8.8e-06 in the reference
+        bc.destroy()
+
+
+def test_graph_records_and_replays_gemm_with_split_k(dev):
+    """A recorded split-K GEMM (fill kernel + atomics) must give the same answer
+    on every replay, with eager work and syncs between replays."""
+    from vkgrad_amd.kernels import Matmul
+    m, n, k = 256, 192, 4096
+    a, b = O.make_operands(m, n, k, True, False, "f16", seed=8, integer=True)
+    ref = O.ref_gemm(a, b, True, False, "f16")
+    ba, bb, bc = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), dev.buffer(m * n * 4, "device")
+    ba.upload(a)
+    bb.upload(b)
+    mm = Matmul(dev, trans_a=True, tile=3, split_k=8)
+    g = dev.graph("splitk")
+    mm(ba, bb, bc, m, n, k, graph=g)
+    g.finish()
+    for i in range(4):
+        bc.upload(np.full((m, n), np.nan, np.float32))
+        g.submit()
+        assert np.array_equal(bc.download(np.float32, (m, n)), ref), f"replay {i}"
+        mm(ba, bb, bc, m, n, k)                      # eager work between replays
+        dev.sync()
+    g.destroy()
+    for x in (ba, bb, bc):
+        x.destroy()
+
+
+def test_elementwise_kernels(dev):
+    from vkgrad_amd.kernels import make_kernels
+    from oracle import ref_mlp as RM
+    K = make_kernels(dev, "f16")
+    rng = np.random.default_rng(0)
+    rows, ncol = 37, 50
+    n = rows * ncol
+    acc = rng.standard_normal((rows, ncol)).astype(np.float32)
+    bias = rng.standard_normal(ncol).astype(np.float32)
+
+    def up(x):
+        b = dev.buffer(max(x.nbytes, 4), "device")
+        b.upload(x)
+        return b
+
+    bacc, bbias = up(acc), up(bias)
+    bz, by = dev.buffer(n * 4, "device"), dev.buffer(n * 2, "device")
+    for name, act in (("bias_gelu", "gelu"), ("bias_relu", "relu")):
+        K[name]([bacc, bbias, bz, by], n, ncol)
+        z = bz.download(np.float32, (rows, ncol))
+        y = by.download(np.float16, (rows, ncol))
+        assert np.array_equal(z, acc + bias[None, :])
+        want = RM.act_fn(z, act).astype(np.float16)
+        assert np.abs(y.astype(np.float32) - want.astype(np.float32)).max() <= 2e-3
+    # col_sum and its accumulating form
+    bs = dev.buffer(ncol * 4, "device")
+    K["col_sum"]([bz, bs], ncol, rows)
+    s1 = bs.download(np.float32, (ncol,))
+    assert np.allclose(s1, z.sum(0), rtol=1e-5, atol=1e-5)
+    K["col_sum_acc"]([bz, bs], ncol, rows)
+    assert np.allclose(bs.download(np.float32, (ncol,)), 2 * s1, rtol=1e-6, atol=1e-6)
+    # cast16 in both types is round-to-nearest-even
+    x = rng.standard_normal(1000).astype(np.float32)
+    bx, b16 = up(x), dev.buffer(2000, "device")
+    K["cast16"]([bx, b16], 1000)
+    assert np.array_equal(b16.download(np.float16, (1000,)), x.astype(np.float16))
+    Kb = make_kernels(dev, "bf16")
+    Kb["cast16"]([bx, b16], 1000)
+    assert np.array_equal(b16.download(np.uint16, (1000,)), O.f32_to_bf16_bits(x))
+    # zero
+    K["zero"]([bx], 1000)
+    assert not bx.download(np.float32, (1000,)).any()

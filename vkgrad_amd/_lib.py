@@ -35,7 +35,8 @@ class Tile(C.Structure):
     _fields_ = [
         ("id", C.c_int32), ("bm", C.c_int32), ("bn", C.c_int32), ("bk", C.c_int32),
         ("waves_m", C.c_int32), ("waves_n", C.c_int32), ("threads", C.c_int32),
-        ("lds_bytes", C.c_int32), ("min_m", C.c_int32), ("name", C.c_char * 48),
+        ("lds_bytes", C.c_int32), ("min_m", C.c_int32), ("stages", C.c_int32), ("fallback", C.c_int32),
+        ("name", C.c_char * 48),
     ]
 
 
@@ -71,6 +72,7 @@ SIGNATURES = {
     "mg_graph_begin": (C.c_int, [_P]),
     "mg_graph_end": (C.c_int, [_P, C.POINTER(_P)]),
     "mg_graph_launch": (C.c_int, [_P, _P, C.POINTER(C.c_double)]),
+    "mg_graph_enqueue": (C.c_int, [_P, _P]),
     "mg_graph_destroy": (C.c_int, [_P, _P]),
     "mg_ew_bias_act": (C.c_int, [_P, _P, _P, _P, _P, C.c_int64, C.c_int64, C.c_int, C.c_int]),
     "mg_ew_act_bwd": (C.c_int, [_P, _P, _P, _P, _P, C.c_int64, C.c_int, C.c_int]),

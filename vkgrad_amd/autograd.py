@@ -27,14 +27,18 @@ from .vk import VkError
 
 def pick_config(m, n, k, trans_a=False, trans_b=False, min_groups=256):
     """Tile chosen without benchmarking (autograd.py:22-41): the largest tile
-    area that still gives min_groups workgroups (one per CU of an MI355X),
-    else the most workgroups.  Returns the tile id.  The library's own picker
-    (mg_pick) refines this with padding waste and K splits; this restatement
-    exists for callers that used the reference function directly."""
+    area that still gives min_groups workgroups (one per CU of an MI355X).  The
+    reference only considers tiles that divide the shape; ragged shapes are
+    legal here, so "divides" becomes "wastes under half of the tile grid on
+    padding".  Returns the tile id.  The library's own picker (mg_pick) prices
+    the same trade-off with K splits as well; this restatement exists for
+    callers that used the reference function directly."""
     best = None
     for t in CONFIGS:
-        groups = -(-m // t["bm"]) * -(-n // t["bn"])
-        score = (groups >= min_groups, t["bm"] * t["bn"], groups)
+        gm, gn = -(-m // t["bm"]), -(-n // t["bn"])
+        groups = gm * gn
+        useful = (m * n) / (gm * t["bm"] * gn * t["bn"])
+        score = (useful >= 0.5, groups >= min_groups, t["bm"] * t["bn"], groups)
         if best is None or score > best[0]:
             best = (score, t["id"])
     if best is None:

@@ -1,10 +1,15 @@
-// Instantiations of the GEMM template: layout TN, dtype BF16, every tile, aligned and general.
+// Instantiations of the GEMM templates: layout TN, dtype BF16, every tile.
+// Entry [tile][0] serves aligned operands, [tile][1] arbitrary alignment (absent
+// for direct-to-LDS tiles, which fall back to a register-staged tile instead).
+#include "gemm_dma_kernel.h"
 #include "gemm_kernel.h"
 #include "tiles.h"
 
 namespace mg {
-#define X(id, bm, bn, bk, wgm, wgn)                                                   \
+#define V(id, bm, bn, bk, wgm, wgn) \
     {launch_gemm<L_TN, D_BF16, bm, bn, bk, wgm, wgn, false>, launch_gemm<L_TN, D_BF16, bm, bn, bk, wgm, wgn, true>},
-launch_fn launch_table_tn_bf16[MG_NUM_TILES][2] = {MG_TILE_LIST(X)};
-#undef X
+#define D(id, bm, bn, bk, wgm, wgn, ns, fb) {launch_gemm_dma<L_TN, D_BF16, bm, bn, bk, wgm, wgn, ns>, nullptr},
+launch_fn launch_table_tn_bf16[MG_NUM_TILES][2] = {MG_TILE_LIST(V, D)};
+#undef V
+#undef D
 }  // namespace mg

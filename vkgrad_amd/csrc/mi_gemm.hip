@@ -33,10 +33,14 @@ __global__ void zero_c_kernel(float *C, int64_t ldc, int M, int N, int64_t sc) {
 
 struct TileDesc {
     int id, bm, bn, bk, wgm, wgn;
+    int nstage;     // 0: register-staged kernel; >0: direct-to-LDS ring depth
+    int fallback;   // register-staged tile of the same BM x BN (self for those)
 };
-#define X(id, bm, bn, bk, wgm, wgn) {id, bm, bn, bk, wgm, wgn},
-static const TileDesc g_tiles[MG_NUM_TILES] = {MG_TILE_LIST(X)};
-#undef X
+#define V(id, bm, bn, bk, wgm, wgn) {id, bm, bn, bk, wgm, wgn, 0, id},
+#define D(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb},
+static const TileDesc g_tiles[MG_NUM_TILES] = {MG_TILE_LIST(V, D)};
+#undef V
+#undef D
 
 static thread_local char g_err[512] = "";
 
@@ -70,6 +74,7 @@ static launch_fn (*table_for(int layout, int dtype))[2] {
 }
 
 static int lds_bytes_for(const TileDesc &t, int layout) {
+    if (t.nstage > 0) return t.nstage * (t.bm + t.bn) * t.bk * 2;
     const bool a_kc = layout != MG_TN, b_kc = layout == MG_NT;
     const int a = a_kc ? t.bm * (t.bk + 8) : t.bk * (t.bm + 32);
     const int b = b_kc ? t.bn * (t.bk + 8) : t.bk * (t.bn + 32);
@@ -95,61 +100,127 @@ struct Plan {
     int tile, split_k, group_m, k_per_split, grid_m, grid_n, xcd_remap;
 };
 
-// Heuristic choice of tile, K split and rasterisation band.  Pure integer
-// arithmetic, so it is testable without a device.
-static void pick_plan(const mg_gemm_args &a, int cus, Plan &pl) {
-    if (cus <= 0) cus = 256;
-    int tile = a.tile;
-    if (tile < 0) {
-        // Largest tile that still yields at least ~one workgroup per CU; tie
-        // break on the least padding waste.
-        double best = -1.0;
-        for (int t = 0; t < MG_NUM_TILES; t++) {
-            const TileDesc &d = g_tiles[t];
-            const int64_t gm = cdiv(a.m, d.bm), gn = cdiv(a.n, d.bn);
-            const double useful = (double)a.m * (double)a.n / ((double)gm * d.bm * (double)gn * d.bn);
-            const int64_t groups = gm * gn * (int64_t)a.nbatch;
-            // per-workgroup efficiency grows with tile area (operand reuse) ...
-            const double area_eff = (double)d.bm * d.bn / (double)(d.bm + d.bn) / 128.0;
-            // ... and whole-chip efficiency with how evenly the grid fills the CUs.
-            const int64_t waves = cdiv(groups, cus);
-            const double fill = (double)groups / (double)(waves * cus);
-            // split-K can recover fill for deep-K problems
-            const double fill_eff = (a.k >= 2048 && fill < 0.5) ? 0.5 + 0.4 * fill : fill;
-            const double score = useful * area_eff * fill_eff;
-            if (score > best) {
-                best = score;
-                tile = t;
-            }
-        }
-    }
-    const TileDesc &d = g_tiles[tile];
-    pl.tile = tile;
-    pl.grid_m = (int)cdiv(a.m, d.bm);
-    pl.grid_n = (int)cdiv(a.n, d.bn);
-    const int64_t groups = (int64_t)pl.grid_m * pl.grid_n * a.nbatch;
-    const int64_t kblocks = cdiv(a.k, d.bk);
-    int split = a.split_k;
-    if (split <= 0) {
-        split = 1;
-        if (groups * 2 <= cus && kblocks >= 8) {
-            split = (int)(cus / groups);
-            // keep at least 4 K-blocks per slice so the pipeline prologue amortises
-            if (split > kblocks / 4) split = (int)(kblocks / 4);
-            if (split < 1) split = 1;
-        }
-    }
+// Preconditions of the direct-to-LDS kernels (gemm_dma_kernel.h).
+static bool dma_eligible(const mg_gemm_args &a, const TileDesc &t, int64_t k_per_split) {
+    if (t.nstage == 0) return true;
+    if (!operands_aligned(a)) return false;
+    if (a.k % t.bk != 0 || k_per_split % t.bk != 0) return false;
+    if (a.layout == MG_TN && a.m < 8) return false;
+    if (a.layout != MG_NT && a.n < 8) return false;
+    return true;
+}
+
+// Sustained MFMA rate of a tile's main loop relative to the chip's dense peak,
+// from measurements on MI355X at large K (it only has to rank the tiles).
+static double tile_efficiency(const TileDesc &t) {
+    const int area = t.bm * t.bn;
+    if (t.nstage > 0) return area >= 65536 ? 0.55 : (area >= 32768 ? 0.45 : 0.48);
+    if (area >= 65536) return 0.42;
+    if (area >= 32768) return 0.36;
+    if (area >= 16384) return 0.34;
+    if (area >= 8192) return 0.22;
+    return 0.14;
+}
+
+static int wgs_per_cu(const TileDesc &t, int layout) {
+    const int by_lds = 163840 / lds_bytes_for(t, layout);
+    const int acc_regs = t.bm * t.bn / (t.wgm * t.wgn * 64);          // per lane
+    const int waves_per_simd = acc_regs > 128 ? 1 : (acc_regs > 64 ? 2 : 4);
+    const int by_regs = waves_per_simd * 4 / (t.wgm * t.wgn);
+    int w = by_lds < by_regs ? by_lds : by_regs;
+    return w < 1 ? 1 : w;
+}
+
+// Estimated time (microseconds) of one (tile, split) choice: rounds of
+// co-resident workgroups, each round paying the main loop at the tile's rate
+// plus the part of its pipeline fill and C traffic that nothing overlaps.
+static double plan_cost_us(const mg_gemm_args &a, const TileDesc &t, int split, int cus) {
+    const int64_t gm = cdiv(a.m, t.bm), gn = cdiv(a.n, t.bn);
+    const int64_t groups = gm * gn * (int64_t)a.nbatch * split;
+    const int wpc = wgs_per_cu(t, a.layout);
+    const int64_t slots = (int64_t)cus * wpc;
+    const int64_t rounds = cdiv(groups, slots);
+    const double cu_rate = tile_efficiency(t) * 2.5e9 / 256.0;       // FLOP per us per CU
+    const double wg_flop = 2.0 * t.bm * t.bn * ((double)a.k / split);
+    // a round keeps min(wpc, groups/cus) workgroups on a CU, sharing its rate
+    const double busy = groups >= slots ? wpc : (groups > cus ? (double)groups / cus : 1.0);
+    const double loop_us = rounds * busy * wg_flop / cu_rate;
+    const double fill_us = rounds * 2.0 / (busy > 1.0 ? busy : 1.0);
+    const double c_bytes = (double)a.m * a.n * 4.0 * a.nbatch * (split > 1 ? 2.0 * split : (a.beta ? 2.0 : 1.0));
+    const double c_us = c_bytes / 4.5e6 * (busy > 1.0 ? 0.6 : 1.0);
+    return loop_us + fill_us + c_us + (split > 1 && !a.beta ? 3.0 : 0.0);
+}
+
+static void finish_plan(const mg_gemm_args &a, int tile, int split, Plan &pl) {
+    const TileDesc *d = &g_tiles[tile];
+    int64_t kblocks = cdiv(a.k, d->bk);
     if (split > kblocks) split = (int)kblocks;
     if (split < 1) split = 1;
     int64_t kb_per = cdiv(kblocks, split);
     split = (int)cdiv(kblocks, kb_per);   // no empty slices
+    if (!dma_eligible(a, *d, kb_per * d->bk)) {
+        tile = d->fallback;
+        d = &g_tiles[tile];
+        kblocks = cdiv(a.k, d->bk);
+        if (split > kblocks) split = (int)kblocks;
+        kb_per = cdiv(kblocks, split);
+        split = (int)cdiv(kblocks, kb_per);
+    }
+    pl.tile = tile;
+    pl.grid_m = (int)cdiv(a.m, d->bm);
+    pl.grid_n = (int)cdiv(a.n, d->bn);
     pl.split_k = split;
-    pl.k_per_split = (int)(kb_per * d.bk);
+    pl.k_per_split = (int)(kb_per * d->bk);
     int gm = a.group_m;
     if (gm <= 0) gm = 8;
     if (gm > pl.grid_m) gm = pl.grid_m;
     pl.group_m = gm;
     pl.xcd_remap = ((int64_t)pl.grid_m * pl.grid_n) % 8 == 0 ? 1 : 0;
+}
+
+// Heuristic choice of tile, K split and rasterisation band (the reference's
+// pick_config, autograd.py:22-41, picks the largest tile that still fills its
+// 12 CUs; here the same trade-off is priced with a small cost model).  Pure
+// arithmetic, so it is testable without a device.
+static void pick_plan(const mg_gemm_args &a, int cus, Plan &pl) {
+    if (cus <= 0) cus = 256;
+    int tile = a.tile, split = a.split_k;
+    if (tile < 0 || split <= 0) {
+        double best = 1e300;
+        int bt = tile < 0 ? 0 : tile, bs = 1;
+        for (int t = 0; t < MG_NUM_TILES; t++) {
+            if (tile >= 0 && t != tile) continue;
+            const TileDesc &d = g_tiles[t];
+            const int64_t kblocks = cdiv(a.k, d.bk);
+            const int64_t groups = cdiv(a.m, d.bm) * cdiv(a.n, d.bn) * (int64_t)a.nbatch;
+            const int64_t slots = (int64_t)cus * wgs_per_cu(d, a.layout);
+            int cand[4] = {1, 0, 0, 0};
+            int nc = 1;
+            if (split > 0) {
+                cand[0] = split;
+            } else if (groups < slots && kblocks >= 8) {
+                int s = (int)(slots / groups);
+                if (s > kblocks / 4) s = (int)(kblocks / 4);
+                if (s > 1) cand[nc++] = s;
+                if (s > 3) cand[nc++] = s / 2;
+                if (2 * s <= kblocks / 4) cand[nc++] = 2 * s;
+            }
+            for (int c = 0; c < nc; c++) {
+                const int s = cand[c];
+                const int64_t kb_per = cdiv(kblocks, s);
+                if (!dma_eligible(a, d, kb_per * d.bk)) continue;
+                const double cost = plan_cost_us(a, d, s, cus);
+                if (cost < best) {
+                    best = cost;
+                    bt = t;
+                    bs = s;
+                }
+            }
+        }
+        tile = bt;
+        split = bs;
+    }
+    finish_plan(a, tile, split, pl);
 }
 
 static int check_args(const mg_gemm_args *a) {
@@ -356,7 +427,12 @@ int mg_tile_info(int id, mg_tile *out) {
     out->threads = t.wgm * t.wgn * 64;
     out->lds_bytes = lds_bytes_for(t, MG_NT);
     out->min_m = 1;
-    snprintf(out->name, sizeof(out->name), "mm_%dx%dx%d_w%dx%d", t.bm, t.bn, t.bk, t.wgm, t.wgn);
+    if (t.nstage > 0)
+        snprintf(out->name, sizeof(out->name), "mmd_%dx%dx%d_w%dx%d_s%d", t.bm, t.bn, t.bk, t.wgm, t.wgn, t.nstage);
+    else
+        snprintf(out->name, sizeof(out->name), "mm_%dx%dx%d_w%dx%d", t.bm, t.bn, t.bk, t.wgm, t.wgn);
+    out->stages = t.nstage;
+    out->fallback = t.fallback;
     return MG_OK;
 }
 
@@ -423,6 +499,7 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     }
     const int general = operands_aligned(a) ? 0 : 1;
     launch_fn fn = table_for(a.layout, a.dtype)[pl.tile][general];
+    if (!fn) return fail(MG_ERR_STATE, "mg_gemm: tile %d has no kernel for this alignment", pl.tile);
     dim3 grid((unsigned)(pl.grid_m * pl.grid_n), (unsigned)pl.split_k, (unsigned)a.nbatch);
     hipError_t e = fn(p, grid, ctx->stream);
     if (e != hipSuccess) return hip_fail(e, "mg_gemm: kernel launch");
@@ -502,6 +579,13 @@ int mg_graph_launch(mg_ctx *ctx, mg_graph *g, double *seconds) {
     HIP_TRY(hipStreamSynchronize(ctx->stream));
     auto t1 = std::chrono::steady_clock::now();
     if (seconds) *seconds = std::chrono::duration<double>(t1 - t0).count();
+    return MG_OK;
+}
+
+int mg_graph_enqueue(mg_ctx *ctx, mg_graph *g) {
+    if (!ctx || !g) return fail(MG_ERR_ARG, "mg_graph_enqueue: NULL argument");
+    if (ctx->capturing) return fail(MG_ERR_STATE, "mg_graph_enqueue: a graph is being recorded");
+    HIP_TRY(hipGraphLaunch(g->exec, ctx->stream));
     return MG_OK;
 }
 

@@ -1,17 +1,30 @@
 // The tile table: every block-tile configuration the library is built with.
-// X(id, BM, BN, BK, WGM, WGN) — WGM x WGN wavefronts of 64 lanes per workgroup.
 // The analogue of the reference's CONFIGS comprehension (kernels.py:326-331).
+//
+// Two kernel families share one id space:
+//   register-staged (gemm_kernel.h): any shape and alignment
+//     V(id, BM, BN, BK, WGM, WGN)
+//   direct-to-LDS   (gemm_dma_kernel.h): aligned operands, K % BK == 0
+//     D(id, BM, BN, BK, WGM, WGN, NSTAGE, fallback_id) — fallback_id names the
+//     register-staged tile of the same BM x BN used when the preconditions fail.
+// WGM x WGN wavefronts of 64 lanes per workgroup.
 #pragma once
 
-#define MG_TILE_LIST(X)      \
-    X(0, 256, 256, 64, 2, 2) \
-    X(1, 256, 128, 64, 2, 2) \
-    X(2, 128, 256, 64, 2, 2) \
-    X(3, 128, 128, 64, 2, 2) \
-    X(4, 64, 64, 64, 2, 2)   \
-    X(5, 64, 256, 64, 1, 4)  \
-    X(6, 32, 256, 64, 1, 4)  \
-    X(7, 256, 64, 64, 4, 1)  \
-    X(8, 256, 32, 64, 4, 1)
+#define MG_TILE_LIST(V, D)         \
+    V(0, 256, 256, 64, 2, 2)       \
+    V(1, 256, 128, 64, 2, 2)       \
+    V(2, 128, 256, 64, 2, 2)       \
+    V(3, 128, 128, 64, 2, 2)       \
+    V(4, 64, 64, 64, 2, 2)         \
+    V(5, 64, 256, 64, 1, 4)        \
+    V(6, 32, 256, 64, 1, 4)        \
+    V(7, 256, 64, 64, 4, 1)        \
+    V(8, 256, 32, 64, 4, 1)        \
+    D(9, 256, 256, 32, 2, 4, 4, 0) \
+    D(10, 256, 256, 64, 2, 4, 2, 0) \
+    D(11, 128, 128, 64, 2, 2, 2, 3) \
+    D(12, 128, 256, 32, 2, 2, 3, 2) \
+    D(13, 256, 128, 32, 2, 2, 3, 1) \
+    D(14, 128, 128, 32, 2, 2, 3, 3)
 
-#define MG_NUM_TILES 9
+#define MG_NUM_TILES 15

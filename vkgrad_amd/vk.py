@@ -142,6 +142,12 @@ class Graph:
         _check(self.dev._lib.mg_graph_launch(self.dev._ctx, self._handle, C.byref(dt)), f"{self.name}: submit")
         return dt.value
 
+    def enqueue(self):
+        """Replay without waiting; the stream keeps order with later work."""
+        if not self._finished:
+            raise VkError(f"{self.name}: call finish() before enqueue()")
+        _check(self.dev._lib.mg_graph_enqueue(self.dev._ctx, self._handle), f"{self.name}: enqueue")
+
     def destroy(self):
         if self._handle is not None:
             h, self._handle = self._handle, None
