@@ -182,6 +182,9 @@ int mg_ew_adamw(mg_ctx *ctx, float *w, const float *g, float *m, float *v, void 
 int mg_ew_zero(mg_ctx *ctx, float *dst, int64_t n);
 /* cast16 (kernels.py:857-860) */
 int mg_ew_cast16(mg_ctx *ctx, const float *src, void *dst, int64_t n, int dtype);
+/* Scratch operands for warm-up and tuning (kernels.py:367-375, 472-474 use uninitialised
+ * memory): n 16-bit values, pseudo-random in [-1, 1), reproducible from `seed`. */
+int mg_ew_fill_uniform16(mg_ctx *ctx, void *dst, int64_t n, uint32_t seed, int dtype);
 /* grad_add (dataparallel.py:54-58): dst[i] += src[i] */
 int mg_ew_grad_add(mg_ctx *ctx, float *dst, const float *src, int64_t n);
 

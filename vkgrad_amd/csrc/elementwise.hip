@@ -123,6 +123,22 @@ __global__ void k_grad_add(float *dst, const float *src, int64_t n) {
     if (i < n) dst[i] += src[i];
 }
 
+// Pseudo-random 16-bit operands in [-1, 1) from a counter hash: timing a GEMM on
+// zeros or on uninitialised memory misstates it (data toggling sets MFMA power,
+// and with it the clock), so the tuner and warm-up fill their scratch with this.
+__global__ void k_fill_uniform16(uint16_t *dst, int64_t n, uint32_t seed, int dtype) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint32_t x = (uint32_t)i * 0x9E3779B1u + seed;
+    x ^= x >> 16;
+    x *= 0x85EBCA6Bu;
+    x ^= x >> 13;
+    x *= 0xC2B2AE35u;
+    x ^= x >> 16;
+    const float v = (float)(x >> 8) * (2.0f / 16777216.0f) - 1.0f;
+    dst[i] = narrow16(v, dtype);
+}
+
 static inline unsigned blocks_for(int64_t n) { return (unsigned)((n + 255) / 256); }
 
 }  // namespace mg
@@ -193,6 +209,13 @@ int mg_ew_cast16(mg_ctx *ctx, const float *src, void *dst, int64_t n, int dtype)
     EW_PRECHECK("mg_ew_cast16", src && dst && count_ok(n) && dtype_ok(dtype));
     hipLaunchKernelGGL(k_cast16, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), src, (uint16_t *)dst, n, dtype);
     EW_POSTCHECK("mg_ew_cast16");
+}
+
+int mg_ew_fill_uniform16(mg_ctx *ctx, void *dst, int64_t n, uint32_t seed, int dtype) {
+    EW_PRECHECK("mg_ew_fill_uniform16", dst && count_ok(n) && dtype_ok(dtype));
+    hipLaunchKernelGGL(k_fill_uniform16, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), (uint16_t *)dst, n, seed,
+                       dtype);
+    EW_POSTCHECK("mg_ew_fill_uniform16");
 }
 
 int mg_ew_grad_add(mg_ctx *ctx, float *dst, const float *src, int64_t n) {

@@ -254,6 +254,9 @@ def warmup(dev, seconds=2.0, force=False):
     a = dev.buffer(m * k * 2, "device")
     b = dev.buffer(k * n * 2, "device")
     c = dev.buffer(m * n * 4, "device")
+    K = make_kernels(dev)
+    K["fill_uniform16"]([a], m * k, 3)
+    K["fill_uniform16"]([b], k * n, 4)
     mm = Matmul(dev)
     t0 = time.perf_counter()
     try:
@@ -330,10 +333,11 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
         warmup(dev)
         bufs = (dev.buffer(nb * m * k * 2, "device"), dev.buffer(nb * k * n * 2, "device"),
                 dev.buffer(nb * m * n * 4, "device"))
-        K = make_kernels(dev)
-        # finite operands: garbage bit patterns may be NaN/denormal and skew timing
-        K["zero"]([bufs[0]], nb * m * k // 2 or 1)
-        K["zero"]([bufs[1]], nb * k * n // 2 or 1)
+        K = make_kernels(dev, dtype)
+        # random operands: zeros or garbage bit patterns misstate the timing (data
+        # toggling sets MFMA power and with it the clock)
+        K["fill_uniform16"]([bufs[0]], nb * m * k, 1)
+        K["fill_uniform16"]([bufs[1]], nb * k * n, 2)
 
         def timer(mm, repeat):
             return mm(bufs[0], bufs[1], bufs[2], m, n, k, repeat=repeat, accumulate=accumulate, **call)
@@ -466,4 +470,6 @@ def make_kernels(dev, dtype="f16"):
     add("cast16", lambda lib, ctx, p, n: lib.mg_ew_cast16(ctx, p[0], p[1], n, dt))
     # dataparallel.py:54-58 — buffers: dst, src
     add("grad_add", lambda lib, ctx, p, n: lib.mg_ew_grad_add(ctx, p[0], p[1], n))
+    # buffers: dst (16-bit) ; args: seed — pseudo-random operands in [-1, 1) for warm-up and tuning
+    add("fill_uniform16", lambda lib, ctx, p, n, seed: lib.mg_ew_fill_uniform16(ctx, p[0], n, int(seed), dt))
     return K
