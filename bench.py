@@ -102,6 +102,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--eager", action="store_true", help="enqueue GEMMs one by one instead of replaying a graph")
+    ap.add_argument("--dense-head", action="store_true",
+                    help="row pitch of logits/dlogits = 50257 exactly (rows then start at odd addresses) instead of "
+                         "the next multiple of 64")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path has no multi-GPU part); run with --gpus 1")
@@ -129,20 +132,24 @@ def main():
             bufs[name] = dict(x=x, w=w, dy=dy, y=dev.buffer(ROWS * fout * 4, "device"),
                               dx=dev.buffer(ROWS * fin * 4, "device"), dw=dev.buffer(fout * fin * 4, "device"))
         sets.append(bufs)
+    # logits / dlogits: N = 50257 columns are computed and counted; their row pitch is padded
+    # to a multiple of 64 elements unless --dense-head, as any allocator of a (rows x vocab)
+    # tensor would (the reference pads the vocabulary itself, transformer.py:258)
+    vpitch = VOCAB if args.dense_head else (VOCAB + 63) // 64 * 64
     head = dict(x=dev.buffer(ROWS * D * 2, "device"), w=dev.buffer(VOCAB * D * 2, "device"),
-                dy=dev.buffer(ROWS * VOCAB * 2, "device"), y=dev.buffer(ROWS * VOCAB * 4, "device"),
+                dy=dev.buffer(ROWS * vpitch * 2, "device"), y=dev.buffer(ROWS * vpitch * 4, "device"),
                 dx=dev.buffer(ROWS * D * 4, "device"), dw=dev.buffer(VOCAB * D * 4, "device"))
     fill_bf16(dev, head["x"], ROWS * D, rng, 1.0)
     fill_bf16(dev, head["w"], VOCAB * D, rng, 0.02)
-    fill_bf16(dev, head["dy"], ROWS * VOCAB, rng, 1.0)
+    fill_bf16(dev, head["dy"], ROWS * vpitch, rng, 1.0)
 
     mms = {}
 
-    def mm_for(layout, m, n, k):
+    def mm_for(layout, m, n, k, **pitch):
         key = (layout, m, n, k)
         if key not in mms:
             ta, tb = LAYOUT_FLAGS[layout]
-            e = lookup_tuned(dev.name, m, n, k, ta, tb, DTYPE)
+            e = lookup_tuned(dev.name, m, n, k, ta, tb, DTYPE, **pitch)
             if e is not None:
                 mms[key] = Matmul(dev, trans_a=ta, trans_b=tb, dtype=DTYPE, tile=e["tile_id"],
                                   split_k=e.get("split_k", 0), group_m=e.get("group_m", 0))
@@ -150,12 +157,15 @@ def main():
                 mms[key] = Matmul(dev, trans_a=ta, trans_b=tb, dtype=DTYPE)
         return mms[key]
 
-    def linear_calls(b, fin, fout, rows=ROWS):
-        """The three GEMMs of one linear: (mm, a, b, c, m, n, k)."""
+    def linear_calls(b, fin, fout, rows=ROWS, ypitch=None):
+        """The three GEMMs of one linear: (mm, a, b, c, m, n, k, pitches).  ypitch is the
+        row pitch of the (rows x fout) tensors y and dy when it is not fout."""
+        yp = {} if ypitch is None else {"ldc": ypitch}
+        dp = {} if ypitch is None else {"lda": ypitch}
         return [
-            (mm_for("NT", rows, fout, fin), b["x"], b["w"], b["y"], rows, fout, fin),
-            (mm_for("NN", rows, fin, fout), b["dy"], b["w"], b["dx"], rows, fin, fout),
-            (mm_for("TN", fout, fin, rows), b["dy"], b["x"], b["dw"], fout, fin, rows),
+            (mm_for("NT", rows, fout, fin, **yp), b["x"], b["w"], b["y"], rows, fout, fin, yp),
+            (mm_for("NN", rows, fin, fout, **dp), b["dy"], b["w"], b["dx"], rows, fin, fout, dp),
+            (mm_for("TN", fout, fin, rows, **dp), b["dy"], b["x"], b["dw"], fout, fin, rows, dp),
         ]
 
     calls = []
@@ -163,17 +173,18 @@ def main():
         b = sets[layer % NSET]
         for name, fin, fout in LINEARS:
             calls += linear_calls(b[name], fin, fout)
-    calls += linear_calls(head, D, VOCAB)
-    step_flops = sum(2.0 * m * n * k for (_, _, _, _, m, n, k) in calls)
+    head_calls = linear_calls(head, D, VOCAB, ypitch=vpitch)
+    calls += head_calls
+    step_flops = sum(2.0 * c[4] * c[5] * c[6] for c in calls)
 
     if args.eager:
         def run_step():
-            for mm, a, b, c, m, n, k in calls:
-                mm.enqueue(a, b, c, m, n, k)
+            for mm, a, b, c, m, n, k, kw in calls:
+                mm.enqueue(a, b, c, m, n, k, **kw)
     else:
         graph = dev.graph("gpt2_small_gemms")
-        for mm, a, b, c, m, n, k in calls:
-            mm(a, b, c, m, n, k, graph=graph)
+        for mm, a, b, c, m, n, k, kw in calls:
+            mm(a, b, c, m, n, k, graph=graph, **kw)
         graph.finish()
 
         def run_step():
@@ -195,13 +206,17 @@ def main():
     per_shape = []
     for name, layout, m, n, k, count in gemm_list():
         mm = mm_for(layout, m, n, k)
-        b = head if name.startswith("head") else sets[0][name.split(".")[0]]
+        is_head = name.startswith("head")
+        b = head if is_head else sets[0][name.split(".")[0]]
         role = name.split(".")[1]
         a_, b_, c_ = {"fwd": (b["x"], b["w"], b["y"]), "dX": (b["dy"], b["w"], b["dx"]),
                       "dW": (b["dy"], b["x"], b["dw"])}[role]
-        t1 = mm(a_, b_, c_, m, n, k)
+        kw = {}
+        if is_head and vpitch != VOCAB:
+            kw = {"ldc": vpitch} if role == "fwd" else {"lda": vpitch}
+        t1 = mm(a_, b_, c_, m, n, k, **kw)
         rep = max(1, int(0.02 / max(t1, 1e-6)))
-        sec = min(mm(a_, b_, c_, m, n, k, repeat=rep) / rep for _ in range(3))
+        sec = min(mm(a_, b_, c_, m, n, k, repeat=rep, **kw) / rep for _ in range(3))
         fl = 2.0 * m * n * k
         by = 2.0 * (m * k + k * n) + 4.0 * m * n
         tile, split, gm = mm.plan(m, n, k)
@@ -222,7 +237,7 @@ def main():
         "vs_baseline": None, "dtype": DTYPE, "data": "synthetic",
         "config": {"workload": "GPT-2-small training GEMMs: d_model 768, 12 layers, 8192 token rows, "
                                "QKV/proj/MLP + tied head 50257, fwd+dX+dW, 147 GEMMs, 6.07 TFLOP per step",
-                   "rows": ROWS, "d_model": D, "layers": LAYERS, "vocab": VOCAB,
+                   "rows": ROWS, "d_model": D, "layers": LAYERS, "vocab": VOCAB, "logits_row_pitch": vpitch,
                    "launch": "eager" if args.eager else "hip-graph replay"},
         "frac_of_mfma_peak": round(tflops / PEAK_TFLOPS, 4),
         "sum_of_event_timed_gemms_ms": round(events_ms, 4),

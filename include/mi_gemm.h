@@ -70,7 +70,15 @@ typedef struct {
     int64_t sa, sb, sc;
     int32_t split_k;       /* 0 = picker decides, 1 = none, >1 = that many K slices */
     int32_t group_m;       /* 0 = picker decides; else row-blocks per rasterisation band */
+    int32_t flags;         /* MG_FLAG_* */
+    int32_t reserved;      /* must be 0 */
 } mg_gemm_args;
+
+/* The buffers of A and B end at their last element: row padding (ld beyond the stored
+ * columns) of the LAST row must not be read.  Without this flag, when an extent is not a
+ * multiple of 8 but the pitch covers it rounded up to 8, the fast kernels may read (never
+ * use) up to 14 bytes of the last row's padding, i.e. buffers must span rows * ld elements. */
+#define MG_FLAG_TIGHT_BUFFERS 1
 
 typedef struct {
     int32_t id;

@@ -90,6 +90,37 @@ def test_direct_to_lds_tiles_exact(dev):
                                         f"max diff {np.abs(got - ref).max()}")
 
 
+def test_direct_to_lds_ragged_k_and_edges_with_padded_pitch(dev):
+    """K not a multiple of BK (nor of 8) and ragged M/N, with row pitches padded to
+    a multiple of 8: the direct-to-LDS kernels stay eligible, multiply the K
+    remainder first through registers, and must never use what they read from
+    the padding (it holds NaN)."""
+    from vkgrad_amd.kernels import CONFIGS, Matmul
+    for m, n, k in [(264, 392, 150), (200, 136, 1001), (129, 257, 77)]:
+        for layout, (ta, tb) in LAYOUTS.items():
+            a_cols = m if ta else k
+            b_cols = k if tb else n
+            lda, ldb = (a_cols + 7) // 8 * 8 + 8, (b_cols + 7) // 8 * 8
+            for t in CONFIGS:
+                if not t["stages"]:
+                    continue
+                mm = Matmul(dev, trans_a=ta, trans_b=tb, tile=t["id"])
+                for split in (1, 2):
+                    r, got, ref = check_case(dev, m, n, k, ta, tb, "bf16", seed=21, tile=t["id"], integer=True,
+                                             bias=True, split_k=split, lda=lda, ldb=ldb)
+                    assert r["exact"], (f"{layout} {m}x{n}x{k} tile {t['name']} split {split}: "
+                                        f"max diff {np.abs(got - ref).max()}")
+
+
+def test_tight_buffers_fall_back(dev):
+    """Unpadded buffers whose extents are not multiples of 8 must not be served by
+    a kernel that reads row padding: same answer through the any-alignment path."""
+    from vkgrad_amd.kernels import CONFIGS
+    dma = next(t for t in CONFIGS if t["stages"])
+    r, got, ref = check_case(dev, 264, 392, 1001, False, True, "f16", seed=5, tile=dma["id"], integer=True)
+    assert r["exact"]
+
+
 def test_direct_to_lds_plan_is_used(dev):
     """The picker must keep a direct-to-LDS tile when its preconditions hold and
     fall back to the register-staged sibling when they do not."""
@@ -97,7 +128,8 @@ def test_direct_to_lds_plan_is_used(dev):
     dma = next(t for t in CONFIGS if t["stages"])
     mm = Matmul(dev, trans_b=True, tile=dma["id"])
     assert mm.plan(512, 512, 512)[0] == dma["id"]
-    assert mm.plan(512, 512, 500)[0] == dma["fallback"]      # K not a multiple of BK
+    assert mm.plan(512, 512, 504)[0] == dma["id"]            # ragged K, pitch still a multiple of 8
+    assert mm.plan(512, 512, 500)[0] == dma["fallback"]      # pitch 500 breaks 16-byte row alignment
 
 
 @pytest.mark.parametrize("layout", list(LAYOUTS))

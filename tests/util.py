@@ -14,10 +14,25 @@ def np16(dtype):
     return np.float16 if dtype == "f16" else np.uint16
 
 
+def pad_pitch(x, ld, fill):
+    """Copy of 2-D x with its rows spread to a pitch of ld elements (padding = fill)."""
+    out = np.full((x.shape[0], ld), fill, dtype=x.dtype)
+    out[:, :x.shape[1]] = x
+    return out
+
+
 def run_gemm(dev, a, b, m, n, k, trans_a=False, trans_b=False, dtype="f16", bias=None,
-             c_in=None, tile=None, split_k=0, group_m=0, kind="device", poison=True):
-    """a, b: stored operands (f16 arrays or bf16 bit patterns).  Returns C (m,n) f32."""
+             c_in=None, tile=None, split_k=0, group_m=0, kind="device", poison=True,
+             lda=None, ldb=None):
+    """a, b: stored operands (f16 arrays or bf16 bit patterns).  Returns C (m,n) f32.
+    lda/ldb: upload the operand with that row pitch; the padding holds NaN so that
+    anything read from it and used shows."""
     from vkgrad_amd.kernels import Matmul
+    nan16 = np.float16(np.nan) if dtype == "f16" else np.uint16(0x7FC0)
+    if lda is not None:
+        a = pad_pitch(a, lda, nan16)
+    if ldb is not None:
+        b = pad_pitch(b, ldb, nan16)
     ba = dev.buffer(max(a.nbytes, 2), kind)
     bb = dev.buffer(max(b.nbytes, 2), kind)
     bc = dev.buffer(m * n * 4, kind)
@@ -34,7 +49,7 @@ def run_gemm(dev, a, b, m, n, k, trans_a=False, trans_b=False, dtype="f16", bias
         if bias is not None:
             bbias = dev.buffer(n * 4, kind)
             bbias.upload(np.ascontiguousarray(bias, np.float32))
-        mm(ba, bb, bc, m, n, k, bias=bbias, accumulate=c_in is not None)
+        mm(ba, bb, bc, m, n, k, bias=bbias, accumulate=c_in is not None, lda=lda, ldb=ldb)
         return bc.download(np.float32, (m, n))
     finally:
         mm.destroy()
@@ -44,7 +59,7 @@ def run_gemm(dev, a, b, m, n, k, trans_a=False, trans_b=False, dtype="f16", bias
 
 
 def check_case(dev, m, n, k, trans_a=False, trans_b=False, dtype="f16", seed=0, bias=False,
-               accumulate=False, tile=None, split_k=0, integer=False, group_m=0):
+               accumulate=False, tile=None, split_k=0, integer=False, group_m=0, lda=None, ldb=None):
     """Run one seeded case and compare with the oracle.  Returns metrics dict."""
     a, b = O.make_operands(m, n, k, trans_a, trans_b, dtype, seed, integer=integer)
     rng = np.random.default_rng(seed + 1000)
@@ -55,7 +70,8 @@ def check_case(dev, m, n, k, trans_a=False, trans_b=False, dtype="f16", seed=0, 
         # per-column-distinct, non-zero biases: a skipped bias add must show
         bias_v = (rng.standard_normal(n) * 3 + np.arange(n) % 7 + 1).astype(np.float32) if bias else None
         c_in = rng.standard_normal((m, n)).astype(np.float32) * 5 if accumulate else None
-    got = run_gemm(dev, a, b, m, n, k, trans_a, trans_b, dtype, bias_v, c_in, tile, split_k, group_m)
+    got = run_gemm(dev, a, b, m, n, k, trans_a, trans_b, dtype, bias_v, c_in, tile, split_k, group_m,
+                   lda=lda, ldb=ldb)
     ref = O.ref_gemm(a, b, trans_a, trans_b, dtype, bias_v, c_in)
     out = dict(maxrel=O.err_maxrel(got, ref), fro=O.err_fro(got, ref),
                exact=bool(np.array_equal(got, ref)), finite=bool(np.isfinite(got).all()),

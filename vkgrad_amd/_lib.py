@@ -11,6 +11,7 @@ MG_NN, MG_NT, MG_TN = 0, 1, 2
 MG_F16, MG_BF16 = 0, 1
 MG_DEVICE, MG_SHARED, MG_CACHED, MG_BAR = 0, 1, 2, 3
 MG_ACT_NONE, MG_ACT_GELU, MG_ACT_RELU = 0, 1, 2
+MG_FLAG_TIGHT_BUFFERS = 1
 
 DTYPES = {"f16": MG_F16, "bf16": MG_BF16}
 KINDS = {"device": MG_DEVICE, "shared": MG_SHARED, "cached": MG_CACHED, "bar": MG_BAR}
@@ -28,6 +29,7 @@ class GemmArgs(C.Structure):
         ("nbatch", C.c_int32), ("tile", C.c_int32),
         ("sa", C.c_int64), ("sb", C.c_int64), ("sc", C.c_int64),
         ("split_k", C.c_int32), ("group_m", C.c_int32),
+        ("flags", C.c_int32), ("reserved", C.c_int32),
     ]
 
 

@@ -14,8 +14,13 @@
 //
 // Preconditions (checked by the host, which otherwise uses gemm_kernel.h):
 //   16-byte aligned operand bases, ld % 8 == 0, batch strides % 8 == 0,
-//   K % BK == 0 and the K slice a multiple of BK,
-//   for an M/N-contiguous operand its extent % 8 == 0 and >= 8.
+//   every K slice but the last a multiple of BK,
+//   ld >= round_up(K, 8) for a K-contiguous operand and ld >= round_up(extent, 8),
+//   extent >= 8 for an M/N-contiguous one, so that a 16-byte chunk that straddles
+//   the matrix edge still lies inside the row pitch (what it reads beyond the
+//   edge is masked: zeroed along K, unused along M/N).
+// K need not be a multiple of BK: the remainder (< BK) is staged through
+// registers with zero fill and multiplied first, before the ring starts.
 #pragma once
 #include "gemm_kernel.h"
 
@@ -59,7 +64,7 @@ struct DmaOp {
                 const int row = min(row0 + r, nrows - 1);
                 g[t] = base + (int64_t)row * ld + kbeg + lc * 8;
             } else {
-                const int col = min(row0 + lc * 8, nrows - 8);
+                const int col = min(row0 + lc * 8, ((nrows + 7) & ~7) - 8);
                 g[t] = base + (int64_t)(kbeg + r) * ld + col;
             }
         }
@@ -79,6 +84,43 @@ struct DmaOp {
             const uint32_t m0v = dst + q * 1024;
             asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0v), "v"(g[t]) : "memory", "m0");
             g[t] += kstep_elems;
+        }
+    }
+
+    // K remainder: fill this operand's LDS region with the block [k0, k0 + BK) of
+    // which only k < kend exists, through registers, zero beyond kend, in the same
+    // swizzled layout the direct loads produce.
+    template <int NTHREADS>
+    static __device__ __forceinline__ void fill_tail(char *region, const uint16_t *base, int64_t ld, int row0,
+                                                     int nrows, int k0, int kend, int tid) {
+        constexpr int NCHUNK = ROWS * BK / 8;
+        for (int c = tid; c < NCHUNK; c += NTHREADS) {
+            u32x4 v = {0u, 0u, 0u, 0u};
+            int off;
+            if constexpr (KC) {
+                const int r = c / CPR, kc = c % CPR;
+                const int k = k0 + kc * 8;
+                if (k < kend) {
+                    const int row = min(row0 + r, nrows - 1);
+                    v = *(const u32x4 *)(base + (int64_t)row * ld + k);
+                    const int nvalid = kend - k;   // elements of this chunk inside K
+#pragma unroll
+                    for (int w = 0; w < 4; w++) {
+                        const uint32_t keep = (2 * w + 1 < nvalid) ? 0xffffffffu : (2 * w < nvalid ? 0x0000ffffu : 0u);
+                        v[w] &= keep;
+                    }
+                }
+                off = r * ROW_BYTES + ((kc ^ swz(r)) * 16);
+            } else {
+                const int kr = c / CPR, rc = c % CPR;
+                const int k = k0 + kr;
+                if (k < kend) {
+                    const int col = min(row0 + rc * 8, ((nrows + 7) & ~7) - 8);
+                    v = *(const u32x4 *)(base + (int64_t)k * ld + col);
+                }
+                off = kr * ROW_BYTES + ((rc ^ swz(kr)) * 16);
+            }
+            *(u32x4 *)(region + off) = v;
         }
     }
 
@@ -157,13 +199,15 @@ gemm_dma_kernel(const GemmParams p) {
     float *C = p.C + zb * p.sc;
     const int kbeg = blockIdx.y * p.k_per_split;
     const int kend = min(p.K, kbeg + p.k_per_split);
-    const int nkb = (kend - kbeg) / BK;
+    const int krem = (kend - kbeg) % BK;          // K remainder, multiplied first
+    const int kdma = kbeg + krem;                 // the ring covers [kdma, kend)
+    const int nkb = (kend - kdma) / BK;
     const bool interior = (m0 + BM <= p.M) && (n0 + BN <= p.N);
 
     OA oa;
     OB ob;
-    oa.init(A, p.lda, m0, p.M, kbeg, wave, lane);
-    ob.init(B, p.ldb, n0, p.N, kbeg, wave, lane);
+    oa.init(A, p.lda, m0, p.M, kdma, wave, lane);
+    ob.init(B, p.ldb, n0, p.N, kdma, wave, lane);
     const int64_t a_step = A_KC ? BK : (int64_t)BK * p.lda;
     const int64_t b_step = B_KC ? BK : (int64_t)BK * p.ldb;
 
@@ -201,6 +245,19 @@ gemm_dma_kernel(const GemmParams p) {
         oa.issue(sp, a_step, wave);
         ob.issue(sp + OA::BYTES, b_step, wave);
     };
+
+    if (krem > 0) {
+        // [kbeg, kbeg + krem): through registers into stage 0, zero-filled to BK.
+        OA::template fill_tail<NW * 64>(dsm, A, p.lda, m0, p.M, kbeg, kbeg + krem, tid);
+        OB::template fill_tail<NW * 64>(dsm + OA::BYTES, B, p.ldb, n0, p.N, kbeg, kbeg + krem, tid);
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) {
+            read_frags(0, kk, 0);
+            mfma_group(0);
+        }
+        __syncthreads();   // all reads of stage 0 done before the ring overwrites it
+    }
 
     // Prologue: fill the ring (NSTAGE blocks, or all of them), publish block 0.
     const int npre = min(nkb, NSTAGE);
@@ -314,10 +371,329 @@ gemm_dma_kernel(const GemmParams p) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// Global memory access of the persistent kernel's epilogue, as inline assembly.
+// Any global load or store the compiler can see inside the K loop makes its
+// wait-count pass insert s_waitcnt vmcnt(..) where registers are reused (and
+// extra live ranges push the kernel into scratch spills, which are vector memory
+// operations themselves); vmcnt also counts the direct-to-LDS loads in flight,
+// so such waits would drain the ring once per tile.  The hardware reads a
+// store's address and data registers when the instruction issues, so stores need
+// no wait; loads are awaited explicitly.  Address = wave-uniform 64-bit base
+// (SGPR pair) + per-lane 32-bit byte offset: one offset register per lane serves
+// all stores of a tile.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void hidden_store(const char *sbase, uint32_t voff, float v) {
+    asm volatile("global_store_dword %0, %1, %2" ::"v"(voff), "v"(v), "s"(sbase) : "memory");
+}
+__device__ __forceinline__ void hidden_atomic_add(const char *sbase, uint32_t voff, float v) {
+    asm volatile("global_atomic_add_f32 %0, %1, %2" ::"v"(voff), "v"(v), "s"(sbase) : "memory");
+}
+__device__ __forceinline__ float hidden_load(const char *sbase, uint32_t voff) {
+    float v;
+    asm volatile("global_load_dword %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
+    return v;
+}
+// Wait for every outstanding vector memory operation; the operands tie the
+// loaded values to the wait so their uses cannot be scheduled above it.
+__device__ __forceinline__ void hidden_wait4(float &a, float &b, float &c, float &d) {
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : : "memory");
+}
+__device__ __forceinline__ void hidden_wait1(float &v) {
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(v) : : "memory");
+}
+
+// wait_dma_and_barrier with a run-time number of K-blocks (of L loads each) that
+// may stay in flight, 0 <= blocks <= MAXB.
+template <int L, int MAXB>
+__device__ __forceinline__ void wait_blocks_and_barrier(int blocks) {
+    static_assert(L * MAXB <= 63, "vmcnt immediate is 6 bits");
+    if constexpr (MAXB >= 3) {
+        if (blocks >= 3) { wait_dma_and_barrier<3 * L>(); return; }
+    }
+    if constexpr (MAXB >= 2) {
+        if (blocks == 2) { wait_dma_and_barrier<2 * L>(); return; }
+    }
+    if constexpr (MAXB >= 1) {
+        if (blocks == 1) { wait_dma_and_barrier<L>(); return; }
+    }
+    wait_dma_and_barrier<0>();
+}
+
+// ---------------------------------------------------------------------------
+// Persistent variant.  The grid holds at most as many workgroups as fit on the
+// chip at once; workgroup w processes work units w, w + gridDim.x, ... where a
+// unit is (K slice, output tile).  The K-blocks of all of a workgroup's units
+// form one flat sequence through the LDS ring, so the loads of the next unit's
+// first blocks are already in flight while the current unit finishes, and its
+// epilogue stores drain while the next unit's MFMAs run: no pipeline refill and
+// no exposed store phase between tiles.  Requires every K slice to be a multiple
+// of BK and BM * ldc * 4 < 2^32 (32-bit store offsets inside a tile).
+//
+// EPI_LOADS selects the epilogue: false = overwrite or atomic-add only; true =
+// also bias and C += (beta = 1), whose loads each drain vmcnt once.
+// ---------------------------------------------------------------------------
+template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool EPI_LOADS>
+__global__ void __launch_bounds__(WGM *WGN * 64)
+gemm_dmap_kernel(const GemmParams p) {
+    constexpr bool A_KC = (LAYOUT != L_TN);
+    constexpr bool B_KC = (LAYOUT == L_NT);
+    constexpr int NW = WGM * WGN;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int KK = BK / 16;
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0 && KK % 2 == 0 && NSTAGE >= 2, "tile shape");
+    using OA = DmaOp<A_KC, BM, BK, NW>;
+    using OB = DmaOp<B_KC, BN, BK, NW>;
+    constexpr int STAGE_BYTES = OA::BYTES + OB::BYTES;
+    constexpr int L = OA::PERW + OB::PERW;
+    constexpr int NDSR = TM * (A_KC ? 1 : 2) + TN * (B_KC ? 1 : 2);
+
+    extern __shared__ __attribute__((aligned(1024))) char dsm[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave / WGN, wave_n = wave % WGN;
+    const int64_t zb = blockIdx.z;
+    const uint16_t *A = p.A + zb * p.sa;
+    const uint16_t *B = p.B + zb * p.sb;
+    float *C = p.C + zb * p.sc;
+
+    // Work units of this workgroup: u = round * gridDim.x + pos, pos renumbered
+    // XCD-major so the workgroups behind one L2 hold neighbouring tiles.  Units
+    // are slice-major (all tiles of K slice 0, then slice 1, ...), so the slices
+    // of one tile are not adding into it at the same moment.
+    const int nwg = gridDim.x;
+    const int ntiles = p.grid_m * p.grid_n;
+    const int n_units = ntiles * p.split_k;
+    int pos = blockIdx.x;
+    if ((nwg & 7) == 0) pos = (pos & 7) * (nwg >> 3) + (pos >> 3);
+
+    struct Unit {
+        int m0, n0, kbeg, nkb;
+    };
+    auto unit_of = [&](int u) -> Unit {
+        const int slice = u / ntiles;
+        const int lin = u - slice * ntiles;
+        const int in_group = p.group_m * p.grid_n;
+        const int gid = lin / in_group;
+        const int first_m = gid * p.group_m;
+        const int gsize = min(p.grid_m - first_m, p.group_m);
+        const int r = lin - gid * in_group;
+        Unit q;
+        q.m0 = (first_m + r % gsize) * BM;
+        q.n0 = (r / gsize) * BN;
+        q.kbeg = slice * p.k_per_split;
+        q.nkb = (min(p.K, q.kbeg + p.k_per_split) - q.kbeg) / BK;
+        return q;
+    };
+
+    const int64_t a_step = A_KC ? BK : (int64_t)BK * p.lda;
+    const int64_t b_step = B_KC ? BK : (int64_t)BK * p.ldb;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t *)dsm;
+
+    // ---- load side ----
+    OA oa;
+    OB ob;
+    int l_u = pos;            // unit being loaded
+    int l_kb = 0, l_nkb = 0;  // next block of it, and its block count
+    int issued = 0;           // K-blocks issued so far (flat)
+    bool l_live = l_u < n_units;
+    auto issue_next = [&]() {
+        if (!l_live) return;
+        if (l_kb == 0) {
+            const Unit q = unit_of(l_u);
+            l_nkb = q.nkb;
+            oa.init(A, p.lda, q.m0, p.M, q.kbeg, wave, lane);
+            ob.init(B, p.ldb, q.n0, p.N, q.kbeg, wave, lane);
+        }
+        const uint32_t sp = lds_base + (issued % NSTAGE) * STAGE_BYTES;
+        oa.issue(sp, a_step, wave);
+        ob.issue(sp + OA::BYTES, b_step, wave);
+        issued++;
+        if (++l_kb == l_nkb) {
+            l_kb = 0;
+            l_u += nwg;
+            l_live = l_u < n_units;
+        }
+    };
+
+    // ---- compute side ----
+    f32x16 acc[TM][TN];
+    auto zero_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+    };
+    zero_acc();
+
+    int a_off[TM], b_off[TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++) a_off[i] = OA::frag_off(wave_m * WTM + i * 32, lane);
+#pragma unroll
+    for (int j = 0; j < TN; j++) b_off[j] = OA::BYTES + OB::frag_off(wave_n * WTN + j * 32, lane);
+
+    u32x4 af[2][TM], bf[2][TN];
+    auto read_frags = [&](int stage, int kk, int slot) {
+        const char *sp = dsm + stage * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < TM; i++) af[slot][i] = OA::frag(sp, a_off[i], kk, lane, wave_m * WTM + i * 32);
+#pragma unroll
+        for (int j = 0; j < TN; j++) bf[slot][j] = OB::frag(sp, b_off[j], kk, lane, wave_n * WTN + j * 32);
+    };
+    auto mfma_group = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) acc[i][j] = mfma32<DT>(af[slot][i], bf[slot][j], acc[i][j]);
+    };
+
+    // Per-lane byte offset of accumulator element (i=0, j=0, r=0) inside a tile.
+    const uint32_t c_voff =
+        (uint32_t)((((int64_t)(wave_m * WTM + (lane >> 5) * 4)) * p.ldc + wave_n * WTN + (lane & 31)) * 4);
+    auto epilogue = [&](const Unit &q) {
+        const bool interior = (q.m0 + BM <= p.M) && (q.n0 + BN <= p.N);
+        const bool add_bias = EPI_LOADS && p.bias != nullptr && q.kbeg == 0;
+        const int row_l = q.m0 + wave_m * WTM + (lane >> 5) * 4;
+        const int col_l = q.n0 + wave_n * WTN + (lane & 31);
+        const char *tile_base = (const char *)(C + (int64_t)q.m0 * p.ldc + q.n0);   // wave-uniform
+        const int64_t row_bytes = p.ldc * 4;
+        float bv[TN];
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            bv[j] = 0.f;
+            if constexpr (EPI_LOADS) {
+                if (add_bias) {   // uniform; out-of-range columns read a clamped, unused value
+                    const int cj = min(col_l + j * 32, p.N - 1);
+                    bv[j] = hidden_load((const char *)p.bias, (uint32_t)cj * 4u);
+                    hidden_wait1(bv[j]);
+                }
+            }
+        }
+        auto write_out = [&](auto mode_c, auto edge_c) {
+            constexpr int MODE = decltype(mode_c)::value;   // 0 overwrite, 1 C +=, 2 atomic +=
+            constexpr bool EDGE = decltype(edge_c)::value != 0;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int r4 = 0; r4 < 4; r4++) {
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        const bool col_ok = !EDGE || (col_l + j * 32 < p.N);
+                        float old[4] = {0.f, 0.f, 0.f, 0.f};
+                        if constexpr (MODE == 1) {
+#pragma unroll
+                            for (int e = 0; e < 4; e++) {
+                                const int ro = i * 32 + r4 * 8 + e;
+                                const bool ok = col_ok && (!EDGE || row_l + ro < p.M);
+                                if (ok) old[e] = hidden_load(tile_base + ro * row_bytes + j * 128, c_voff);
+                            }
+                            hidden_wait4(old[0], old[1], old[2], old[3]);
+                        }
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const int ro = i * 32 + r4 * 8 + e;
+                            const bool ok = col_ok && (!EDGE || row_l + ro < p.M);
+                            float v = acc[i][j][r4 * 4 + e];
+                            if constexpr (EPI_LOADS) v += bv[j];
+                            if constexpr (MODE == 1) v = old[e] + v;
+                            if (ok) {
+                                if constexpr (MODE == 2) hidden_atomic_add(tile_base + ro * row_bytes + j * 128, c_voff, v);
+                                else hidden_store(tile_base + ro * row_bytes + j * 128, c_voff, v);
+                            }
+                        }
+                    }
+                }
+            }
+        };
+        const int mode = p.split_k > 1 ? 2 : ((EPI_LOADS && p.beta) ? 1 : 0);
+        if (interior) {
+            if (mode == 0) write_out(IntC<0>{}, IntC<0>{});
+            else if (mode == 2) write_out(IntC<2>{}, IntC<0>{});
+            else if constexpr (EPI_LOADS) write_out(IntC<1>{}, IntC<0>{});
+        } else {
+            if (mode == 0) write_out(IntC<0>{}, IntC<1>{});
+            else if (mode == 2) write_out(IntC<2>{}, IntC<1>{});
+            else if constexpr (EPI_LOADS) write_out(IntC<1>{}, IntC<1>{});
+        }
+    };
+
+    if (!l_live) return;   // more workgroups than units
+
+    // Prologue: fill the ring, publish block 0.
+    for (int s = 0; s < NSTAGE; s++) issue_next();
+    wait_blocks_and_barrier<L, NSTAGE - 1>(issued - 1);
+    read_frags(0, 0, 0);
+
+    int c_u = pos;
+    Unit cq = unit_of(c_u);
+    int c_kb = 0;
+    int stage = 0;
+    // Invariant at the top of iteration ci: blocks ci .. issued-1 are issued,
+    // block ci is visible to all waves, its kk=0 fragments are in af[0], bf[0].
+    // Epilogue stores are younger than any load waited for below, so waiting on
+    // the load count alone can only over-wait, never under-wait.
+    for (int ci = 0; ci < issued; ci++) {
+        const int nstage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) {
+            const int cur = kk & 1, nxt = cur ^ 1;
+            if (kk < KK - 1) {
+                read_frags(stage, kk + 1, nxt);
+                mfma_group(cur);
+                interleave_group<TM * TN, NDSR, 0, 0>();
+            }
+            if (kk == KK - 2) {
+                // block ci+1 must have landed; blocks ci+2 .. issued-1 may stay in flight
+                const int ahead = issued - (ci + 2);
+                wait_blocks_and_barrier<L, NSTAGE - 2>(ahead < 0 ? 0 : (ahead > NSTAGE - 2 ? NSTAGE - 2 : ahead));
+                issue_next();   // into the stage block ci just vacated
+            }
+            if (kk == KK - 1) {
+                if (ci + 1 < issued) read_frags(nstage, 0, nxt);
+                mfma_group(cur);
+                interleave_group<TM * TN, NDSR, 0, 0>();
+            }
+        }
+        stage = nstage;
+        if (++c_kb == cq.nkb) {
+            epilogue(cq);
+            c_kb = 0;
+            c_u += nwg;
+            if (c_u < n_units) {
+                cq = unit_of(c_u);
+                zero_acc();
+            }
+        }
+    }
+}
+
 template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE>
 hipError_t launch_gemm_dma(const GemmParams &p, dim3 grid, hipStream_t stream) {
     using TT = DmaTraits<LAYOUT, BM, BN, BK, WGM, WGN, NSTAGE>;
     auto kern = gemm_dma_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, NSTAGE>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        if (TT::LDS_BYTES > 65536) {
+            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               TT::LDS_BYTES);
+            if (e != hipSuccess) return e;
+        }
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(TT::NTHREADS), TT::LDS_BYTES, stream, p);
+    return hipGetLastError();
+}
+
+// Persistent launcher: grid.x is the number of resident workgroups the host chose.
+template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool EPI_LOADS>
+hipError_t launch_gemm_dmap(const GemmParams &p, dim3 grid, hipStream_t stream) {
+    using TT = DmaTraits<LAYOUT, BM, BN, BK, WGM, WGN, NSTAGE>;
+    auto kern = gemm_dmap_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, NSTAGE, EPI_LOADS>;
     static bool attr_done = false;
     if (!attr_done) {
         if (TT::LDS_BYTES > 65536) {

@@ -100,13 +100,23 @@ struct Plan {
     int tile, split_k, group_m, k_per_split, grid_m, grid_n, xcd_remap;
 };
 
-// Preconditions of the direct-to-LDS kernels (gemm_dma_kernel.h).
-static bool dma_eligible(const mg_gemm_args &a, const TileDesc &t, int64_t k_per_split) {
+// Preconditions of the direct-to-LDS kernels (gemm_dma_kernel.h): aligned bases
+// and pitches, K slices that are multiples of BK (the last may be ragged), and
+// row pitches that cover the 16-byte chunk straddling a ragged edge.
+static bool dma_eligible(const mg_gemm_args &a, const TileDesc &t, int64_t k_per_split, int split) {
     if (t.nstage == 0) return true;
-    if (!operands_aligned(a)) return false;
-    if (a.k % t.bk != 0 || k_per_split % t.bk != 0) return false;
-    if (a.layout == MG_TN && a.m < 8) return false;
-    if (a.layout != MG_NT && a.n < 8) return false;
+    const bool a_kc = a.layout != MG_TN, b_kc = a.layout == MG_NT;
+    if (((uintptr_t)a.a | (uintptr_t)a.b) & 15) return false;
+    if ((a.lda | a.ldb) & 7) return false;
+    if (a.nbatch > 1 && ((a.sa | a.sb) & 7)) return false;
+    if (split > 1 && k_per_split % t.bk != 0) return false;
+    const int64_t k8 = (a.k + 7) & ~(int64_t)7, m8 = (a.m + 7) & ~(int64_t)7, n8 = (a.n + 7) & ~(int64_t)7;
+    if (a_kc ? a.lda < k8 : (a.lda < m8 || a.m < 8)) return false;
+    if (b_kc ? a.ldb < k8 : (a.ldb < n8 || a.n < 8)) return false;
+    // A chunk that straddles a ragged edge reads row padding; on the last row that is
+    // beyond the matrix, so the caller must own it (MG_FLAG_TIGHT_BUFFERS says it does not).
+    const bool ragged = (a_kc ? (a.k & 7) : (a.m & 7)) || (b_kc ? (a.k & 7) : (a.n & 7));
+    if (ragged && (a.flags & MG_FLAG_TIGHT_BUFFERS)) return false;
     return true;
 }
 
@@ -158,7 +168,7 @@ static void finish_plan(const mg_gemm_args &a, int tile, int split, Plan &pl) {
     if (split < 1) split = 1;
     int64_t kb_per = cdiv(kblocks, split);
     split = (int)cdiv(kblocks, kb_per);   // no empty slices
-    if (!dma_eligible(a, *d, kb_per * d->bk)) {
+    if (!dma_eligible(a, *d, kb_per * d->bk, split)) {
         tile = d->fallback;
         d = &g_tiles[tile];
         kblocks = cdiv(a.k, d->bk);
@@ -208,7 +218,7 @@ static void pick_plan(const mg_gemm_args &a, int cus, Plan &pl) {
             for (int c = 0; c < nc; c++) {
                 const int s = cand[c];
                 const int64_t kb_per = cdiv(kblocks, s);
-                if (!dma_eligible(a, d, kb_per * d.bk)) continue;
+                if (!dma_eligible(a, d, kb_per * d.bk, s)) continue;
                 const double cost = plan_cost_us(a, d, s, cus);
                 if (cost < best) {
                     best = cost;
@@ -254,6 +264,8 @@ static int check_args(const mg_gemm_args *a) {
     if (a->tile < -1 || a->tile >= MG_NUM_TILES) return fail(MG_ERR_ARG, "mg_gemm: unknown tile id %d", a->tile);
     if (a->split_k < 0 || a->split_k > 65535) return fail(MG_ERR_ARG, "mg_gemm: split_k %d out of range", a->split_k);
     if (a->group_m < 0) return fail(MG_ERR_ARG, "mg_gemm: group_m %d is negative", a->group_m);
+    if ((a->flags & ~MG_FLAG_TIGHT_BUFFERS) || a->reserved)
+        return fail(MG_ERR_ARG, "mg_gemm: unknown flags 0x%x", a->flags);
     return MG_OK;
 }
 
@@ -497,7 +509,9 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
         }
         HIP_TRY(hipGetLastError());
     }
-    const int general = operands_aligned(a) ? 0 : 1;
+    // direct-to-LDS tiles: eligibility was settled by the plan; register-staged
+    // tiles: the any-alignment instantiation unless every chunk is aligned and whole
+    const int general = t.nstage > 0 ? 0 : (operands_aligned(a) ? 0 : 1);
     launch_fn fn = table_for(a.layout, a.dtype)[pl.tile][general];
     if (!fn) return fail(MG_ERR_STATE, "mg_gemm: tile %d has no kernel for this alignment", pl.tile);
     dim3 grid((unsigned)(pl.grid_m * pl.grid_n), (unsigned)pl.split_k, (unsigned)a.nbatch);

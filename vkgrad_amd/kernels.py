@@ -126,6 +126,11 @@ class Matmul:
         need_a = ((nb - 1) * sa + (a_rows - 1) * ga.lda + a_cols) * esz
         need_b = ((nb - 1) * sb + (b_rows - 1) * ga.ldb + b_cols) * esz
         need_c = ((nb - 1) * sc + (m - 1) * ga.ldc + n) * 4
+        # the fast kernels may read (never use) the last row's padding up to the next
+        # multiple of 8 columns; tell the library when a buffer does not contain it
+        full_a = ((nb - 1) * sa + (a_rows - 1) * ga.lda + ((a_cols + 7) & ~7)) * esz
+        full_b = ((nb - 1) * sb + (b_rows - 1) * ga.ldb + ((b_cols + 7) & ~7)) * esz
+        ga.flags = L.MG_FLAG_TIGHT_BUFFERS if (full_a > a.size or full_b > b.size) else 0
         if m > 0 and n > 0 and k > 0:
             if need_a > a.size or need_b > b.size or need_c > c.size:
                 raise VkError(f"{self.name}: shape {m}x{n}x{k} (nbatch {nb}) needs {need_a}/{need_b}/{need_c} "
@@ -222,17 +227,25 @@ def _save_cache(cache, path=None):
     os.replace(tmp, path)
 
 
+def _pitch_tag(m, n, k, trans_a, trans_b, lda, ldb, ldc):
+    """Non-default row pitches as a key suffix (they decide which kernels are eligible)."""
+    d = (m if trans_a else k, k if trans_b else n, n)
+    got = tuple(int(x) if x is not None else dflt for x, dflt in zip((lda, ldb, ldc), d))
+    return "" if got == d else f"|ld{got[0]},{got[1]},{got[2]}"
+
+
 def tune_key(dev_name, m, n, k, trans_a, trans_b, dtype="f16", batched=False, nbatch=1,
-             accumulate=False):
-    """Cache key; the reference's shape (kernels.py:459-460) plus dtype and beta."""
+             accumulate=False, lda=None, ldb=None, ldc=None):
+    """Cache key; the reference's shape (kernels.py:459-460) plus dtype, beta and pitches."""
     return (f"{dev_name}|{m}x{n}x{k}|ta{int(trans_a)}tb{int(trans_b)}|{dtype}"
-            f"{'|acc' if accumulate else ''}{'|bat' + str(nbatch) if batched else ''}")
+            f"{'|acc' if accumulate else ''}{'|bat' + str(nbatch) if batched else ''}"
+            f"{_pitch_tag(m, n, k, trans_a, trans_b, lda, ldb, ldc)}")
 
 
 def lookup_tuned(dev_name, m, n, k, trans_a, trans_b, dtype="f16", batched=False, nbatch=1,
-                 accumulate=False):
+                 accumulate=False, lda=None, ldb=None, ldc=None):
     """Cached pick for a shape, user cache first, then the shipped table."""
-    key = tune_key(dev_name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate)
+    key = tune_key(dev_name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate, lda, ldb, ldc)
     for path in (_TUNE_CACHE, _SHIPPED_CACHE):
         e = _load_cache(path).get(key)
         if e is not None:
@@ -308,7 +321,7 @@ def candidate_space(m, n, k, cus=256, nbatch=1):
 
 def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=False,
                     use_cache=True, batched=False, nbatch=1, *, dtype="f16", accumulate=False,
-                    timer=None):
+                    timer=None, lda=None, ldb=None, ldc=None):
     """Pick the fastest (tile, split_k, group_m) for one shape (kernels.py:450-603).
 
     Stage one times every candidate round-robin over equal GPU time and keeps
@@ -318,29 +331,34 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
     Returns (Matmul, best) with best keys config, lds, tflops, ms, tile,
     evaluated, pruned, group_m, split_k, tile_id.
     """
-    key = tune_key(dev.name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate)
+    key = tune_key(dev.name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate, lda, ldb, ldc)
     if use_cache:
-        e = lookup_tuned(dev.name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate)
+        e = lookup_tuned(dev.name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate, lda, ldb, ldc)
         if e is not None:
             return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=e["tile_id"],
                           dtype=dtype, split_k=e.get("split_k", 0), group_m=e.get("group_m", 0)), e
 
     nb = nbatch if batched else 1
-    strides = (m * k, k * n, m * n)
+    pa = int(lda) if lda is not None else (m if trans_a else k)      # row pitches
+    pb = int(ldb) if ldb is not None else (k if trans_b else n)
+    pc = int(ldc) if ldc is not None else n
+    ea, eb, ec = (k if trans_a else m) * pa, (n if trans_b else k) * pb, m * pc   # elements per matrix
+    strides = (ea, eb, ec)
     call = dict(nbatch=nb, strides=strides) if batched else {}
     bufs = None
     if timer is None:
         warmup(dev)
-        bufs = (dev.buffer(nb * m * k * 2, "device"), dev.buffer(nb * k * n * 2, "device"),
-                dev.buffer(nb * m * n * 4, "device"))
+        bufs = (dev.buffer(nb * ea * 2, "device"), dev.buffer(nb * eb * 2, "device"),
+                dev.buffer(nb * ec * 4, "device"))
         K = make_kernels(dev, dtype)
         # random operands: zeros or garbage bit patterns misstate the timing (data
         # toggling sets MFMA power and with it the clock)
-        K["fill_uniform16"]([bufs[0]], nb * m * k, 1)
-        K["fill_uniform16"]([bufs[1]], nb * k * n, 2)
+        K["fill_uniform16"]([bufs[0]], nb * ea, 1)
+        K["fill_uniform16"]([bufs[1]], nb * eb, 2)
 
         def timer(mm, repeat):
-            return mm(bufs[0], bufs[1], bufs[2], m, n, k, repeat=repeat, accumulate=accumulate, **call)
+            return mm(bufs[0], bufs[1], bufs[2], m, n, k, repeat=repeat, accumulate=accumulate,
+                      lda=lda, ldb=ldb, ldc=ldc, **call)
 
     try:
         cands = [Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=t, dtype=dtype,
