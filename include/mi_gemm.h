@@ -88,7 +88,9 @@ typedef struct {
     int32_t lds_bytes;         /* for the NT layout; other layouts differ by padding */
     int32_t min_m;             /* informational: smallest M this tile is meant for */
     int32_t stages;            /* 0: register-staged kernel (any alignment); >0: direct-to-LDS ring depth */
-    int32_t fallback;          /* tile used instead when a direct-to-LDS tile's preconditions fail */
+    int32_t fallback;          /* tile used instead when this tile's preconditions fail (self: none) */
+    int32_t persistent;        /* 1: a grid of resident workgroups loops over the output tiles */
+    int32_t reserved;
     char name[48];
 } mg_tile;
 

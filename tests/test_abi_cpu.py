@@ -119,9 +119,15 @@ def test_tile_table(lib):
         assert t.bm % (32 * t.waves_m) == 0 and t.bn % (32 * t.waves_n) == 0
         assert t.lds_bytes <= 160 * 1024
         assert 0 <= t.fallback < n
-        fb = L.Tile()
-        lib.mg_tile_info(t.fallback, C.byref(fb))
-        assert fb.stages == 0 and (fb.bm, fb.bn) == (t.bm, t.bn)
+        # the fallback chain ends at a register-staged tile of the same BM x BN
+        fb, hops = t, 0
+        while fb.stages:
+            nxt = L.Tile()
+            lib.mg_tile_info(fb.fallback, C.byref(nxt))
+            assert (nxt.bm, nxt.bn) == (t.bm, t.bn) and nxt.id != fb.id
+            fb, hops = nxt, hops + 1
+            assert hops <= 3
+        assert fb.fallback == fb.id and not fb.persistent
         seen.add(t.name)
     assert len(seen) == n
     assert lib.mg_tile_info(n, C.byref(L.Tile())) == L.MG_ERR_ARG

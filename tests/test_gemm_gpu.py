@@ -116,7 +116,7 @@ def test_tight_buffers_fall_back(dev):
     """Unpadded buffers whose extents are not multiples of 8 must not be served by
     a kernel that reads row padding: same answer through the any-alignment path."""
     from vkgrad_amd.kernels import CONFIGS
-    dma = next(t for t in CONFIGS if t["stages"])
+    dma = next(t for t in CONFIGS if t["stages"] and not t["persistent"])
     r, got, ref = check_case(dev, 264, 392, 1001, False, True, "f16", seed=5, tile=dma["id"], integer=True)
     assert r["exact"]
 
@@ -125,11 +125,15 @@ def test_direct_to_lds_plan_is_used(dev):
     """The picker must keep a direct-to-LDS tile when its preconditions hold and
     fall back to the register-staged sibling when they do not."""
     from vkgrad_amd.kernels import CONFIGS, Matmul
-    dma = next(t for t in CONFIGS if t["stages"])
+    dma = next(t for t in CONFIGS if t["stages"] and not t["persistent"])
     mm = Matmul(dev, trans_b=True, tile=dma["id"])
     assert mm.plan(512, 512, 512)[0] == dma["id"]
     assert mm.plan(512, 512, 504)[0] == dma["id"]            # ragged K, pitch still a multiple of 8
     assert mm.plan(512, 512, 500)[0] == dma["fallback"]      # pitch 500 breaks 16-byte row alignment
+    per = next(t for t in CONFIGS if t["persistent"])
+    mp = Matmul(dev, trans_b=True, tile=per["id"])
+    assert mp.plan(512, 512, 512)[0] == per["id"]
+    assert mp.plan(512, 512, 504)[0] == per["fallback"]      # persistent tiles need whole K blocks
 
 
 @pytest.mark.parametrize("layout", list(LAYOUTS))

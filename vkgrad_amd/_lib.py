@@ -38,7 +38,7 @@ class Tile(C.Structure):
         ("id", C.c_int32), ("bm", C.c_int32), ("bn", C.c_int32), ("bk", C.c_int32),
         ("waves_m", C.c_int32), ("waves_n", C.c_int32), ("threads", C.c_int32),
         ("lds_bytes", C.c_int32), ("min_m", C.c_int32), ("stages", C.c_int32), ("fallback", C.c_int32),
-        ("name", C.c_char * 48),
+        ("persistent", C.c_int32), ("reserved", C.c_int32), ("name", C.c_char * 48),
     ]
 
 

@@ -379,28 +379,34 @@ gemm_dma_kernel(const GemmParams p) {
 // operations themselves); vmcnt also counts the direct-to-LDS loads in flight,
 // so such waits would drain the ring once per tile.  The hardware reads a
 // store's address and data registers when the instruction issues, so stores need
-// no wait; loads are awaited explicitly.  Address = wave-uniform 64-bit base
-// (SGPR pair) + per-lane 32-bit byte offset: one offset register per lane serves
-// all stores of a tile.
+// no wait.  Addresses are per-lane 64-bit VGPR pointers plus an immediate: an
+// SGPR base written by a scalar instruction just before would need wait states
+// the compiler does not insert for assembly it cannot see into.
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ void hidden_store(const char *sbase, uint32_t voff, float v) {
-    asm volatile("global_store_dword %0, %1, %2" ::"v"(voff), "v"(v), "s"(sbase) : "memory");
+template <int IMM>
+__device__ __forceinline__ void hidden_store(float *ptr, float v) {
+    asm volatile("global_store_dword %0, %1, off offset:%2" ::"v"(ptr), "v"(v), "n"(IMM) : "memory");
 }
-__device__ __forceinline__ void hidden_atomic_add(const char *sbase, uint32_t voff, float v) {
-    asm volatile("global_atomic_add_f32 %0, %1, %2" ::"v"(voff), "v"(v), "s"(sbase) : "memory");
+// C += v without reading C into registers: the L2 performs the add.  One writer
+// per element, so the result is the same single float add a load/add/store gives.
+template <int IMM>
+__device__ __forceinline__ void hidden_atomic_add(float *ptr, float v) {
+    asm volatile("global_atomic_add_f32 %0, %1, off offset:%2" ::"v"(ptr), "v"(v), "n"(IMM) : "memory");
 }
-__device__ __forceinline__ float hidden_load(const char *sbase, uint32_t voff) {
+// Load and wait in one statement: the compiler does not know the destination is
+// pending, so it must never get the chance to copy it before the wait.
+__device__ __forceinline__ float hidden_load_wait(const float *ptr) {
     float v;
-    asm volatile("global_load_dword %0, %1, %2" : "=v"(v) : "v"(voff), "s"(sbase) : "memory");
+    asm volatile("global_load_dword %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(ptr) : "memory");
     return v;
 }
-// Wait for every outstanding vector memory operation; the operands tie the
-// loaded values to the wait so their uses cannot be scheduled above it.
-__device__ __forceinline__ void hidden_wait4(float &a, float &b, float &c, float &d) {
-    asm volatile("s_waitcnt vmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : : "memory");
-}
-__device__ __forceinline__ void hidden_wait1(float &v) {
-    asm volatile("s_waitcnt vmcnt(0)" : "+v"(v) : : "memory");
+
+template <int J, int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (J < N) {
+        f(IntC<J>{});
+        static_for<J + 1, N>(f);
+    }
 }
 
 // wait_dma_and_barrier with a run-time number of K-blocks (of L loads each) that
@@ -428,10 +434,10 @@ __device__ __forceinline__ void wait_blocks_and_barrier(int blocks) {
 // first blocks are already in flight while the current unit finishes, and its
 // epilogue stores drain while the next unit's MFMAs run: no pipeline refill and
 // no exposed store phase between tiles.  Requires every K slice to be a multiple
-// of BK and BM * ldc * 4 < 2^32 (32-bit store offsets inside a tile).
+// of BK.
 //
-// EPI_LOADS selects the epilogue: false = overwrite or atomic-add only; true =
-// also bias and C += (beta = 1), whose loads each drain vmcnt once.
+// EPI_LOADS = true adds the bias epilogue (its loads drain vmcnt once per tile);
+// C += (beta = 1 or split-K) is an L2 atomic add and needs no load.
 // ---------------------------------------------------------------------------
 template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool EPI_LOADS>
 __global__ void __launch_bounds__(WGM *WGN * 64)
@@ -552,73 +558,54 @@ gemm_dmap_kernel(const GemmParams p) {
             for (int j = 0; j < TN; j++) acc[i][j] = mfma32<DT>(af[slot][i], bf[slot][j], acc[i][j]);
     };
 
-    // Per-lane byte offset of accumulator element (i=0, j=0, r=0) inside a tile.
-    const uint32_t c_voff =
-        (uint32_t)((((int64_t)(wave_m * WTM + (lane >> 5) * 4)) * p.ldc + wave_n * WTN + (lane & 31)) * 4);
+    // Epilogue of one unit.  The tile is walked row by row with one running
+    // per-lane pointer; the TN column blocks of a row are immediate offsets.
+    // beta = 1 and split-K both add into C with L2 atomics (no loads); the only
+    // loads are the TN bias values.
     auto epilogue = [&](const Unit &q) {
         const bool interior = (q.m0 + BM <= p.M) && (q.n0 + BN <= p.N);
         const bool add_bias = EPI_LOADS && p.bias != nullptr && q.kbeg == 0;
         const int row_l = q.m0 + wave_m * WTM + (lane >> 5) * 4;
         const int col_l = q.n0 + wave_n * WTN + (lane & 31);
-        const char *tile_base = (const char *)(C + (int64_t)q.m0 * p.ldc + q.n0);   // wave-uniform
-        const int64_t row_bytes = p.ldc * 4;
+        const int64_t ldc = p.ldc;
         float bv[TN];
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             bv[j] = 0.f;
             if constexpr (EPI_LOADS) {
-                if (add_bias) {   // uniform; out-of-range columns read a clamped, unused value
-                    const int cj = min(col_l + j * 32, p.N - 1);
-                    bv[j] = hidden_load((const char *)p.bias, (uint32_t)cj * 4u);
-                    hidden_wait1(bv[j]);
-                }
+                if (add_bias) bv[j] = hidden_load_wait(p.bias + min(col_l + j * 32, p.N - 1));
             }
         }
-        auto write_out = [&](auto mode_c, auto edge_c) {
-            constexpr int MODE = decltype(mode_c)::value;   // 0 overwrite, 1 C +=, 2 atomic +=
+        auto write_out = [&](auto atomic_c, auto edge_c) {
+            constexpr bool ATOMIC = decltype(atomic_c)::value != 0;
             constexpr bool EDGE = decltype(edge_c)::value != 0;
+            float *ptr = C + (int64_t)row_l * ldc + col_l;
 #pragma unroll
             for (int i = 0; i < TM; i++) {
 #pragma unroll
-                for (int r4 = 0; r4 < 4; r4++) {
-#pragma unroll
-                    for (int j = 0; j < TN; j++) {
-                        const bool col_ok = !EDGE || (col_l + j * 32 < p.N);
-                        float old[4] = {0.f, 0.f, 0.f, 0.f};
-                        if constexpr (MODE == 1) {
-#pragma unroll
-                            for (int e = 0; e < 4; e++) {
-                                const int ro = i * 32 + r4 * 8 + e;
-                                const bool ok = col_ok && (!EDGE || row_l + ro < p.M);
-                                if (ok) old[e] = hidden_load(tile_base + ro * row_bytes + j * 128, c_voff);
-                            }
-                            hidden_wait4(old[0], old[1], old[2], old[3]);
+                for (int r = 0; r < 16; r++) {
+                    const int ro = i * 32 + (r >> 2) * 8 + (r & 3);
+                    const bool row_ok = !EDGE || (row_l + ro < p.M);
+                    static_for<0, TN>([&](auto jc) {
+                        constexpr int j = decltype(jc)::value;
+                        float v = acc[i][j][r];
+                        if constexpr (EPI_LOADS) v += bv[j];
+                        if (row_ok && (!EDGE || col_l + j * 32 < p.N)) {
+                            if constexpr (ATOMIC) hidden_atomic_add<j * 128>(ptr, v);
+                            else hidden_store<j * 128>(ptr, v);
                         }
-#pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            const int ro = i * 32 + r4 * 8 + e;
-                            const bool ok = col_ok && (!EDGE || row_l + ro < p.M);
-                            float v = acc[i][j][r4 * 4 + e];
-                            if constexpr (EPI_LOADS) v += bv[j];
-                            if constexpr (MODE == 1) v = old[e] + v;
-                            if (ok) {
-                                if constexpr (MODE == 2) hidden_atomic_add(tile_base + ro * row_bytes + j * 128, c_voff, v);
-                                else hidden_store(tile_base + ro * row_bytes + j * 128, c_voff, v);
-                            }
-                        }
-                    }
+                    });
+                    ptr += ((r & 3) == 3) ? 5 * ldc : ldc;   // rows go 0,1,2,3, 8,9,10,11, 16, ...
                 }
             }
         };
-        const int mode = p.split_k > 1 ? 2 : ((EPI_LOADS && p.beta) ? 1 : 0);
+        const bool atomic = p.split_k > 1 || p.beta;
         if (interior) {
-            if (mode == 0) write_out(IntC<0>{}, IntC<0>{});
-            else if (mode == 2) write_out(IntC<2>{}, IntC<0>{});
-            else if constexpr (EPI_LOADS) write_out(IntC<1>{}, IntC<0>{});
+            if (atomic) write_out(IntC<1>{}, IntC<0>{});
+            else write_out(IntC<0>{}, IntC<0>{});
         } else {
-            if (mode == 0) write_out(IntC<0>{}, IntC<1>{});
-            else if (mode == 2) write_out(IntC<2>{}, IntC<1>{});
-            else if constexpr (EPI_LOADS) write_out(IntC<1>{}, IntC<1>{});
+            if (atomic) write_out(IntC<1>{}, IntC<1>{});
+            else write_out(IntC<0>{}, IntC<1>{});
         }
     };
 

@@ -34,13 +34,16 @@ __global__ void zero_c_kernel(float *C, int64_t ldc, int M, int N, int64_t sc) {
 struct TileDesc {
     int id, bm, bn, bk, wgm, wgn;
     int nstage;     // 0: register-staged kernel; >0: direct-to-LDS ring depth
-    int fallback;   // register-staged tile of the same BM x BN (self for those)
+    int fallback;   // tile of the same BM x BN with weaker preconditions (self: none)
+    int persistent; // 1: grid of resident workgroups looping over tiles
 };
-#define V(id, bm, bn, bk, wgm, wgn) {id, bm, bn, bk, wgm, wgn, 0, id},
-#define D(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb},
-static const TileDesc g_tiles[MG_NUM_TILES] = {MG_TILE_LIST(V, D)};
+#define V(id, bm, bn, bk, wgm, wgn) {id, bm, bn, bk, wgm, wgn, 0, id, 0},
+#define D(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 0},
+#define P(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 1},
+static const TileDesc g_tiles[MG_NUM_TILES] = {MG_TILE_LIST(V, D, P)};
 #undef V
 #undef D
+#undef P
 
 static thread_local char g_err[512] = "";
 
@@ -117,6 +120,9 @@ static bool dma_eligible(const mg_gemm_args &a, const TileDesc &t, int64_t k_per
     // beyond the matrix, so the caller must own it (MG_FLAG_TIGHT_BUFFERS says it does not).
     const bool ragged = (a_kc ? (a.k & 7) : (a.m & 7)) || (b_kc ? (a.k & 7) : (a.n & 7));
     if (ragged && (a.flags & MG_FLAG_TIGHT_BUFFERS)) return false;
+    if (t.persistent) {
+        if (a.k % t.bk != 0 || k_per_split % t.bk != 0) return false;
+    }
     return true;
 }
 
@@ -168,7 +174,7 @@ static void finish_plan(const mg_gemm_args &a, int tile, int split, Plan &pl) {
     if (split < 1) split = 1;
     int64_t kb_per = cdiv(kblocks, split);
     split = (int)cdiv(kblocks, kb_per);   // no empty slices
-    if (!dma_eligible(a, *d, kb_per * d->bk, split)) {
+    while (!dma_eligible(a, *d, kb_per * d->bk, split) && d->fallback != tile) {
         tile = d->fallback;
         d = &g_tiles[tile];
         kblocks = cdiv(a.k, d->bk);
@@ -439,12 +445,15 @@ int mg_tile_info(int id, mg_tile *out) {
     out->threads = t.wgm * t.wgn * 64;
     out->lds_bytes = lds_bytes_for(t, MG_NT);
     out->min_m = 1;
-    if (t.nstage > 0)
+    if (t.persistent)
+        snprintf(out->name, sizeof(out->name), "mmp_%dx%dx%d_w%dx%d_s%d", t.bm, t.bn, t.bk, t.wgm, t.wgn, t.nstage);
+    else if (t.nstage > 0)
         snprintf(out->name, sizeof(out->name), "mmd_%dx%dx%d_w%dx%d_s%d", t.bm, t.bn, t.bk, t.wgm, t.wgn, t.nstage);
     else
         snprintf(out->name, sizeof(out->name), "mm_%dx%dx%d_w%dx%d", t.bm, t.bn, t.bk, t.wgm, t.wgn);
     out->stages = t.nstage;
     out->fallback = t.fallback;
+    out->persistent = t.persistent;
     return MG_OK;
 }
 
@@ -511,10 +520,18 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     }
     // direct-to-LDS tiles: eligibility was settled by the plan; register-staged
     // tiles: the any-alignment instantiation unless every chunk is aligned and whole
-    const int general = t.nstage > 0 ? 0 : (operands_aligned(a) ? 0 : 1);
+    int general = t.nstage > 0 ? 0 : (operands_aligned(a) ? 0 : 1);
+    dim3 grid((unsigned)(pl.grid_m * pl.grid_n), (unsigned)pl.split_k, (unsigned)a.nbatch);
+    if (t.persistent) {
+        // resident workgroups loop over (slice, tile) units; [1] = epilogue with bias
+        general = a.bias != nullptr ? 1 : 0;
+        const int64_t units = (int64_t)pl.grid_m * pl.grid_n * pl.split_k;
+        const int64_t slots = (int64_t)ctx->prop.multiProcessorCount * wgs_per_cu(t, a.layout);
+        grid = dim3((unsigned)(units < slots ? units : slots), 1, (unsigned)a.nbatch);
+        p.xcd_remap = 0;
+    }
     launch_fn fn = table_for(a.layout, a.dtype)[pl.tile][general];
     if (!fn) return fail(MG_ERR_STATE, "mg_gemm: tile %d has no kernel for this alignment", pl.tile);
-    dim3 grid((unsigned)(pl.grid_m * pl.grid_n), (unsigned)pl.split_k, (unsigned)a.nbatch);
     hipError_t e = fn(p, grid, ctx->stream);
     if (e != hipSuccess) return hip_fail(e, "mg_gemm: kernel launch");
     return MG_OK;

@@ -4,13 +4,16 @@
 // Two kernel families share one id space:
 //   register-staged (gemm_kernel.h): any shape and alignment
 //     V(id, BM, BN, BK, WGM, WGN)
-//   direct-to-LDS   (gemm_dma_kernel.h): aligned operands, K % BK == 0
+//   direct-to-LDS   (gemm_dma_kernel.h): aligned operands and pitches
 //     D(id, BM, BN, BK, WGM, WGN, NSTAGE, fallback_id) — fallback_id names the
 //     register-staged tile of the same BM x BN used when the preconditions fail.
+//   persistent direct-to-LDS: additionally K slices that are multiples of BK
+//     P(id, BM, BN, BK, WGM, WGN, NSTAGE, fallback_id) — falls back to the
+//     one-tile-per-workgroup direct-to-LDS tile of the same shape.
 // WGM x WGN wavefronts of 64 lanes per workgroup.
 #pragma once
 
-#define MG_TILE_LIST(V, D)         \
+#define MG_TILE_LIST(V, D, P)      \
     V(0, 256, 256, 64, 2, 2)       \
     V(1, 256, 128, 64, 2, 2)       \
     V(2, 128, 256, 64, 2, 2)       \
@@ -25,6 +28,9 @@
     D(11, 128, 128, 64, 2, 2, 2, 3) \
     D(12, 128, 256, 32, 2, 2, 3, 2) \
     D(13, 256, 128, 32, 2, 2, 3, 1) \
-    D(14, 128, 128, 32, 2, 2, 3, 3)
+    D(14, 128, 128, 32, 2, 2, 3, 3) \
+    P(15, 256, 256, 64, 2, 4, 2, 10) \
+    P(16, 256, 256, 32, 2, 4, 4, 9) \
+    P(17, 128, 128, 64, 2, 2, 2, 11)
 
-#define MG_NUM_TILES 15
+#define MG_NUM_TILES 18

@@ -31,7 +31,7 @@ def _tiles():
         t = L.Tile()
         _check(lib.mg_tile_info(i, C.byref(t)), "tile table")
         out.append(dict(id=t.id, bm=t.bm, bn=t.bn, bk=t.bk, waves_m=t.waves_m, waves_n=t.waves_n,
-                        threads=t.threads, lds_bytes=t.lds_bytes, stages=t.stages, fallback=t.fallback,
+                        threads=t.threads, lds_bytes=t.lds_bytes, stages=t.stages, fallback=t.fallback, persistent=t.persistent,
                         name=t.name.decode()))
     return out
 
