@@ -46,6 +46,21 @@ def gemm_list():
 
 LAYOUT_FLAGS = {"NN": (False, False), "NT": (False, True), "TN": (True, False)}
 
+# HBM-side bytes per launch (L2 fetches + L2 write-backs) of each GEMM of the step,
+# measured on MI355X with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over
+# `bench.py --pmc-pass`, each counter scaled by what it reads for the cast kernel of
+# known size in the same pass (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).  A figure is
+# only valid for the (tile, split_k) it was measured with; for another plan the
+# bench line reports null.  gemm -> (tile, split_k, fetch bytes, write bytes)
+MEASURED_TRAFFIC = {
+    "qkv.fwd": (11, 1, 66.0e6, 75.5e6), "qkv.dX": (11, 1, 67.2e6, 25.2e6), "qkv.dW": (11, 4, 160.1e6, 28.3e6),
+    "proj.fwd": (11, 1, 22.2e6, 25.2e6), "proj.dX": (11, 1, 22.2e6, 25.2e6), "proj.dW": (17, 6, 39.3e6, 14.2e6),
+    "fc1.fwd": (11, 1, 75.2e6, 100.7e6), "fc1.dX": (11, 1, 96.1e6, 25.2e6), "fc1.dW": (17, 3, 100.6e6, 28.3e6),
+    "fc2.fwd": (11, 1, 88.7e6, 25.2e6), "fc2.dX": (11, 1, 75.1e6, 100.7e6), "fc2.dW": (17, 3, 93.4e6, 28.3e6),
+    "head.fwd": (15, 1, 1454.5e6, 1647.1e6), "head.dX": (0, 5, 1617.4e6, 133.7e6),
+    "head.dW": (10, 1, 1231.2e6, 154.4e6),
+}
+
 
 def fill_bf16(dev, buf, n, rng, scale):
     """Upload n bf16 values ~N(0, scale) in slabs (keeps host memory small)."""
@@ -105,6 +120,10 @@ def main():
     ap.add_argument("--dense-head", action="store_true",
                     help="row pitch of logits/dlogits = 50257 exactly (rows then start at odd addresses) instead of "
                          "the next multiple of 64")
+    ap.add_argument("--pmc-pass", action="store_true",
+                    help="for a counter run under rocprofv3 --pmc: 3 launches of a cast kernel of known size "
+                         "(calibration), then every distinct GEMM of the step twice, eagerly; prints the dispatch "
+                         "order instead of the benchmark line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path has no multi-GPU part); run with --gpus 1")
@@ -177,6 +196,33 @@ def main():
     calls += head_calls
     step_flops = sum(2.0 * c[4] * c[5] * c[6] for c in calls)
 
+    if args.pmc_pass:
+        from vkgrad_amd.kernels import make_kernels
+        K = make_kernels(dev, DTYPE)
+        ncal = 1 << 26
+        src, dst = dev.buffer(ncal * 4, "device"), dev.buffer(ncal * 2, "device")
+        K["zero"]([src], ncal)
+        order = []
+        for _ in range(3):
+            K["cast16"]([src, dst], ncal)
+            order.append({"kernel": "k_cast16", "fetch_bytes": ncal * 4, "write_bytes": ncal * 2})
+        seen = set()
+        for mm, a, b, c, m, n, k, kw in calls:
+            key = (id(mm), m, n, k)
+            if key in seen:
+                continue
+            seen.add(key)
+            tile, split, gm = mm.plan(m, n, k, **kw)
+            for _ in range(2):
+                mm(a, b, c, m, n, k, **kw)
+                order.append({"gemm": f"{'NT' if mm.trans_b else ('TN' if mm.trans_a else 'NN')} {m}x{n}x{k}",
+                              "tile": tile, "split_k": split, "zero_fill_launch_first": split > 1,
+                              "algorithmic_bytes": 2 * (m * k + k * n) + 4 * m * n})
+        dev.sync()
+        print(json.dumps({"dispatch_order": order}))
+        dev.destroy()
+        return
+
     if args.eager:
         def run_step():
             for mm, a, b, c, m, n, k, kw in calls:
@@ -219,15 +265,22 @@ def main():
         sec = min(mm(a_, b_, c_, m, n, k, repeat=rep, **kw) / rep for _ in range(3))
         fl = 2.0 * m * n * k
         by = 2.0 * (m * k + k * n) + 4.0 * m * n
-        tile, split, gm = mm.plan(m, n, k)
+        tile, split, gm = mm.plan(m, n, k, **kw)
         per_shape.append({"gemm": name, "layout": layout, "m": m, "n": n, "k": k, "count": count,
                           "us": round(sec * 1e6, 2), "tflops": round(fl / sec / 1e12, 1),
                           "frac_mfma": round(fl / sec / 1e12 / PEAK_TFLOPS, 4),
                           "gbps": round(by / sec / 1e9, 1), "tile": tile, "split_k": split})
     dom = max(per_shape, key=lambda r: r["us"] * r["count"])
+    mt = MEASURED_TRAFFIC.get(dom["gemm"])
+    traffic = None
+    if mt and (mt[0], mt[1]) == (dom["tile"], dom["split_k"]) and not args.dense_head:
+        traffic = mt[2] + mt[3]
     roofline = {"bound": "mfma", "kernel": f"gemm {dom['gemm']} {dom['layout']} {dom['m']}x{dom['n']}x{dom['k']}",
                 "achieved": dom["tflops"], "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(dom["tflops"] / PEAK_TFLOPS, 4), "traffic": None}
+                "frac": round(dom["tflops"] / PEAK_TFLOPS, 4), "traffic": traffic,
+                "traffic_unit": "bytes per launch (HBM side of L2: fetch + write-back)",
+                "algorithmic_bytes": int(2 * (dom["m"] * dom["k"] + dom["k"] * dom["n"]) + 4 * dom["m"] * dom["n"]),
+                "flops_per_launch": 2.0 * dom["m"] * dom["n"] * dom["k"]}
     events_ms = sum(r["us"] * r["count"] for r in per_shape) / 1e3
 
     out = {

@@ -166,6 +166,17 @@ def test_beta0_overwrites_nan(dev):
         _assert_close(r, f"TN poisoned split {split}")
 
 
+@pytest.mark.parametrize("tile", [3, 11, 17])
+def test_split_k_clear_respects_pitch_and_tails(dev, tile):
+    """beta=0 with a K split clears C first: with a padded row pitch (aligned and
+    not), an odd width, and a poisoned C, the result is exact and the padding
+    between rows keeps its contents."""
+    for n, ldc in [(320, 320), (317, 328), (317, 321), (5, 5), (1027, 1032)]:
+        r, got, ref = check_case(dev, 200, n, 1024, True, False, "f16", seed=n, integer=True, split_k=4,
+                                 tile=tile, ldc=ldc)
+        assert r["exact"], f"tile {tile} n {n} ldc {ldc}: max diff {np.abs(got - ref).max()}"
+
+
 def test_wrong_layout_fails(dev):
     """Negative control (idea: test_hf_gpt2.py:129-136): a square operand read
     with the wrong layout passes every shape check and must fail on values."""

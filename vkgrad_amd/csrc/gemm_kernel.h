@@ -354,25 +354,19 @@ gemm_kernel(const GemmParams p) {
 #pragma unroll
         for (int kk = 0; kk < KK; kk++) {
             const int cur = kk & 1, nxt = cur ^ 1;
-#ifndef EXP_NO_FRAG
             if (kk < KK - 1) {
                 read_frags(As, kk + 1, nxt);
             } else if (MODE == 1 || kb + 1 < nkb) {
                 read_frags(An, 0, nxt);   // next stage is complete: the barrier below has passed
             }
-#endif
             if (kk == KK - 2) {
-#ifndef EXP_NO_STORE
                 if (MODE == 1 || kb + 1 < nkb) {
                     sa.store(An, tid);
                     sb.store(An + SA::ELEMS, tid);
                 }
-#endif
                 if constexpr (MODE == 1) {
-#ifndef EXP_NO_GLOAD
                     sa.load_fast(a_tile(kb + 2), p.lda, tid);
                     sb.load_fast(b_tile(kb + 2), p.ldb, tid);
-#endif
                 } else {
                     if (kb + 2 < nkb) load_block(kb + 2);
                 }
@@ -382,23 +376,15 @@ gemm_kernel(const GemmParams p) {
                 if (kk == KK - 2) interleave_group<TM * TN, NDSR, NLOAD, NLOAD>();
                 else interleave_group<TM * TN, NDSR, 0, 0>();
             }
-#ifndef EXP_NO_BARRIER
             if (kk == KK - 2) __syncthreads();
-#endif
         }
     };
 
     int kb = 0;
-#ifdef EXP_NO_MAINLOOP
-    kb = nkb;
-#endif
     const int n_steady = nkb_fast - 2;   // iterations whose kb+2 prefetch is interior
     for (; kb < n_steady; kb++) kblock(IntC<1>{}, kb);
     for (; kb < nkb; kb++) kblock(IntC<0>{}, kb);
 
-#ifdef EXP_NO_EPILOGUE
-    if (p.M > 0) { if (acc[0][0][0] == 123.456f) C[0] = 1.f; return; }
-#endif
     // Epilogue.  Accumulator register r of lane l holds
     //   row (r/4)*8 + (l/32)*4 + r%4,  column l%32   of its 32x32 tile,
     // so one store instruction writes two full 128-byte row segments.  The mode

@@ -24,11 +24,20 @@ extern launch_fn launch_table_tn_bf16[MG_NUM_TILES][2];
 // Pre-pass for split-K with beta == 0: C = 0 (a fill kernel, so the sequence can
 // be captured in a graph).
 // ---------------------------------------------------------------------------
-__global__ void zero_c_kernel(float *C, int64_t ldc, int M, int N, int64_t sc) {
+// Rows are walked with a grid stride; a thread clears four consecutive columns,
+// as one 16-byte store when `vec` says every such group is aligned.
+__global__ void zero_c_kernel(float *C, int64_t ldc, int M, int N, int64_t sc, int vec) {
     float *Cz = C + (int64_t)blockIdx.z * sc;
-    const int col = blockIdx.x * blockDim.x + threadIdx.x;
-    const int row = blockIdx.y;
-    if (col < N && row < M) Cz[(int64_t)row * ldc + col] = 0.f;
+    const int col = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (col >= N) return;
+    for (int row = blockIdx.y; row < M; row += gridDim.y) {
+        float *q = Cz + (int64_t)row * ldc + col;
+        if (vec && col + 3 < N) {
+            *reinterpret_cast<float4 *>(q) = make_float4(0.f, 0.f, 0.f, 0.f);
+        } else {
+            for (int e = 0; e < 4 && col + e < N; e++) q[e] = 0.f;
+        }
+    }
 }
 
 struct TileDesc {
@@ -505,17 +514,18 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     if (lds_bytes_for(t, a.layout) > (int)ctx->prop.maxSharedMemoryPerMultiProcessor)
         return fail(MG_ERR_ARG, "mg_gemm: tile %d needs %d bytes of LDS", pl.tile, lds_bytes_for(t, a.layout));
     if (pl.split_k > 1 && a.beta == 0) {
-        dim3 zg((unsigned)cdiv(a.n, 256), (unsigned)a.m, (unsigned)a.nbatch);
-        if (a.m > 65535) {
-            // rows beyond the grid-y limit: fold into several launches
-            for (int64_t r0 = 0; r0 < a.m; r0 += 65535) {
-                const int rows = (int)((a.m - r0) < 65535 ? (a.m - r0) : 65535);
-                dim3 g2((unsigned)cdiv(a.n, 256), (unsigned)rows, (unsigned)a.nbatch);
-                hipLaunchKernelGGL(zero_c_kernel, g2, dim3(256), 0, ctx->stream, a.c + r0 * a.ldc, a.ldc, rows, (int)a.n, p.sc);
-            }
-        } else {
-            hipLaunchKernelGGL(zero_c_kernel, zg, dim3(256), 0, ctx->stream, a.c, a.ldc, (int)a.m, (int)a.n, p.sc);
-        }
+        // A dense C (pitch == N, batches back to back) is cleared as one long row.
+        const bool dense = a.ldc == a.n && (a.nbatch == 1 || p.sc == a.m * a.n) &&
+                           a.m * a.n * (int64_t)a.nbatch < 0x40000000LL;
+        const int zm = dense ? 1 : (int)a.m;
+        const int zn = dense ? (int)(a.m * a.n * a.nbatch) : (int)a.n;
+        const int zb = dense ? 1 : a.nbatch;
+        const int vec = (reinterpret_cast<uintptr_t>(a.c) % 16 == 0) && (dense || (a.ldc % 4 == 0 && p.sc % 4 == 0));
+        unsigned gx = (unsigned)cdiv(zn, 1024);
+        unsigned gy = (unsigned)(zm < 4096 ? zm : 4096);
+        if (gx > 65535u * 16u) return fail(MG_ERR_ARG, "mg_gemm: C too large for the split-K clear");
+        hipLaunchKernelGGL(zero_c_kernel, dim3(gx, gy, (unsigned)zb), dim3(256), 0, ctx->stream, a.c, a.ldc, zm, zn,
+                           p.sc, vec);
         HIP_TRY(hipGetLastError());
     }
     // direct-to-LDS tiles: eligibility was settled by the plan; register-staged

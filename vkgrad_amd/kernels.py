@@ -165,18 +165,18 @@ class Matmul:
         ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc)
         _check(self.dev._lib.mg_gemm(self.dev._ctx, C.byref(ga)), self.name)
 
-    def plan(self, m, n, k, nbatch=1):
+    def plan(self, m, n, k, nbatch=1, lda=None, ldb=None, ldc=None):
         """(tile id, split_k, group_m) the library would use for this shape."""
         ga = L.GemmArgs()
         ga.struct_size = C.sizeof(L.GemmArgs)
         ga.layout, ga.dtype = self.layout, L.DTYPES[self.dtype]
         ga.m, ga.n, ga.k = int(m), int(n), int(k)
         ga.a = ga.b = ga.c = 16     # placeholders: the picker never dereferences
-        ga.lda = m if self.trans_a else k
-        ga.ldb = k if self.trans_b else n
-        ga.ldc = n
+        ga.lda = int(lda) if lda is not None else (m if self.trans_a else k)
+        ga.ldb = int(ldb) if ldb is not None else (k if self.trans_b else n)
+        ga.ldc = int(ldc) if ldc is not None else n
         ga.nbatch, ga.tile = (int(nbatch) if self.batched else 1), self.tile
-        ga.sc = m * n
+        ga.sc = m * ga.ldc
         ga.split_k, ga.group_m = self.split_k, self.group_m
         t, s, g = C.c_int(), C.c_int(), C.c_int()
         _check(self.dev._lib.mg_pick(C.byref(ga), self.dev.compute_units, C.byref(t), C.byref(s), C.byref(g)),
@@ -309,9 +309,11 @@ def candidate_space(m, n, k, cus=256, nbatch=1):
         if groups < cus and kblocks >= 4:
             for target in (cus, 2 * cus):
                 s = max(1, min(target // groups, kblocks // 2))
-                splits.add(s)
-                if s > 2:
-                    splits.add(s // 2)
+                # the neighbours too: atomic traffic grows with the split, so the
+                # fastest one is often just below what fills the chip
+                for c in (s - 1, s, s + 1, s // 2):
+                    if 1 <= c <= kblocks // 2:
+                        splits.add(c)
         for s in sorted(splits):
             out.append((t["id"], s))
     if not out:
