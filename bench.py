@@ -171,7 +171,8 @@ def main():
             e = lookup_tuned(dev.name, m, n, k, ta, tb, DTYPE, **pitch)
             if e is not None:
                 mms[key] = Matmul(dev, trans_a=ta, trans_b=tb, dtype=DTYPE, tile=e["tile_id"],
-                                  split_k=e.get("split_k", 0), group_m=e.get("group_m", 0))
+                                  split_k=e.get("split_k", 0), group_m=e.get("group_m", 0),
+                                  atomic_split=e.get("atomic_split", False))
             else:
                 mms[key] = Matmul(dev, trans_a=ta, trans_b=tb, dtype=DTYPE)
         return mms[key]

@@ -79,6 +79,12 @@ typedef struct {
  * multiple of 8 but the pitch covers it rounded up to 8, the fast kernels may read (never
  * use) up to 14 bytes of the last row's padding, i.e. buffers must span rows * ld elements. */
 #define MG_FLAG_TIGHT_BUFFERS 1
+/* With a K split (split_k > 1, or chosen by the picker) the slices normally meet in the
+ * context's workspace and are summed in slice order by the slice that finishes last: no
+ * clear of C, bit-reproducible.  This flag makes them add into C with float atomics instead
+ * (after a clear kernel when beta == 0), which is also what happens when the partial tiles
+ * do not fit the workspace; it can be faster when C is large and the split is deep. */
+#define MG_FLAG_SPLITK_ATOMIC 2
 
 typedef struct {
     int32_t id;

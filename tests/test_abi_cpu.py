@@ -212,7 +212,7 @@ def test_autotuner_logic_with_fake_timer(tmp_path, monkeypatch):
     fast_tile = K.CONFIGS[3]["id"]
 
     def timer(mm, repeat):
-        calls.append((mm.tile, mm.split_k, mm.group_m, repeat))
+        calls.append((mm.tile, mm.split_k, mm.group_m, repeat, mm.atomic_split))
         per = 1e-4 if mm.tile == fast_tile else 5e-4
         if mm.group_m == 4:
             per *= 0.9
@@ -228,7 +228,7 @@ def test_autotuner_logic_with_fake_timer(tmp_path, monkeypatch):
     reps_slow = {c[3] for c in stage1 if c[0] != fast_tile}
     assert reps_fast and reps_slow and min(reps_fast) == 5 * max(reps_slow)
     # round-robin: no candidate is measured twice in a row within stage one
-    timed = [c[:2] for c in stage1]
+    timed = [(c[0], c[1], c[4]) for c in stage1]   # a K split is a candidate twice: workspace and atomic
     ncand = len(set(timed))
     assert ncand > 1 and len(timed) == 3 * ncand
     assert timed[:ncand] == timed[ncand:2 * ncand] == timed[2 * ncand:]

@@ -177,6 +177,37 @@ def test_split_k_clear_respects_pitch_and_tails(dev, tile):
         assert r["exact"], f"tile {tile} n {n} ldc {ldc}: max diff {np.abs(got - ref).max()}"
 
 
+@pytest.mark.parametrize("tile", [0, 10, 15, 17])
+def test_split_k_is_bit_reproducible(dev, tile):
+    """The K slices meet in a workspace and are summed in slice order by whichever
+    slice arrives last, so random data gives the same bits on every run."""
+    outs = []
+    for _ in range(3):
+        r, got, _ = check_case(dev, 512, 512, 4096, True, False, "bf16", seed=77, split_k=8, tile=tile, bias=True,
+                               accumulate=True)
+        _assert_close(r, f"tile {tile}")
+        outs.append(got)
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
+def test_split_k_without_workspace_adds_atomically(monkeypatch):
+    """With the workspace switched off the slices add into C with atomics (after a
+    clear when beta = 0): exact on integers, within tolerance on random data."""
+    from vkgrad_amd.vk import Device
+    monkeypatch.setenv("MIGEMM_SPLITK_WORKSPACE_MB", "0")
+    d = Device()
+    try:
+        for tile in (3, 11, 17):
+            r, got, ref = check_case(d, 200, 317, 1024, True, False, "f16", seed=3, integer=True, split_k=4,
+                                     tile=tile, ldc=328)
+            assert r["exact"], f"tile {tile}: max diff {np.abs(got - ref).max()}"
+            r, _, _ = check_case(d, 192, 320, 2048, False, True, "bf16", seed=6, split_k=3, tile=tile, bias=True,
+                                 accumulate=True)
+            _assert_close(r, f"tile {tile}")
+    finally:
+        d.destroy()
+
+
 def test_wrong_layout_fails(dev):
     """Negative control (idea: test_hf_gpt2.py:129-136): a square operand read
     with the wrong layout passes every shape check and must fail on values."""

@@ -12,6 +12,7 @@ MG_F16, MG_BF16 = 0, 1
 MG_DEVICE, MG_SHARED, MG_CACHED, MG_BAR = 0, 1, 2, 3
 MG_ACT_NONE, MG_ACT_GELU, MG_ACT_RELU = 0, 1, 2
 MG_FLAG_TIGHT_BUFFERS = 1
+MG_FLAG_SPLITK_ATOMIC = 2
 
 DTYPES = {"f16": MG_F16, "bf16": MG_BF16}
 KINDS = {"device": MG_DEVICE, "shared": MG_SHARED, "cached": MG_CACHED, "bar": MG_BAR}

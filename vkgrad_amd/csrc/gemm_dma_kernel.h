@@ -297,7 +297,17 @@ gemm_dma_kernel(const GemmParams p) {
     }
 
     // Epilogue: identical to gemm_kernel.h.
-    const bool add_bias = p.bias != nullptr && blockIdx.y == 0;
+    bool add_bias = p.bias != nullptr && blockIdx.y == 0;
+    int mode = p.split_k > 1 ? 2 : (p.beta ? 1 : 0);
+    if (p.split_k > 1 && p.ws != nullptr) {
+        __syncthreads();   // every wave is done with the ring: its first word serves as the flag
+        if (!splitk_gather<TM, TN, NW * 64>(acc, p.ws, p.cnt, (int64_t)blockIdx.z * gridDim.x + blockIdx.x,
+                                             (int64_t)gridDim.x * gridDim.z, blockIdx.y, gridDim.y, tid,
+                                             reinterpret_cast<int *>(dsm)))
+            return;
+        add_bias = p.bias != nullptr;
+        mode = p.beta ? 1 : 0;
+    }
     const int row_l = m0 + wave_m * WTM + (lane >> 5) * 4;
     const int col_l = n0 + wave_n * WTN + (lane & 31);
     float *cl = C + (int64_t)row_l * p.ldc + col_l;
@@ -340,7 +350,6 @@ gemm_dma_kernel(const GemmParams p) {
             }
         }
     };
-    const int mode = p.split_k > 1 ? 2 : (p.beta ? 1 : 0);
     if (interior) {
         if (mode == 0) write_out(IntC<0>{}, IntC<0>{});
         else if (mode == 1) write_out(IntC<1>{}, IntC<0>{});
@@ -437,6 +446,7 @@ gemm_dmap_kernel(const GemmParams p) {
     constexpr int NDSR = TM * (A_KC ? 1 : 2) + TN * (B_KC ? 1 : 2);
 
     extern __shared__ __attribute__((aligned(1024))) char dsm[];
+    __shared__ int gather_flag;   // the ring always holds prefetched blocks, so the flag lives beside it
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -458,7 +468,7 @@ gemm_dmap_kernel(const GemmParams p) {
     if ((nwg & 7) == 0) pos = (pos & 7) * (nwg >> 3) + (pos >> 3);
 
     struct Unit {
-        int m0, n0, kbeg, nkb;
+        int m0, n0, kbeg, nkb, lin, slice;
     };
     auto unit_of = [&](int u) -> Unit {
         const int slice = u / ntiles;
@@ -471,6 +481,8 @@ gemm_dmap_kernel(const GemmParams p) {
         Unit q;
         q.m0 = (first_m + r % gsize) * BM;
         q.n0 = (r / gsize) * BN;
+        q.lin = lin;
+        q.slice = slice;
         q.kbeg = slice * p.k_per_split;
         q.nkb = (min(p.K, q.kbeg + p.k_per_split) - q.kbeg) / BK;
         return q;
@@ -545,7 +557,15 @@ gemm_dmap_kernel(const GemmParams p) {
     // loads are the TN bias values.
     auto epilogue = [&](const Unit &q) {
         const bool interior = (q.m0 + BM <= p.M) && (q.n0 + BN <= p.N);
-        const bool add_bias = EPI_LOADS && p.bias != nullptr && q.kbeg == 0;
+        bool add_bias = EPI_LOADS && p.bias != nullptr && q.kbeg == 0;
+        bool atomic = p.split_k > 1 || p.beta;
+        if (p.split_k > 1 && p.ws != nullptr) {
+            if (!splitk_gather<TM, TN, NW * 64>(acc, p.ws, p.cnt, zb * ntiles + q.lin, (int64_t)ntiles * gridDim.z,
+                                                 q.slice, p.split_k, tid, &gather_flag))
+                return;
+            add_bias = EPI_LOADS && p.bias != nullptr;
+            atomic = p.beta != 0;
+        }
         const int row_l = q.m0 + wave_m * WTM + (lane >> 5) * 4;
         const int col_l = q.n0 + wave_n * WTN + (lane & 31);
         const int64_t ldc = p.ldc;
@@ -580,7 +600,6 @@ gemm_dmap_kernel(const GemmParams p) {
                 }
             }
         };
-        const bool atomic = p.split_k > 1 || p.beta;
         if (interior) {
             if (atomic) write_out(IntC<1>{}, IntC<0>{});
             else write_out(IntC<0>{}, IntC<0>{});

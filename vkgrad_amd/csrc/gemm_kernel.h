@@ -49,6 +49,8 @@ struct GemmParams {
     int split_k;          // number of K slices (gridDim.y)
     int k_per_split;      // K elements per slice, a multiple of BK
     int xcd_remap;        // 1: renumber workgroups so neighbours share an XCD
+    float *ws;            // split-K workspace (split_k * tiles * BM * BN floats) or null: add with atomics
+    int *cnt;             // one arrival counter per tile, zero between launches
 };
 
 template <int DT>
@@ -226,6 +228,69 @@ struct IntC {
     static constexpr int value = N;
 };
 
+// ---------------------------------------------------------------------------
+// Split-K through a workspace.  Every K slice of a tile stores its partial
+// accumulators, then counts itself in; the slice that arrives last sums all the
+// partials in slice order and goes on to write the tile.  Nobody waits for
+// anybody, the sum order is fixed (so results are bit-reproducible from run to
+// run), C needs no clearing beforehand, and bias and beta are applied once, by
+// the writer.
+//
+// Visibility between workgroups (which may sit behind different L2s) comes from
+// device-scope accesses: the partials are written and read with relaxed
+// device-scope atomics, which go through to the coherence point and never leave
+// a stale or dirty line in a private cache, and a slice counts itself in only
+// after its stores have completed (vmcnt 0).  That avoids device-scope fences,
+// which write back and invalidate a whole L2 under the workgroups still
+// streaming their operands through it.
+//
+// Returns true in the workgroup that has to write the tile; its acc then holds
+// the complete sum.  `flag` points at one int of LDS nobody else is using.
+// ---------------------------------------------------------------------------
+template <int TM, int TN, int NTHREADS>
+__device__ __forceinline__ bool splitk_gather(f32x16 (&acc)[TM][TN], float *ws, int *cnt, int64_t tile, int64_t ntiles,
+                                              int slice, int nslices, int tid, int *flag) {
+    constexpr int64_t TILE_FLOATS = (int64_t)TM * TN * 16 * NTHREADS;
+    float *mine = ws + ((int64_t)slice * ntiles + tile) * TILE_FLOATS + tid;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                __hip_atomic_store(mine + (int64_t)((i * TN + j) * 16 + r) * NTHREADS, acc[i][j][r], __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this lane's partials have reached the coherence point
+    __syncthreads();
+    if (tid == 0) {
+        const int old = __hip_atomic_fetch_add(cnt + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag = (old == nslices - 1);
+    }
+    __syncthreads();
+    const bool last = *flag != 0;
+    __syncthreads();      // flag may be reused (persistent kernel) once everyone has read it
+    if (!last) return false;
+    if (tid == 0) cnt[tile] = 0;   // ready for the next launch
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+    for (int sl = 0; sl < nslices; sl++) {
+        const float *src = ws + ((int64_t)sl * ntiles + tile) * TILE_FLOATS + tid;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    acc[i][j][r] += __hip_atomic_load(src + (int64_t)((i * TN + j) * 16 + r) * NTHREADS,
+                                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return true;
+}
+
 // Pin the instruction mix of one MFMA group for the backend scheduler: the
 // group's LDS reads, LDS writes and global loads are spread evenly between its
 // MFMAs instead of being issued in a burst in front of them.
@@ -390,7 +455,17 @@ gemm_kernel(const GemmParams p) {
     // so one store instruction writes two full 128-byte row segments.  The mode
     // (overwrite / read-add / atomic-add) and the edge test are uniform over the
     // workgroup and hoisted out of the element loops.
-    const bool add_bias = p.bias != nullptr && blockIdx.y == 0;
+    bool add_bias = p.bias != nullptr && blockIdx.y == 0;
+    int mode = p.split_k > 1 ? 2 : (p.beta ? 1 : 0);
+    if (p.split_k > 1 && p.ws != nullptr) {
+        __syncthreads();   // every wave is done with the LDS stages: smem[0..1] serves as the flag
+        if (!splitk_gather<TM, TN, WGM * WGN * 64>(acc, p.ws, p.cnt, (int64_t)blockIdx.z * gridDim.x + blockIdx.x,
+                                                    (int64_t)gridDim.x * gridDim.z, blockIdx.y, gridDim.y, tid,
+                                                    reinterpret_cast<int *>(smem)))
+            return;
+        add_bias = p.bias != nullptr;
+        mode = p.beta ? 1 : 0;
+    }
     const int row_l = m0 + wave_m * WTM + (lane >> 5) * 4;
     const int col_l = n0 + wave_n * WTN + (lane & 31);
     float *cl = C + (int64_t)row_l * p.ldc + col_l;
@@ -433,7 +508,6 @@ gemm_kernel(const GemmParams p) {
             }
         }
     };
-    const int mode = p.split_k > 1 ? 2 : (p.beta ? 1 : 0);
     if (interior) {
         if (mode == 0) write_out(IntC<0>{}, IntC<0>{});
         else if (mode == 1) write_out(IntC<1>{}, IntC<0>{});

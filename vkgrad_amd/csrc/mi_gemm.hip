@@ -5,6 +5,7 @@
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 
@@ -279,7 +280,7 @@ static int check_args(const mg_gemm_args *a) {
     if (a->tile < -1 || a->tile >= MG_NUM_TILES) return fail(MG_ERR_ARG, "mg_gemm: unknown tile id %d", a->tile);
     if (a->split_k < 0 || a->split_k > 65535) return fail(MG_ERR_ARG, "mg_gemm: split_k %d out of range", a->split_k);
     if (a->group_m < 0) return fail(MG_ERR_ARG, "mg_gemm: group_m %d is negative", a->group_m);
-    if ((a->flags & ~MG_FLAG_TIGHT_BUFFERS) || a->reserved)
+    if ((a->flags & ~(MG_FLAG_TIGHT_BUFFERS | MG_FLAG_SPLITK_ATOMIC)) || a->reserved)
         return fail(MG_ERR_ARG, "mg_gemm: unknown flags 0x%x", a->flags);
     return MG_OK;
 }
@@ -294,7 +295,18 @@ struct mg_ctx {
     hipEvent_t ev0, ev1;
     hipDeviceProp_t prop;
     bool capturing;
+    // Split-K workspace: partial tiles of the K slices plus one arrival counter
+    // per tile (zero between launches).  Allocated once, at init, so that its
+    // address can be baked into captured graphs; a GEMM whose partials do not
+    // fit adds into C with atomics instead.
+    float *ws;
+    int64_t ws_bytes;
+    int *cnt;
 };
+static const int64_t MG_MAX_COUNTED_TILES = 1 << 18;
+// Above this many bytes of partial tiles the slices add with atomics even though the
+// workspace could hold them: measured on MI355X, the gather loses once C is that large.
+static const int64_t MG_WS_AUTO_LIMIT = 96ll << 20;
 
 struct mg_graph {
     hipGraph_t graph;
@@ -336,6 +348,26 @@ int mg_init(int device_index, mg_ctx **out) {
         delete c;
         return fail(MG_ERR_NODEVICE, "mg_init: device is %s; this library is built for gfx950 only", arch);
     }
+    c->ws = nullptr;
+    c->cnt = nullptr;
+    c->ws_bytes = 256ll << 20;
+    if (const char *env = getenv("MIGEMM_SPLITK_WORKSPACE_MB")) c->ws_bytes = (int64_t)atoll(env) << 20;
+    if (c->ws_bytes > 0) {
+        e = hipMalloc((void **)&c->ws, (size_t)c->ws_bytes);
+        if (e == hipSuccess) e = hipMalloc((void **)&c->cnt, MG_MAX_COUNTED_TILES * sizeof(int));
+        if (e == hipSuccess) e = hipMemset(c->cnt, 0, MG_MAX_COUNTED_TILES * sizeof(int));
+        if (e != hipSuccess) {
+            (void)hipFree(c->ws);
+            (void)hipFree(c->cnt);
+            (void)hipEventDestroy(c->ev0);
+            (void)hipEventDestroy(c->ev1);
+            (void)hipStreamDestroy(c->stream);
+            delete c;
+            return hip_fail(e, "mg_init: split-K workspace");
+        }
+    } else {
+        c->ws_bytes = 0;
+    }
     *out = c;
     return MG_OK;
 }
@@ -347,6 +379,8 @@ int mg_destroy(mg_ctx *ctx) {
     (void)hipEventDestroy(ctx->ev0);
     (void)hipEventDestroy(ctx->ev1);
     (void)hipStreamDestroy(ctx->stream);
+    (void)hipFree(ctx->ws);
+    (void)hipFree(ctx->cnt);
     delete ctx;
     return MG_OK;
 }
@@ -513,7 +547,19 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     if ((int64_t)pl.grid_m * pl.grid_n > 0x7fffffffLL) return fail(MG_ERR_ARG, "mg_gemm: grid too large");
     if (lds_bytes_for(t, a.layout) > (int)ctx->prop.maxSharedMemoryPerMultiProcessor)
         return fail(MG_ERR_ARG, "mg_gemm: tile %d needs %d bytes of LDS", pl.tile, lds_bytes_for(t, a.layout));
-    if (pl.split_k > 1 && a.beta == 0) {
+    p.ws = nullptr;
+    p.cnt = nullptr;
+    if (pl.split_k > 1) {
+        // partial tiles go through the workspace when they fit
+        const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n * a.nbatch;
+        const int64_t need = tiles * pl.split_k * t.bm * t.bn * (int64_t)sizeof(float);
+        if (ctx->ws && need <= ctx->ws_bytes && need <= MG_WS_AUTO_LIMIT && tiles <= MG_MAX_COUNTED_TILES &&
+            !(a.flags & MG_FLAG_SPLITK_ATOMIC)) {
+            p.ws = ctx->ws;
+            p.cnt = ctx->cnt;
+        }
+    }
+    if (pl.split_k > 1 && a.beta == 0 && p.ws == nullptr) {
         // A dense C (pitch == N, batches back to back) is cleared as one long row.
         const bool dense = a.ldc == a.n && (a.nbatch == 1 || p.sc == a.m * a.n) &&
                            a.m * a.n * (int64_t)a.nbatch < 0x40000000LL;

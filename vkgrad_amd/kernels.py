@@ -63,7 +63,7 @@ class Matmul:
 
     def __init__(self, dev, sg=None, wm=None, wn=None, trans_a=False, trans_b=False,
                  capture_stats=False, lds=True, bk=64, batched=False, acc16=False,
-                 group_m=0, *, tile=None, dtype="f16", split_k=0):
+                 group_m=0, *, tile=None, dtype="f16", split_k=0, atomic_split=False):
         if acc16:
             raise VkError("acc16 (f16 output) is not provided: no call site of the path uses it")
         if dtype not in L.DTYPES:
@@ -77,6 +77,7 @@ class Matmul:
         self.group_m = int(group_m)
         self.dtype = dtype
         self.split_k = int(split_k)
+        self.atomic_split = bool(atomic_split)   # K slices add into C with atomics, not via the workspace
         if tile is None and sg is not None:
             tile = _nearest_tile(sg * (wm or 1) * 16, (wn or 1) * 16)
         if tile is not None and not 0 <= tile < len(CONFIGS):
@@ -91,7 +92,7 @@ class Matmul:
             base = "mm_auto"
         self.name = (f"{base}_{dtype}{'_ta' if trans_a else ''}{'_tb' if trans_b else ''}"
                      f"{'_bat' if batched else ''}{'_g' + str(group_m) if group_m else ''}"
-                     f"{'_s' + str(split_k) if split_k > 1 else ''}")
+                     f"{'_s' + str(split_k) if split_k > 1 else ''}{'_at' if atomic_split else ''}")
         self._keep = []
 
     def fits(self, m, n, k):
@@ -131,6 +132,8 @@ class Matmul:
         full_a = ((nb - 1) * sa + (a_rows - 1) * ga.lda + ((a_cols + 7) & ~7)) * esz
         full_b = ((nb - 1) * sb + (b_rows - 1) * ga.ldb + ((b_cols + 7) & ~7)) * esz
         ga.flags = L.MG_FLAG_TIGHT_BUFFERS if (full_a > a.size or full_b > b.size) else 0
+        if self.atomic_split:
+            ga.flags |= L.MG_FLAG_SPLITK_ATOMIC
         if m > 0 and n > 0 and k > 0:
             if need_a > a.size or need_b > b.size or need_c > c.size:
                 raise VkError(f"{self.name}: shape {m}x{n}x{k} (nbatch {nb}) needs {need_a}/{need_b}/{need_c} "
@@ -338,7 +341,8 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
         e = lookup_tuned(dev.name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate, lda, ldb, ldc)
         if e is not None:
             return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=e["tile_id"],
-                          dtype=dtype, split_k=e.get("split_k", 0), group_m=e.get("group_m", 0)), e
+                          dtype=dtype, split_k=e.get("split_k", 0), group_m=e.get("group_m", 0),
+                          atomic_split=e.get("atomic_split", False)), e
 
     nb = nbatch if batched else 1
     pa = int(lda) if lda is not None else (m if trans_a else k)      # row pitches
@@ -363,9 +367,11 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
                       lda=lda, ldb=ldb, ldc=ldc, **call)
 
     try:
+        # a K split is timed both ways: slices meeting in the workspace, and adding atomically
         cands = [Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=t, dtype=dtype,
-                        split_k=s, group_m=0)
-                 for t, s in candidate_space(m, n, k, getattr(dev, "compute_units", 256), nb)]
+                        split_k=s, group_m=0, atomic_split=at)
+                 for t, s in candidate_space(m, n, k, getattr(dev, "compute_units", 256), nb)
+                 for at in ((False, True) if s > 1 else (False,))]
         if not cands:
             raise VkError(f"no matmul config fits {m}x{n}x{k}")
 
@@ -384,14 +390,16 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
             t = best_t[id(x)]
             tf = x.flops(m, n, k) * nb / t / 1e12
             results.append({"config": [x.bm, x.bn, x.bk], "lds": True, "tflops": tf, "ms": t * 1e3,
-                            "tile": [x.bm, x.bn], "tile_id": x.tile, "split_k": x.split_k})
+                            "tile": [x.bm, x.bn], "tile_id": x.tile, "split_k": x.split_k,
+                            "atomic_split": x.atomic_split})
             if verbose:
                 print(f"    tile {x.bm:3d}x{x.bn:3d} split_k={x.split_k:2d}  {tf:8.2f} TFLOPS  {t * 1e6:9.1f} us")
         results.sort(key=lambda r: -r["tflops"])
         best = dict(results[0])
 
         variants = [Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=best["tile_id"],
-                           dtype=dtype, split_k=best["split_k"], group_m=g) for g in (0, 1, 2, 4, 16)]
+                           dtype=dtype, split_k=best["split_k"], group_m=g, atomic_split=best["atomic_split"])
+                    for g in (0, 1, 2, 4, 16)]
         gt = measure(variants)
         scored = sorted(((v.flops(m, n, k) * nb / gt[id(v)] / 1e12, v.group_m) for v in variants), reverse=True)
         if verbose:
@@ -406,7 +414,8 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
             cache[key] = best
             _save_cache(cache)
         return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=best["tile_id"],
-                      dtype=dtype, split_k=best["split_k"], group_m=best["group_m"]), best
+                      dtype=dtype, split_k=best["split_k"], group_m=best["group_m"],
+                      atomic_split=best["atomic_split"]), best
     finally:
         if bufs:
             for x in bufs:
