@@ -136,17 +136,31 @@ static bool dma_eligible(const mg_gemm_args &a, const TileDesc &t, int64_t k_per
     return true;
 }
 
-// Sustained MFMA rate of a tile's main loop relative to the chip's dense peak,
-// from measurements on MI355X at large K (it only has to rank the tiles).
-static double tile_efficiency(const TileDesc &t) {
-    const int area = t.bm * t.bn;
-    if (t.nstage > 0) return area >= 65536 ? 0.55 : (area >= 32768 ? 0.45 : 0.48);
-    if (area >= 65536) return 0.42;
-    if (area >= 32768) return 0.36;
-    if (area >= 16384) return 0.34;
-    if (area >= 8192) return 0.22;
-    return 0.14;
-}
+// Cost table of the picker, fitted to timings of every (tile, split) candidate over 54
+// shapes on MI355X (benchmark shapes, squares, skinny and deep-K cases, random bf16
+// operands): time = 1.5 us + rounds * (overhead + K-blocks * block_time * occupancy).
+// {per-workgroup overhead in us, time per K-block in us} by tile and layout NN, NT, TN.
+// It only has to rank candidates; the tuner measures.
+static const float g_cost[MG_NUM_TILES][3][2] = {
+    {{8.20f, 1.735f}, {13.99f, 1.490f}, {7.02f, 1.568f}},   // 0 mm_256x256x64_w2x2
+    {{6.47f, 1.019f}, {12.43f, 0.788f}, {4.21f, 0.996f}},   // 1 mm_256x128x64_w2x2
+    {{6.57f, 0.971f}, {11.43f, 0.797f}, {4.06f, 1.035f}},   // 2 mm_128x256x64_w2x2
+    {{5.46f, 1.023f}, {7.79f, 0.812f}, {3.07f, 0.978f}},    // 3 mm_128x128x64_w2x2
+    {{2.29f, 0.570f}, {1.10f, 0.752f}, {2.00f, 0.582f}},    // 4 mm_64x64x64_w2x2
+    {{5.28f, 0.629f}, {7.41f, 0.599f}, {3.31f, 0.684f}},    // 5 mm_64x256x64_w1x4
+    {{3.38f, 0.522f}, {4.98f, 0.476f}, {3.23f, 0.533f}},    // 6 mm_32x256x64_w1x4
+    {{5.29f, 0.648f}, {4.75f, 0.660f}, {3.38f, 0.678f}},    // 7 mm_256x64x64_w4x1
+    {{3.46f, 0.555f}, {3.44f, 0.552f}, {2.97f, 0.576f}},    // 8 mm_256x32x64_w4x1
+    {{5.87f, 0.716f}, {12.93f, 0.610f}, {4.52f, 0.694f}},   // 9 mmd_256x256x32_w2x4_s4
+    {{7.02f, 1.336f}, {12.86f, 1.163f}, {4.69f, 1.275f}},   // 10 mmd_256x256x64_w2x4_s2
+    {{6.05f, 0.844f}, {6.24f, 0.827f}, {3.05f, 0.969f}},    // 11 mmd_128x128x64_w2x2_s2
+    {{5.35f, 0.843f}, {9.50f, 0.814f}, {4.11f, 0.783f}},    // 12 mmd_128x256x32_w2x2_s3
+    {{5.52f, 0.899f}, {11.10f, 0.822f}, {4.23f, 0.787f}},   // 13 mmd_256x128x32_w2x2_s3
+    {{5.22f, 0.486f}, {5.92f, 0.576f}, {3.21f, 0.460f}},    // 14 mmd_128x128x32_w2x2_s3
+    {{7.29f, 1.397f}, {6.65f, 1.446f}, {4.48f, 1.377f}},    // 15 mmp_256x256x64_w2x4_s2
+    {{7.27f, 0.809f}, {6.45f, 0.810f}, {4.21f, 0.792f}},    // 16 mmp_256x256x32_w2x4_s4
+    {{6.21f, 0.873f}, {3.06f, 1.026f}, {3.10f, 0.985f}},    // 17 mmp_128x128x64_w2x2_s2
+};
 
 static int wgs_per_cu(const TileDesc &t, int layout) {
     const int by_lds = 163840 / lds_bytes_for(t, layout);
@@ -157,24 +171,24 @@ static int wgs_per_cu(const TileDesc &t, int layout) {
     return w < 1 ? 1 : w;
 }
 
-// Estimated time (microseconds) of one (tile, split) choice: rounds of
-// co-resident workgroups, each round paying the main loop at the tile's rate
-// plus the part of its pipeline fill and C traffic that nothing overlaps.
+// Estimated time (microseconds) of one (tile, split) choice: rounds of co-resident
+// workgroups, each paying its overhead plus its K-blocks; a CU that holds fewer
+// workgroups than it could runs each of them faster, down to a latency floor.
 static double plan_cost_us(const mg_gemm_args &a, const TileDesc &t, int split, int cus) {
     const int64_t gm = cdiv(a.m, t.bm), gn = cdiv(a.n, t.bn);
-    const int64_t groups = gm * gn * (int64_t)a.nbatch * split;
+    const int64_t units = gm * gn * (int64_t)a.nbatch * split;
     const int wpc = wgs_per_cu(t, a.layout);
     const int64_t slots = (int64_t)cus * wpc;
-    const int64_t rounds = cdiv(groups, slots);
-    const double cu_rate = tile_efficiency(t) * 2.5e9 / 256.0;       // FLOP per us per CU
-    const double wg_flop = 2.0 * t.bm * t.bn * ((double)a.k / split);
-    // a round keeps min(wpc, groups/cus) workgroups on a CU, sharing its rate
-    const double busy = groups >= slots ? wpc : (groups > cus ? (double)groups / cus : 1.0);
-    const double loop_us = rounds * busy * wg_flop / cu_rate;
-    const double fill_us = rounds * 2.0 / (busy > 1.0 ? busy : 1.0);
-    const double c_bytes = (double)a.m * a.n * 4.0 * a.nbatch * (split > 1 ? 2.0 * split : (a.beta ? 2.0 : 1.0));
-    const double c_us = c_bytes / 4.5e6 * (busy > 1.0 ? 0.6 : 1.0);
-    return loop_us + fill_us + c_us + (split > 1 && !a.beta ? 3.0 : 0.0);
+    double rounds = t.persistent ? (double)units / (double)slots : (double)cdiv(units, slots);
+    if (rounds < 1.0) rounds = 1.0;
+    const int64_t resident = cdiv(units, cus) < wpc ? cdiv(units, cus) : wpc;
+    double occupancy = (double)resident / wpc;
+    if (occupancy < 0.6) occupancy = 0.6;
+    const int lay = a.layout == MG_NN ? 0 : (a.layout == MG_NT ? 1 : 2);
+    const double kb = (double)cdiv(cdiv(a.k, t.bk), split);
+    double us = 1.5 + rounds * (g_cost[t.id][lay][0] + kb * occupancy * g_cost[t.id][lay][1]);
+    if (split > 1) us += 2.0 + (double)a.m * a.n * 4.0 * a.nbatch * split * 2.0 / 3.0e6;   // partials out and back
+    return us;
 }
 
 static void finish_plan(const mg_gemm_args &a, int tile, int split, Plan &pl) {
@@ -220,16 +234,20 @@ static void pick_plan(const mg_gemm_args &a, int cus, Plan &pl) {
             const int64_t kblocks = cdiv(a.k, d.bk);
             const int64_t groups = cdiv(a.m, d.bm) * cdiv(a.n, d.bn) * (int64_t)a.nbatch;
             const int64_t slots = (int64_t)cus * wgs_per_cu(d, a.layout);
-            int cand[4] = {1, 0, 0, 0};
+            int cand[8] = {1, 0, 0, 0, 0, 0, 0, 0};
             int nc = 1;
             if (split > 0) {
                 cand[0] = split;
-            } else if (groups < slots && kblocks >= 8) {
-                int s = (int)(slots / groups);
-                if (s > kblocks / 4) s = (int)(kblocks / 4);
-                if (s > 1) cand[nc++] = s;
-                if (s > 3) cand[nc++] = s / 2;
-                if (2 * s <= kblocks / 4) cand[nc++] = 2 * s;
+            } else if (groups < slots && kblocks >= 4) {
+                // splits that bring the grid to about a half, one or two workgroups per slot
+                const int64_t cap = kblocks / 2;
+                for (int64_t target : {slots / 2, slots, 2 * slots, (int64_t)cus}) {
+                    int64_t s = target / groups;
+                    if (s > cap) s = cap;
+                    bool seen = s < 2;
+                    for (int c = 0; c < nc; c++) seen = seen || cand[c] == (int)s;
+                    if (!seen) cand[nc++] = (int)s;
+                }
             }
             for (int c = 0; c < nc; c++) {
                 const int s = cand[c];

@@ -300,11 +300,16 @@ def candidate_space(m, n, k, cus=256, nbatch=1):
     """(tile, split_k) pairs worth timing for a shape: every tile whose padding
     waste is tolerable, with K splits that bring an under-filled grid up to
     about one or two workgroups per CU."""
+    def useful_of(t):
+        gm, gn = -(-m // t["bm"]), -(-n // t["bn"])
+        return (m * n) / (gm * t["bm"] * gn * t["bn"])
+
+    # skinny problems waste most of every tile: keep the tiles that waste least
+    floor = min(0.45, 0.7 * max(useful_of(t) for t in CONFIGS))
     out = []
     for t in CONFIGS:
         gm, gn = -(-m // t["bm"]), -(-n // t["bn"])
-        useful = (m * n) / (gm * t["bm"] * gn * t["bn"])
-        if useful < 0.45 and len(CONFIGS) > 1:
+        if useful_of(t) < floor and len(CONFIGS) > 1:
             continue
         groups = gm * gn * nbatch
         kblocks = -(-k // t["bk"])
