@@ -208,6 +208,29 @@ def test_split_k_without_workspace_adds_atomically(monkeypatch):
         d.destroy()
 
 
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+def test_stream_k_tiles_exact(dev, layout):
+    """Stream-K tiles: the tiles beyond the last whole round of the resident grid are cut
+    along K into one run per workgroup and the pieces meet in the workspace.  Shapes with
+    more tiles than slots (a remainder after whole rounds), fewer tiles than slots (all
+    pieces), ragged edges, bias and beta = 1; bit exact on integer data and bit identical
+    from run to run on random data."""
+    from vkgrad_amd.kernels import CONFIGS
+    ta, tb = LAYOUTS[layout]
+    sk = [t for t in CONFIGS if t["persistent"] == 2]
+    assert len(sk) >= 2
+    for t in sk:
+        big = 3000 if t["bm"] == 128 else 4400          # 576 tiles on 512 slots / 324 on 256
+        for m, n, k in [(big, big, 512), (1000, 1016, 1024), (392, 648, 2048), (128, 128, 4096)]:
+            r, got, ref = check_case(dev, m, n, k, ta, tb, "bf16", seed=m + k, integer=True, tile=t["id"], bias=True,
+                                     accumulate=True)
+            assert r["exact"], f"{t['name']} {layout} {m}x{n}x{k}: max diff {np.abs(got - ref).max()}"
+        r, got, ref = check_case(dev, 1000, 1016, 1024, ta, tb, "f16", seed=9, tile=t["id"])
+        _assert_close(r, f"{t['name']} {layout}")
+        r2, got2, _ = check_case(dev, 1000, 1016, 1024, ta, tb, "f16", seed=9, tile=t["id"])
+        assert np.array_equal(got, got2)
+
+
 def test_wrong_layout_fails(dev):
     """Negative control (idea: test_hf_gpt2.py:129-136): a square operand read
     with the wrong layout passes every shape check and must fail on values."""

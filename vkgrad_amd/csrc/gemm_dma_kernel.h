@@ -301,8 +301,9 @@ gemm_dma_kernel(const GemmParams p) {
     int mode = p.split_k > 1 ? 2 : (p.beta ? 1 : 0);
     if (p.split_k > 1 && p.ws != nullptr) {
         __syncthreads();   // every wave is done with the ring: its first word serves as the flag
-        if (!splitk_gather<TM, TN, NW * 64>(acc, p.ws, p.cnt, (int64_t)blockIdx.z * gridDim.x + blockIdx.x,
-                                             (int64_t)gridDim.x * gridDim.z, blockIdx.y, gridDim.y, tid,
+        const int64_t tile_id = (int64_t)blockIdx.z * gridDim.x + blockIdx.x, ntiles = (int64_t)gridDim.x * gridDim.z;
+        if (!splitk_gather<TM, TN, NW * 64>(acc, p.ws, p.cnt + tile_id, blockIdx.y, gridDim.y,
+                                             [&](int sl) { return (int64_t)sl * ntiles + tile_id; }, tid,
                                              reinterpret_cast<int *>(dsm)))
             return;
         add_bias = p.bias != nullptr;
@@ -429,7 +430,7 @@ __device__ __forceinline__ void wait_blocks_and_barrier(int blocks) {
 // EPI_LOADS = true adds the bias epilogue (its loads drain vmcnt once per tile);
 // C += (beta = 1 or split-K) is an L2 atomic add and needs no load.
 // ---------------------------------------------------------------------------
-template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool EPI_LOADS>
+template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool EPI_LOADS, bool STREAMK>
 __global__ void __launch_bounds__(WGM *WGN * 64)
 gemm_dmap_kernel(const GemmParams p) {
     constexpr bool A_KC = (LAYOUT != L_TN);
@@ -457,32 +458,74 @@ gemm_dmap_kernel(const GemmParams p) {
     const uint16_t *B = p.B + zb * p.sb;
     float *C = p.C + zb * p.sc;
 
-    // Work units of this workgroup: u = round * gridDim.x + pos, pos renumbered
-    // XCD-major so the workgroups behind one L2 hold neighbouring tiles.  Units
-    // are slice-major (all tiles of K slice 0, then slice 1, ...), so the slices
-    // of one tile are not adding into it at the same moment.
+    // Work units of this workgroup.  Positions are renumbered XCD-major so the
+    // workgroups behind one L2 hold neighbouring tiles.
+    //   plain:    unit i is (K slice, tile) number pos + i * gridDim.x, slice-major (all
+    //             tiles of slice 0, then slice 1, ...), so the slices of one tile are
+    //             not meeting at the same moment.
+    //   stream-K: the tiles that fill whole rounds are dealt out the same way; the K-blocks
+    //             of the remaining tiles (less than one round) are cut into gridDim.x equal
+    //             contiguous runs, one per workgroup, done first.  A run covers the end of
+    //             one tile and/or the start of the next; the pieces of a tile meet in the
+    //             workspace like K slices (slot 2 * pos for a workgroup's first piece,
+    //             2 * pos + 1 for its second).
     const int nwg = gridDim.x;
     const int ntiles = p.grid_m * p.grid_n;
-    const int n_units = ntiles * p.split_k;
     int pos = blockIdx.x;
     if ((nwg & 7) == 0) pos = (pos & 7) * (nwg >> 3) + (pos >> 3);
 
     struct Unit {
-        int m0, n0, kbeg, nkb, lin, slice;
+        int m0, n0, kbeg, nkb, lin, slice, nslices;
     };
-    auto unit_of = [&](int u) -> Unit {
-        const int slice = u / ntiles;
-        const int lin = u - slice * ntiles;
+    auto place = [&](int lin, Unit &q) {
         const int in_group = p.group_m * p.grid_n;
         const int gid = lin / in_group;
         const int first_m = gid * p.group_m;
         const int gsize = min(p.grid_m - first_m, p.group_m);
         const int r = lin - gid * in_group;
-        Unit q;
         q.m0 = (first_m + r % gsize) * BM;
         q.n0 = (r / gsize) * BN;
         q.lin = lin;
+    };
+    // stream-K bookkeeping (all zero in plain mode).  Run w covers the blocks
+    // [run_begin(w), run_begin(w + 1)) of the remaining tiles, numbered tile-major.
+    const bool stream_k = STREAMK && p.stream_k;   // a stream-K tile without workspace runs plain
+    const int nkb_tile = p.K / BK;
+    const int full_rounds = stream_k ? p.sk_full_rounds : 0;
+    const int rem_wgs = stream_k ? p.sk_rem_wgs : 0;
+    auto run_begin = [&](int w) -> int { return w * p.sk_q + min(w, p.sk_r); };
+    int rb0 = 0, rb1 = 0, t_first = 0, rem_units = 0;
+    if (STREAMK && pos < rem_wgs) {
+        rb0 = run_begin(pos);
+        rb1 = run_begin(pos + 1);
+        t_first = rb0 / nkb_tile;
+        rem_units = (rb1 - 1) / nkb_tile - t_first + 1;
+    }
+    const int n_plain = stream_k ? full_rounds : (ntiles * p.split_k - pos + nwg - 1) / nwg;
+    const int my_units = rem_units + (n_plain > 0 ? n_plain : 0);
+
+    auto unit_at = [&](int i) -> Unit {
+        Unit q;
+        if (STREAMK && i < rem_units) {
+            const int t = t_first + i;                          // tile among the remaining ones
+            const int t0 = t * nkb_tile, t1 = t0 + nkb_tile;
+            const int lo = max(rb0, t0) - t0, hi = min(rb1, t1) - t0;
+            place(full_rounds * nwg + t, q);
+            q.kbeg = lo * BK;
+            q.nkb = hi - lo;
+            // the runs that meet this tile belong to consecutive workgroups around this one
+            int first_w = pos, last_w = pos;
+            while (first_w > 0 && run_begin(first_w) > t0) first_w--;
+            while (last_w + 1 < rem_wgs && run_begin(last_w + 1) < t1) last_w++;
+            q.slice = pos - first_w;
+            q.nslices = last_w - first_w + 1;
+            return q;
+        }
+        const int u = pos + (i - rem_units) * nwg;
+        const int slice = stream_k ? 0 : u / ntiles;
+        place(u - slice * ntiles, q);
         q.slice = slice;
+        q.nslices = stream_k ? 1 : p.split_k;
         q.kbeg = slice * p.k_per_split;
         q.nkb = (min(p.K, q.kbeg + p.k_per_split) - q.kbeg) / BK;
         return q;
@@ -495,14 +538,14 @@ gemm_dmap_kernel(const GemmParams p) {
     // ---- load side ----
     OA oa;
     OB ob;
-    int l_u = pos;            // unit being loaded
+    int l_i = 0;              // unit being loaded
     int l_kb = 0, l_nkb = 0;  // next block of it, and its block count
     int issued = 0;           // K-blocks issued so far (flat)
-    bool l_live = l_u < n_units;
+    bool l_live = my_units > 0;
     auto issue_next = [&]() {
         if (!l_live) return;
         if (l_kb == 0) {
-            const Unit q = unit_of(l_u);
+            const Unit q = unit_at(l_i);
             l_nkb = q.nkb;
             oa.init(A, p.lda, q.m0, p.M, q.kbeg, wave, lane);
             ob.init(B, p.ldb, q.n0, p.N, q.kbeg, wave, lane);
@@ -513,8 +556,7 @@ gemm_dmap_kernel(const GemmParams p) {
         issued++;
         if (++l_kb == l_nkb) {
             l_kb = 0;
-            l_u += nwg;
-            l_live = l_u < n_units;
+            l_live = ++l_i < my_units;
         }
     };
 
@@ -558,11 +600,25 @@ gemm_dmap_kernel(const GemmParams p) {
     auto epilogue = [&](const Unit &q) {
         const bool interior = (q.m0 + BM <= p.M) && (q.n0 + BN <= p.N);
         bool add_bias = EPI_LOADS && p.bias != nullptr && q.kbeg == 0;
-        bool atomic = p.split_k > 1 || p.beta;
-        if (p.split_k > 1 && p.ws != nullptr) {
-            if (!splitk_gather<TM, TN, NW * 64>(acc, p.ws, p.cnt, zb * ntiles + q.lin, (int64_t)ntiles * gridDim.z,
-                                                 q.slice, p.split_k, tid, &gather_flag))
-                return;
+        bool atomic = q.nslices > 1 || p.beta;
+        if (q.nslices > 1 && p.ws != nullptr) {
+            const int64_t tile_id = zb * ntiles + q.lin;
+            // Workspace slot of piece sl.  Stream-K: the piece belongs to workgroup
+            // w = pos - q.slice + sl and is that workgroup's second piece when its run
+            // started in an earlier tile.  Plain split: slices are slot planes over the tiles.
+            const int64_t all_tiles = (int64_t)ntiles * gridDim.z;
+            const int t0 = (q.lin - full_rounds * nwg) * nkb_tile;
+            const bool mine = splitk_gather<TM, TN, NW * 64>(
+                acc, p.ws, p.cnt + tile_id, q.slice, q.nslices,
+                [&](int sl) -> int64_t {
+                    if (STREAMK && stream_k) {
+                        const int w = pos - q.slice + sl;
+                        return (zb * nwg + w) * 2 + (run_begin(w) < t0 ? 1 : 0);
+                    }
+                    return (int64_t)sl * all_tiles + tile_id;
+                },
+                tid, &gather_flag);
+            if (!mine) return;
             add_bias = EPI_LOADS && p.bias != nullptr;
             atomic = p.beta != 0;
         }
@@ -616,8 +672,8 @@ gemm_dmap_kernel(const GemmParams p) {
     wait_blocks_and_barrier<L, NSTAGE - 1>(issued - 1);
     read_frags(0, 0, 0);
 
-    int c_u = pos;
-    Unit cq = unit_of(c_u);
+    int c_i = 0;
+    Unit cq = unit_at(0);
     int c_kb = 0;
     int stage = 0;
     // Invariant at the top of iteration ci: blocks ci .. issued-1 are issued,
@@ -650,9 +706,8 @@ gemm_dmap_kernel(const GemmParams p) {
         if (++c_kb == cq.nkb) {
             epilogue(cq);
             c_kb = 0;
-            c_u += nwg;
-            if (c_u < n_units) {
-                cq = unit_of(c_u);
+            if (++c_i < my_units) {
+                cq = unit_at(c_i);
                 zero_acc();
             }
         }
@@ -677,10 +732,10 @@ hipError_t launch_gemm_dma(const GemmParams &p, dim3 grid, hipStream_t stream) {
 }
 
 // Persistent launcher: grid.x is the number of resident workgroups the host chose.
-template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool EPI_LOADS>
+template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool EPI_LOADS, bool STREAMK>
 hipError_t launch_gemm_dmap(const GemmParams &p, dim3 grid, hipStream_t stream) {
     using TT = DmaTraits<LAYOUT, BM, BN, BK, WGM, WGN, NSTAGE>;
-    auto kern = gemm_dmap_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, NSTAGE, EPI_LOADS>;
+    auto kern = gemm_dmap_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, NSTAGE, EPI_LOADS, STREAMK>;
     static bool attr_done = false;
     if (!attr_done) {
         if (TT::LDS_BYTES > 65536) {

@@ -1,7 +1,7 @@
 // Instantiations of the GEMM templates: layout TN, dtype BF16, every tile.
 // Entry [tile][0] serves aligned operands, [tile][1] arbitrary alignment (absent
 // for direct-to-LDS tiles, which fall back to a register-staged tile instead).
-// Persistent tiles use [0] for the plain epilogue and [1] for the one with bias.
+// Persistent and stream-K tiles use [0] for the plain epilogue and [1] for the one with bias.
 #include "gemm_dma_kernel.h"
 #include "gemm_kernel.h"
 #include "tiles.h"
@@ -11,10 +11,14 @@ namespace mg {
     {launch_gemm<L_TN, D_BF16, bm, bn, bk, wgm, wgn, false>, launch_gemm<L_TN, D_BF16, bm, bn, bk, wgm, wgn, true>},
 #define D(id, bm, bn, bk, wgm, wgn, ns, fb) {launch_gemm_dma<L_TN, D_BF16, bm, bn, bk, wgm, wgn, ns>, nullptr},
 #define P(id, bm, bn, bk, wgm, wgn, ns, fb)                          \
-    {launch_gemm_dmap<L_TN, D_BF16, bm, bn, bk, wgm, wgn, ns, false>, \
-     launch_gemm_dmap<L_TN, D_BF16, bm, bn, bk, wgm, wgn, ns, true>},
-launch_fn launch_table_tn_bf16[MG_NUM_TILES][2] = {MG_TILE_LIST(V, D, P)};
+    {launch_gemm_dmap<L_TN, D_BF16, bm, bn, bk, wgm, wgn, ns, false, false>, \
+     launch_gemm_dmap<L_TN, D_BF16, bm, bn, bk, wgm, wgn, ns, true, false>},
+#define S(id, bm, bn, bk, wgm, wgn, ns, fb)                                \
+    {launch_gemm_dmap<L_TN, D_BF16, bm, bn, bk, wgm, wgn, ns, false, true>, \
+     launch_gemm_dmap<L_TN, D_BF16, bm, bn, bk, wgm, wgn, ns, true, true>},
+launch_fn launch_table_tn_bf16[MG_NUM_TILES][2] = {MG_TILE_LIST(V, D, P, S)};
 #undef V
 #undef D
 #undef P
+#undef S
 }  // namespace mg

@@ -51,6 +51,11 @@ struct GemmParams {
     int xcd_remap;        // 1: renumber workgroups so neighbours share an XCD
     float *ws;            // split-K workspace (split_k * tiles * BM * BN floats) or null: add with atomics
     int *cnt;             // one arrival counter per tile, zero between launches
+    int stream_k;         // stream-K kernel only: balance the last partial round over all workgroups
+    // stream-K partition, computed by the host for the launched grid: whole rounds of tiles,
+    // workgroups that take a run of the remaining K-blocks, and the run length (sk_q blocks,
+    // one more for the first sk_r workgroups)
+    int sk_full_rounds, sk_rem_wgs, sk_q, sk_r;
 };
 
 template <int DT>
@@ -245,13 +250,14 @@ struct IntC {
 // streaming their operands through it.
 //
 // Returns true in the workgroup that has to write the tile; its acc then holds
-// the complete sum.  `flag` points at one int of LDS nobody else is using.
+// the complete sum.  slot_of(s) names the workspace slot (in partial tiles) of
+// slice s; `flag` points at one int of LDS nobody else is using.
 // ---------------------------------------------------------------------------
-template <int TM, int TN, int NTHREADS>
-__device__ __forceinline__ bool splitk_gather(f32x16 (&acc)[TM][TN], float *ws, int *cnt, int64_t tile, int64_t ntiles,
-                                              int slice, int nslices, int tid, int *flag) {
+template <int TM, int TN, int NTHREADS, class SlotOf>
+__device__ __forceinline__ bool splitk_gather(f32x16 (&acc)[TM][TN], float *ws, int *counter, int slice, int nslices,
+                                              SlotOf slot_of, int tid, int *flag) {
     constexpr int64_t TILE_FLOATS = (int64_t)TM * TN * 16 * NTHREADS;
-    float *mine = ws + ((int64_t)slice * ntiles + tile) * TILE_FLOATS + tid;
+    float *mine = ws + slot_of(slice) * TILE_FLOATS + tid;
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -263,14 +269,14 @@ __device__ __forceinline__ bool splitk_gather(f32x16 (&acc)[TM][TN], float *ws, 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this lane's partials have reached the coherence point
     __syncthreads();
     if (tid == 0) {
-        const int old = __hip_atomic_fetch_add(cnt + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         *flag = (old == nslices - 1);
     }
     __syncthreads();
     const bool last = *flag != 0;
     __syncthreads();      // flag may be reused (persistent kernel) once everyone has read it
     if (!last) return false;
-    if (tid == 0) cnt[tile] = 0;   // ready for the next launch
+    if (tid == 0) *counter = 0;   // ready for the next launch
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -278,7 +284,7 @@ __device__ __forceinline__ bool splitk_gather(f32x16 (&acc)[TM][TN], float *ws, 
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
     for (int sl = 0; sl < nslices; sl++) {
-        const float *src = ws + ((int64_t)sl * ntiles + tile) * TILE_FLOATS + tid;
+        const float *src = ws + slot_of(sl) * TILE_FLOATS + tid;
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -459,8 +465,9 @@ gemm_kernel(const GemmParams p) {
     int mode = p.split_k > 1 ? 2 : (p.beta ? 1 : 0);
     if (p.split_k > 1 && p.ws != nullptr) {
         __syncthreads();   // every wave is done with the LDS stages: smem[0..1] serves as the flag
-        if (!splitk_gather<TM, TN, WGM * WGN * 64>(acc, p.ws, p.cnt, (int64_t)blockIdx.z * gridDim.x + blockIdx.x,
-                                                    (int64_t)gridDim.x * gridDim.z, blockIdx.y, gridDim.y, tid,
+        const int64_t tile_id = (int64_t)blockIdx.z * gridDim.x + blockIdx.x, ntiles = (int64_t)gridDim.x * gridDim.z;
+        if (!splitk_gather<TM, TN, WGM * WGN * 64>(acc, p.ws, p.cnt + tile_id, blockIdx.y, gridDim.y,
+                                                    [&](int sl) { return (int64_t)sl * ntiles + tile_id; }, tid,
                                                     reinterpret_cast<int *>(smem)))
             return;
         add_bias = p.bias != nullptr;

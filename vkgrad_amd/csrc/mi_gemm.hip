@@ -45,15 +45,17 @@ struct TileDesc {
     int id, bm, bn, bk, wgm, wgn;
     int nstage;     // 0: register-staged kernel; >0: direct-to-LDS ring depth
     int fallback;   // tile of the same BM x BN with weaker preconditions (self: none)
-    int persistent; // 1: grid of resident workgroups looping over tiles
+    int persistent; // 1: grid of resident workgroups looping over tiles; 2: the same with stream-K balancing
 };
 #define V(id, bm, bn, bk, wgm, wgn) {id, bm, bn, bk, wgm, wgn, 0, id, 0},
 #define D(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 0},
 #define P(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 1},
-static const TileDesc g_tiles[MG_NUM_TILES] = {MG_TILE_LIST(V, D, P)};
+#define S(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 2},
+static const TileDesc g_tiles[MG_NUM_TILES] = {MG_TILE_LIST(V, D, P, S)};
 #undef V
 #undef D
 #undef P
+#undef S
 
 static thread_local char g_err[512] = "";
 
@@ -133,6 +135,9 @@ static bool dma_eligible(const mg_gemm_args &a, const TileDesc &t, int64_t k_per
     if (t.persistent) {
         if (a.k % t.bk != 0 || k_per_split % t.bk != 0) return false;
     }
+    if (t.persistent == 2 && split > 1) return false;   // stream-K cuts K itself
+    // the 256 x 256 stream-K kernel with the bias epilogue does not fit the register file
+    if (t.persistent == 2 && a.bias && t.bm * t.bn > 128 * 128) return false;
     return true;
 }
 
@@ -160,6 +165,8 @@ static const float g_cost[MG_NUM_TILES][3][2] = {
     {{7.29f, 1.397f}, {6.65f, 1.446f}, {4.48f, 1.377f}},    // 15 mmp_256x256x64_w2x4_s2
     {{7.27f, 0.809f}, {6.45f, 0.810f}, {4.21f, 0.792f}},    // 16 mmp_256x256x32_w2x4_s4
     {{6.21f, 0.873f}, {3.06f, 1.026f}, {3.10f, 0.985f}},    // 17 mmp_128x128x64_w2x2_s2
+    {{7.29f, 1.397f}, {6.65f, 1.446f}, {4.48f, 1.377f}},    // 18 mmk_256x256x64_w2x4_s2 (as 15)
+    {{6.21f, 0.873f}, {3.06f, 1.026f}, {3.10f, 0.985f}},    // 19 mmk_128x128x64_w2x2_s2 (as 17)
 };
 
 static int wgs_per_cu(const TileDesc &t, int layout) {
@@ -171,6 +178,17 @@ static int wgs_per_cu(const TileDesc &t, int layout) {
     return w < 1 ? 1 : w;
 }
 
+// Grid of a persistent launch.  Plain: one workgroup per slot, or per unit if there are
+// fewer.  Stream-K: also when tiles are fewer than slots every slot gets a run of K-blocks,
+// as long as a run stays at least four blocks long.
+static int64_t persistent_grid(const TileDesc &t, int64_t tiles, int split, int64_t kblocks, int64_t slots) {
+    const int64_t units = tiles * split;
+    if (t.persistent != 2 || units >= slots) return units < slots ? units : slots;
+    int64_t g = tiles * kblocks / 4;
+    if (g < tiles) g = tiles;
+    return g < slots ? g : slots;
+}
+
 // Estimated time (microseconds) of one (tile, split) choice: rounds of co-resident
 // workgroups, each paying its overhead plus its K-blocks; a CU that holds fewer
 // workgroups than it could runs each of them faster, down to a latency floor.
@@ -180,6 +198,20 @@ static double plan_cost_us(const mg_gemm_args &a, const TileDesc &t, int split, 
     const int wpc = wgs_per_cu(t, a.layout);
     const int64_t slots = (int64_t)cus * wpc;
     double rounds = t.persistent ? (double)units / (double)slots : (double)cdiv(units, slots);
+    if (t.persistent == 2) {
+        // stream-K: every workgroup gets the same number of K-blocks, plus the meeting of the pieces
+        const int64_t kblocks = cdiv(a.k, t.bk);
+        const int64_t g = persistent_grid(t, gm * gn, 1, kblocks, slots);
+        const double per_wg = (double)(gm * gn) * (double)kblocks / (double)g;   // blocks per workgroup
+        const int lay2 = a.layout == MG_NN ? 0 : (a.layout == MG_NT ? 1 : 2);
+        double occ = (double)cdiv(g, cus) / wpc;
+        if (occ > 1.0) occ = 1.0;
+        if (occ < 0.6) occ = 0.6;
+        double tiles_per_wg = (double)(gm * gn) / (double)g;
+        if (tiles_per_wg < 1.0) tiles_per_wg = 1.0;
+        return 1.5 + tiles_per_wg * g_cost[t.id][lay2][0] + per_wg * occ * g_cost[t.id][lay2][1] +
+               ((gm * gn) % g != 0 ? 4.0 : 0.0);
+    }
     if (rounds < 1.0) rounds = 1.0;
     const int64_t resident = cdiv(units, cus) < wpc ? cdiv(units, cus) : wpc;
     double occupancy = (double)resident / wpc;
@@ -196,6 +228,7 @@ static void finish_plan(const mg_gemm_args &a, int tile, int split, Plan &pl) {
     int64_t kblocks = cdiv(a.k, d->bk);
     if (split > kblocks) split = (int)kblocks;
     if (split < 1) split = 1;
+    if (d->persistent == 2) split = 1;
     int64_t kb_per = cdiv(kblocks, split);
     split = (int)cdiv(kblocks, kb_per);   // no empty slices
     while (!dma_eligible(a, *d, kb_per * d->bk, split) && d->fallback != tile) {
@@ -507,7 +540,8 @@ int mg_tile_info(int id, mg_tile *out) {
     out->lds_bytes = lds_bytes_for(t, MG_NT);
     out->min_m = 1;
     if (t.persistent)
-        snprintf(out->name, sizeof(out->name), "mmp_%dx%dx%d_w%dx%d_s%d", t.bm, t.bn, t.bk, t.wgm, t.wgn, t.nstage);
+        snprintf(out->name, sizeof(out->name), "%s_%dx%dx%d_w%dx%d_s%d", t.persistent == 2 ? "mmk" : "mmp", t.bm, t.bn, t.bk,
+                 t.wgm, t.wgn, t.nstage);
     else if (t.nstage > 0)
         snprintf(out->name, sizeof(out->name), "mmd_%dx%dx%d_w%dx%d_s%d", t.bm, t.bn, t.bk, t.wgm, t.wgn, t.nstage);
     else
@@ -567,6 +601,8 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
         return fail(MG_ERR_ARG, "mg_gemm: tile %d needs %d bytes of LDS", pl.tile, lds_bytes_for(t, a.layout));
     p.ws = nullptr;
     p.cnt = nullptr;
+    p.stream_k = 0;
+    p.sk_full_rounds = p.sk_rem_wgs = p.sk_q = p.sk_r = 0;
     if (pl.split_k > 1) {
         // partial tiles go through the workspace when they fit
         const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n * a.nbatch;
@@ -599,9 +635,27 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     if (t.persistent) {
         // resident workgroups loop over (slice, tile) units; [1] = epilogue with bias
         general = a.bias != nullptr ? 1 : 0;
-        const int64_t units = (int64_t)pl.grid_m * pl.grid_n * pl.split_k;
+        const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n;
         const int64_t slots = (int64_t)ctx->prop.multiProcessorCount * wgs_per_cu(t, a.layout);
-        grid = dim3((unsigned)(units < slots ? units : slots), 1, (unsigned)a.nbatch);
+        int64_t g = persistent_grid(t, tiles, pl.split_k, a.k / t.bk, slots);
+        if (t.persistent == 2 && pl.split_k == 1) {
+            // two workspace slots per workgroup and batch; without them the tile runs as plain persistent
+            const int64_t need = 2 * g * a.nbatch * t.bm * t.bn * (int64_t)sizeof(float);
+            const int64_t rem_blocks = (tiles % g) * (a.k / t.bk);
+            if (ctx->ws && need <= ctx->ws_bytes && tiles * a.nbatch <= MG_MAX_COUNTED_TILES &&
+                rem_blocks < 0x7fffffffLL) {
+                p.stream_k = 1;
+                p.sk_full_rounds = (int)(tiles / g);
+                p.sk_rem_wgs = (int)(rem_blocks < g ? rem_blocks : g);
+                p.sk_q = p.sk_rem_wgs ? (int)(rem_blocks / p.sk_rem_wgs) : 0;
+                p.sk_r = p.sk_rem_wgs ? (int)(rem_blocks % p.sk_rem_wgs) : 0;
+                p.ws = ctx->ws;
+                p.cnt = ctx->cnt;
+            } else {
+                g = tiles < slots ? tiles : slots;
+            }
+        }
+        grid = dim3((unsigned)g, 1, (unsigned)a.nbatch);
         p.xcd_remap = 0;
     }
     launch_fn fn = table_for(a.layout, a.dtype)[pl.tile][general];

@@ -10,10 +10,15 @@
 //   persistent direct-to-LDS: additionally K slices that are multiples of BK
 //     P(id, BM, BN, BK, WGM, WGN, NSTAGE, fallback_id) — falls back to the
 //     one-tile-per-workgroup direct-to-LDS tile of the same shape.
+//   stream-K: the persistent kernel again, but the tiles that do not fill a whole
+//     round of the resident grid are cut along K into one equal run per workgroup
+//     (pieces meet in the context's workspace), so every CU finishes together.
+//     S(id, BM, BN, BK, WGM, WGN, NSTAGE, fallback_id) — falls back to the
+//     persistent tile of the same shape (no workspace, or ragged K).
 // WGM x WGN wavefronts of 64 lanes per workgroup.
 #pragma once
 
-#define MG_TILE_LIST(V, D, P)      \
+#define MG_TILE_LIST(V, D, P, S)   \
     V(0, 256, 256, 64, 2, 2)       \
     V(1, 256, 128, 64, 2, 2)       \
     V(2, 128, 256, 64, 2, 2)       \
@@ -31,6 +36,8 @@
     D(14, 128, 128, 32, 2, 2, 3, 3) \
     P(15, 256, 256, 64, 2, 4, 2, 10) \
     P(16, 256, 256, 32, 2, 4, 4, 9) \
-    P(17, 128, 128, 64, 2, 2, 2, 11)
+    P(17, 128, 128, 64, 2, 2, 2, 11) \
+    S(18, 256, 256, 64, 2, 4, 2, 15) \
+    S(19, 128, 128, 64, 2, 2, 2, 17)
 
-#define MG_NUM_TILES 18
+#define MG_NUM_TILES 20

@@ -314,7 +314,7 @@ def candidate_space(m, n, k, cus=256, nbatch=1):
         groups = gm * gn * nbatch
         kblocks = -(-k // t["bk"])
         splits = {1}
-        if groups < cus and kblocks >= 4:
+        if groups < cus and kblocks >= 4 and t.get("persistent") != 2:   # stream-K tiles cut K themselves
             for target in (cus, 2 * cus):
                 s = max(1, min(target // groups, kblocks // 2))
                 # the neighbours too: atomic traffic grows with the split, so the
