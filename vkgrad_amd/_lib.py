@@ -4,7 +4,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmigemm.so")
+LIB_PATH = os.environ.get("VKGRAD_AMD_LIB") or os.path.join(_HERE, "libmigemm.so")
 
 MG_OK, MG_ERR_ARG, MG_ERR_HIP, MG_ERR_STATE, MG_ERR_NOMEM, MG_ERR_NODEVICE = range(6)
 MG_NN, MG_NT, MG_TN = 0, 1, 2

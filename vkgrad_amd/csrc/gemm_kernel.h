@@ -509,7 +509,7 @@ gemm_kernel(const GemmParams p) {
                         if constexpr (MODE == 2)
                             __hip_atomic_fetch_add(ct + ro * ldc, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         else
-                            ct[ro * ldc] = v;
+                            __builtin_nontemporal_store(v, ct + ro * ldc);   // written once: stream past the L2
                     }
                 }
             }
