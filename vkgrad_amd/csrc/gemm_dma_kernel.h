@@ -87,6 +87,12 @@ struct DmaOp {
         }
     }
 
+    // Skip one K-block (another wavefront group issues it).
+    __device__ __forceinline__ void advance(int64_t kstep_elems) {
+#pragma unroll
+        for (int t = 0; t < PERW; t++) g[t] += kstep_elems;
+    }
+
     // K remainder: fill this operand's LDS region with the block [k0, k0 + BK) of
     // which only k < kend exists, through registers, zero beyond kend, in the same
     // swizzled layout the direct loads produce.
@@ -177,10 +183,18 @@ gemm_dma_kernel(const GemmParams p) {
     constexpr int TM = WTM / 32, TN = WTN / 32;
     constexpr int KK = BK / 16;
     static_assert(WTM % 32 == 0 && WTN % 32 == 0 && KK % 2 == 0 && NSTAGE >= 2, "tile shape");
-    using OA = DmaOp<A_KC, BM, BK, NW>;
-    using OB = DmaOp<B_KC, BN, BK, NW>;
+    // With eight waves (two per SIMD) and a two-stage ring, the loads of a K-block are
+    // issued by half the waves, one per SIMD, alternating between the halves from block
+    // to block.  A wave that issues a burst of direct loads stalls in the issue stage
+    // until the texture path has taken them (16 clocks per instruction, 1024 per
+    // K-block and CU); with every wave issuing at once all MFMA pipes idle for that
+    // long, with one issuing wave per SIMD the other keeps its pipe busy meanwhile.
+    constexpr bool ALT = (NW == 8 && NSTAGE == 2);
+    constexpr int NWI = ALT ? NW / 2 : NW;          // waves that issue the loads of one K-block
+    using OA = DmaOp<A_KC, BM, BK, NWI>;
+    using OB = DmaOp<B_KC, BN, BK, NWI>;
     constexpr int STAGE_BYTES = OA::BYTES + OB::BYTES;
-    constexpr int L = OA::PERW + OB::PERW;          // direct loads per wave per K-block
+    constexpr int L = OA::PERW + OB::PERW;          // direct loads per issuing wave per K-block
     constexpr int NDSR = TM * (A_KC ? 1 : 2) + TN * (B_KC ? 1 : 2);
 
     extern __shared__ __attribute__((aligned(1024))) char dsm[];
@@ -189,6 +203,8 @@ gemm_dma_kernel(const GemmParams p) {
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = wave / WGN, wave_n = wave % WGN;
+    const int wi = ALT ? (wave & (NWI - 1)) : wave;   // index among the issuing waves
+    const int grp = ALT ? wave / NWI : 0;             // issues the K-blocks of this parity
 
     int pid_m, pid_n;
     tile_coords(p, pid_m, pid_n);
@@ -204,12 +220,13 @@ gemm_dma_kernel(const GemmParams p) {
     const int nkb = (kend - kdma) / BK;
     const bool interior = (m0 + BM <= p.M) && (n0 + BN <= p.N);
 
+    // An issuing group starts at the block of its parity and steps two blocks at a time.
     OA oa;
     OB ob;
-    oa.init(A, p.lda, m0, p.M, kdma, wave, lane);
-    ob.init(B, p.ldb, n0, p.N, kdma, wave, lane);
-    const int64_t a_step = A_KC ? BK : (int64_t)BK * p.lda;
-    const int64_t b_step = B_KC ? BK : (int64_t)BK * p.ldb;
+    oa.init(A, p.lda, m0, p.M, kdma + grp * BK, wi, lane);
+    ob.init(B, p.ldb, n0, p.N, kdma + grp * BK, wi, lane);
+    const int64_t a_step = (A_KC ? BK : (int64_t)BK * p.lda) * (ALT ? 2 : 1);
+    const int64_t b_step = (B_KC ? BK : (int64_t)BK * p.ldb) * (ALT ? 2 : 1);
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -240,10 +257,12 @@ gemm_dma_kernel(const GemmParams p) {
             for (int j = 0; j < TN; j++) acc[i][j] = mfma32<DT>(af[slot][i], bf[slot][j], acc[i][j]);
     };
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_void_t *)dsm;
-    auto issue_block = [&](int stage) {
+    // block: index of the K-block within the ring's sequence (decides the issuing group)
+    auto issue_block = [&](int stage, int block) {
+        if (ALT && (block & 1) != grp) return;
         const uint32_t sp = lds_base + stage * STAGE_BYTES;
-        oa.issue(sp, a_step, wave);
-        ob.issue(sp + OA::BYTES, b_step, wave);
+        oa.issue(sp, a_step, wi);
+        ob.issue(sp + OA::BYTES, b_step, wi);
     };
 
     if (krem > 0) {
@@ -261,8 +280,9 @@ gemm_dma_kernel(const GemmParams p) {
 
     // Prologue: fill the ring (NSTAGE blocks, or all of them), publish block 0.
     const int npre = min(nkb, NSTAGE);
-    for (int s = 0; s < npre; s++) issue_block(s);
-    if (npre >= NSTAGE) wait_dma_and_barrier<(NSTAGE - 1) * L>();
+    for (int s = 0; s < npre; s++) issue_block(s, s);
+    // (alternating groups: a wave has issued one block at most, so it waits for all it has)
+    if (npre >= NSTAGE && !ALT) wait_dma_and_barrier<(NSTAGE - 1) * L>();
     else wait_dma_and_barrier<0>();
     if (nkb > 0) read_frags(0, 0, 0);
 
@@ -285,7 +305,7 @@ gemm_dma_kernel(const GemmParams p) {
                 if (later >= NSTAGE - 2) wait_dma_and_barrier<(NSTAGE - 2) * L>();
                 else if (later == 1 && NSTAGE > 3) wait_dma_and_barrier<L>();
                 else wait_dma_and_barrier<0>();
-                if (kb + NSTAGE < nkb) issue_block(stage);
+                if (kb + NSTAGE < nkb) issue_block(stage, kb + NSTAGE);
             }
             if (kk == KK - 1) {
                 if (kb + 1 < nkb) read_frags(nstage, 0, nxt);
@@ -443,8 +463,10 @@ gemm_dmap_kernel(const GemmParams p) {
     constexpr int TM = WTM / 32, TN = WTN / 32;
     constexpr int KK = BK / 16;
     static_assert(WTM % 32 == 0 && WTN % 32 == 0 && KK % 2 == 0 && NSTAGE >= 2, "tile shape");
-    using OA = DmaOp<A_KC, BM, BK, NW>;
-    using OB = DmaOp<B_KC, BN, BK, NW>;
+    constexpr bool ALT = (NW == 8 && NSTAGE == 2);   // issuing waves alternate per K-block, as in gemm_dma_kernel
+    constexpr int NWI = ALT ? NW / 2 : NW;
+    using OA = DmaOp<A_KC, BM, BK, NWI>;
+    using OB = DmaOp<B_KC, BN, BK, NWI>;
     constexpr int STAGE_BYTES = OA::BYTES + OB::BYTES;
     constexpr int L = OA::PERW + OB::PERW;
     constexpr int NDSR = TM * (A_KC ? 1 : 2) + TN * (B_KC ? 1 : 2);
@@ -456,6 +478,8 @@ gemm_dmap_kernel(const GemmParams p) {
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = wave / WGN, wave_n = wave % WGN;
+    const int wi = ALT ? (wave & (NWI - 1)) : wave;
+    const int grp = ALT ? wave / NWI : 0;
     const int64_t zb = blockIdx.z;
     const uint16_t *A = p.A + zb * p.sa;
     const uint16_t *B = p.B + zb * p.sb;
@@ -550,12 +574,17 @@ gemm_dmap_kernel(const GemmParams p) {
         if (l_kb == 0) {
             const Unit q = unit_at(l_i);
             l_nkb = q.nkb;
-            oa.init(A, p.lda, q.m0, p.M, q.kbeg, wave, lane);
-            ob.init(B, p.ldb, q.n0, p.N, q.kbeg, wave, lane);
+            oa.init(A, p.lda, q.m0, p.M, q.kbeg, wi, lane);
+            ob.init(B, p.ldb, q.n0, p.N, q.kbeg, wi, lane);
         }
         const uint32_t sp = lds_base + (issued % NSTAGE) * STAGE_BYTES;
-        oa.issue(sp, a_step, wave);
-        ob.issue(sp + OA::BYTES, b_step, wave);
+        if (!ALT || (issued & 1) == grp) {
+            oa.issue(sp, a_step, wi);
+            ob.issue(sp + OA::BYTES, b_step, wi);
+        } else {
+            oa.advance(a_step);
+            ob.advance(b_step);
+        }
         issued++;
         if (++l_kb == l_nkb) {
             l_kb = 0;
@@ -672,7 +701,8 @@ gemm_dmap_kernel(const GemmParams p) {
 
     // Prologue: fill the ring, publish block 0.
     for (int s = 0; s < NSTAGE; s++) issue_next();
-    wait_blocks_and_barrier<L, NSTAGE - 1>(issued - 1);
+    // (alternating groups: a wave has issued one block at most, so it waits for all it has)
+    wait_blocks_and_barrier<L, NSTAGE - 1>(ALT ? 0 : issued - 1);
     read_frags(0, 0, 0);
 
     int c_i = 0;
