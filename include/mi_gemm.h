@@ -97,7 +97,7 @@ typedef struct {
     int32_t fallback;          /* tile used instead when this tile's preconditions fail (self: none) */
     int32_t persistent;        /* 1: a grid of resident workgroups loops over the output tiles;
                                 * 2: the same, and the tiles beyond the last whole round are cut along K into
-                                *    one equal run per workgroup (stream-K; needs the context's workspace,
+                                *    equal pieces, one per workgroup (stream-K; needs the context's workspace,
                                 *    without it the tile runs as kind 1) */
     int32_t reserved;
     char name[48];

@@ -490,12 +490,14 @@ gemm_dmap_kernel(const GemmParams p) {
     //   plain:    unit i is (K slice, tile) number pos + i * gridDim.x, slice-major (all
     //             tiles of slice 0, then slice 1, ...), so the slices of one tile are
     //             not meeting at the same moment.
-    //   stream-K: the tiles that fill whole rounds are dealt out the same way; the K-blocks
-    //             of the remaining tiles (less than one round) are cut into gridDim.x equal
-    //             contiguous runs, one per workgroup, done first.  A run covers the end of
-    //             one tile and/or the start of the next; the pieces of a tile meet in the
-    //             workspace like K slices (slot 2 * pos for a workgroup's first piece,
-    //             2 * pos + 1 for its second).
+    //   stream-K: the tiles that fill whole rounds are dealt out the same way; each of the
+    //             remaining tiles (less than one round) is cut along K into sk_pieces equal
+    //             pieces, one per workgroup, done first and piece-major like K slices, so
+    //             that the workgroups sharing an operand panel walk the same K-blocks at the
+    //             same time and keep hitting each other's lines in the L2.  (Cutting the
+    //             remaining K-blocks into runs of exactly equal length instead balances
+    //             better on paper, but then no two workgroups are at the same K offset and
+    //             every load misses: measured twice as slow.)
     const int nwg = gridDim.x;
     const int ntiles = p.grid_m * p.grid_n;
     int pos = blockIdx.x;
@@ -514,38 +516,26 @@ gemm_dmap_kernel(const GemmParams p) {
         q.n0 = (r / gsize) * BN;
         q.lin = lin;
     };
-    // stream-K bookkeeping (all zero in plain mode).  Run w covers the blocks
-    // [run_begin(w), run_begin(w + 1)) of the remaining tiles, numbered tile-major.
+    // stream-K bookkeeping (all zero in plain mode)
     const bool stream_k = STREAMK && p.stream_k;   // a stream-K tile without workspace runs plain
     const int nkb_tile = p.K / BK;
     const int full_rounds = stream_k ? p.sk_full_rounds : 0;
-    const int rem_wgs = stream_k ? p.sk_rem_wgs : 0;
-    auto run_begin = [&](int w) -> int { return w * p.sk_q + min(w, p.sk_r); };
-    int rb0 = 0, rb1 = 0, t_first = 0, rem_units = 0;
-    if (STREAMK && pos < rem_wgs) {
-        rb0 = run_begin(pos);
-        rb1 = run_begin(pos + 1);
-        t_first = rb0 / nkb_tile;
-        rem_units = (rb1 - 1) / nkb_tile - t_first + 1;
-    }
+    const int rem_tiles = stream_k ? p.sk_rem_tiles : 0;
+    const int pieces = stream_k ? p.sk_pieces : 1;
+    const int rem_units = (STREAMK && pos < rem_tiles * pieces) ? 1 : 0;
     const int n_plain = stream_k ? full_rounds : (ntiles * p.split_k - pos + nwg - 1) / nwg;
     const int my_units = rem_units + (n_plain > 0 ? n_plain : 0);
 
     auto unit_at = [&](int i) -> Unit {
         Unit q;
         if (STREAMK && i < rem_units) {
-            const int t = t_first + i;                          // tile among the remaining ones
-            const int t0 = t * nkb_tile, t1 = t0 + nkb_tile;
-            const int lo = max(rb0, t0) - t0, hi = min(rb1, t1) - t0;
+            const int piece = pos / rem_tiles, t = pos - piece * rem_tiles;
+            const int lo = piece * nkb_tile / pieces, hi = (piece + 1) * nkb_tile / pieces;
             place(full_rounds * nwg + t, q);
             q.kbeg = lo * BK;
             q.nkb = hi - lo;
-            // the runs that meet this tile belong to consecutive workgroups around this one
-            int first_w = pos, last_w = pos;
-            while (first_w > 0 && run_begin(first_w) > t0) first_w--;
-            while (last_w + 1 < rem_wgs && run_begin(last_w + 1) < t1) last_w++;
-            q.slice = pos - first_w;
-            q.nslices = last_w - first_w + 1;
+            q.slice = piece;
+            q.nslices = pieces;
             return q;
         }
         const int u = pos + (i - rem_units) * nwg;
@@ -635,21 +625,13 @@ gemm_dmap_kernel(const GemmParams p) {
         bool atomic = q.nslices > 1 || p.beta;
         if (q.nslices > 1 && p.ws != nullptr) {
             const int64_t tile_id = zb * ntiles + q.lin;
-            // Workspace slot of piece sl.  Stream-K: the piece belongs to workgroup
-            // w = pos - q.slice + sl and is that workgroup's second piece when its run
-            // started in an earlier tile.  Plain split: slices are slot planes over the tiles.
-            const int64_t all_tiles = (int64_t)ntiles * gridDim.z;
-            const int t0 = (q.lin - full_rounds * nwg) * nkb_tile;
+            // Workspace slot of piece sl: slot planes over the tiles that are cut (all of them
+            // for a plain split, the remaining ones for stream-K).
+            const int64_t plane = stream_k ? (int64_t)rem_tiles * gridDim.z : (int64_t)ntiles * gridDim.z;
+            const int64_t in_plane = stream_k ? zb * rem_tiles + (q.lin - full_rounds * nwg) : tile_id;
             const bool mine = splitk_gather<TM, TN, NW * 64>(
                 acc, p.ws, p.cnt + tile_id, q.slice, q.nslices,
-                [&](int sl) -> int64_t {
-                    if (STREAMK && stream_k) {
-                        const int w = pos - q.slice + sl;
-                        return (zb * nwg + w) * 2 + (run_begin(w) < t0 ? 1 : 0);
-                    }
-                    return (int64_t)sl * all_tiles + tile_id;
-                },
-                tid, &gather_flag);
+                [&](int sl) -> int64_t { return (int64_t)sl * plane + in_plane; }, tid, &gather_flag);
             if (!mine) return;
             add_bias = EPI_LOADS && p.bias != nullptr;
             atomic = p.beta != 0;

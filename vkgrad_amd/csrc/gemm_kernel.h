@@ -51,11 +51,11 @@ struct GemmParams {
     int xcd_remap;        // 1: renumber workgroups so neighbours share an XCD
     float *ws;            // split-K workspace (split_k * tiles * BM * BN floats) or null: add with atomics
     int *cnt;             // one arrival counter per tile, zero between launches
-    int stream_k;         // stream-K kernel only: balance the last partial round over all workgroups
+    int stream_k;         // stream-K kernel only: cut the tiles of the last, partial round along K
     // stream-K partition, computed by the host for the launched grid: whole rounds of tiles,
-    // workgroups that take a run of the remaining K-blocks, and the run length (sk_q blocks,
-    // one more for the first sk_r workgroups)
-    int sk_full_rounds, sk_rem_wgs, sk_q, sk_r;
+    // tiles left over after them, and the number of equal K pieces each of those is cut into
+    // (sk_rem_tiles * sk_pieces <= gridDim.x workgroups take one piece each)
+    int sk_full_rounds, sk_rem_tiles, sk_pieces;
 };
 
 template <int DT>
@@ -286,13 +286,20 @@ __device__ __forceinline__ bool splitk_gather(f32x16 (&acc)[TM][TN], float *ws, 
     for (int sl = 0; sl < nslices; sl++) {
         const float *src = ws + slot_of(sl) * TILE_FLOATS + tid;
 #pragma unroll
-        for (int i = 0; i < TM; i++)
+        for (int i = 0; i < TM; i++) {
+            // a row of tiles is fetched as one batch of independent loads, then added
+            float part[TN][16];
 #pragma unroll
             for (int j = 0; j < TN; j++)
 #pragma unroll
                 for (int r = 0; r < 16; r++)
-                    acc[i][j][r] += __hip_atomic_load(src + (int64_t)((i * TN + j) * 16 + r) * NTHREADS,
-                                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    part[j][r] = __hip_atomic_load(src + (int64_t)((i * TN + j) * 16 + r) * NTHREADS, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] += part[j][r];
+        }
     }
     return true;
 }

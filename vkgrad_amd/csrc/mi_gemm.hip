@@ -147,26 +147,26 @@ static bool dma_eligible(const mg_gemm_args &a, const TileDesc &t, int64_t k_per
 // {per-workgroup overhead in us, time per K-block in us} by tile and layout NN, NT, TN.
 // It only has to rank candidates; the tuner measures.
 static const float g_cost[MG_NUM_TILES][3][2] = {
-    {{8.20f, 1.735f}, {13.99f, 1.490f}, {7.02f, 1.568f}},   // 0 mm_256x256x64_w2x2
-    {{6.47f, 1.019f}, {12.43f, 0.788f}, {4.21f, 0.996f}},   // 1 mm_256x128x64_w2x2
-    {{6.57f, 0.971f}, {11.43f, 0.797f}, {4.06f, 1.035f}},   // 2 mm_128x256x64_w2x2
-    {{5.46f, 1.023f}, {7.79f, 0.812f}, {3.07f, 0.978f}},    // 3 mm_128x128x64_w2x2
-    {{2.29f, 0.570f}, {1.10f, 0.752f}, {2.00f, 0.582f}},    // 4 mm_64x64x64_w2x2
-    {{5.28f, 0.629f}, {7.41f, 0.599f}, {3.31f, 0.684f}},    // 5 mm_64x256x64_w1x4
-    {{3.38f, 0.522f}, {4.98f, 0.476f}, {3.23f, 0.533f}},    // 6 mm_32x256x64_w1x4
-    {{5.29f, 0.648f}, {4.75f, 0.660f}, {3.38f, 0.678f}},    // 7 mm_256x64x64_w4x1
-    {{3.46f, 0.555f}, {3.44f, 0.552f}, {2.97f, 0.576f}},    // 8 mm_256x32x64_w4x1
-    {{5.87f, 0.716f}, {12.93f, 0.610f}, {4.52f, 0.694f}},   // 9 mmd_256x256x32_w2x4_s4
-    {{7.02f, 1.336f}, {12.86f, 1.163f}, {4.69f, 1.275f}},   // 10 mmd_256x256x64_w2x4_s2
-    {{6.05f, 0.844f}, {6.24f, 0.827f}, {3.05f, 0.969f}},    // 11 mmd_128x128x64_w2x2_s2
-    {{5.35f, 0.843f}, {9.50f, 0.814f}, {4.11f, 0.783f}},    // 12 mmd_128x256x32_w2x2_s3
-    {{5.52f, 0.899f}, {11.10f, 0.822f}, {4.23f, 0.787f}},   // 13 mmd_256x128x32_w2x2_s3
-    {{5.22f, 0.486f}, {5.92f, 0.576f}, {3.21f, 0.460f}},    // 14 mmd_128x128x32_w2x2_s3
-    {{7.29f, 1.397f}, {6.65f, 1.446f}, {4.48f, 1.377f}},    // 15 mmp_256x256x64_w2x4_s2
-    {{7.27f, 0.809f}, {6.45f, 0.810f}, {4.21f, 0.792f}},    // 16 mmp_256x256x32_w2x4_s4
-    {{6.21f, 0.873f}, {3.06f, 1.026f}, {3.10f, 0.985f}},    // 17 mmp_128x128x64_w2x2_s2
-    {{7.29f, 1.397f}, {6.65f, 1.446f}, {4.48f, 1.377f}},    // 18 mmk_256x256x64_w2x4_s2 (as 15)
-    {{6.21f, 0.873f}, {3.06f, 1.026f}, {3.10f, 0.985f}},    // 19 mmk_128x128x64_w2x2_s2 (as 17)
+    {{6.63f, 1.813f}, {12.84f, 1.644f}, {5.81f, 1.695f}},   // 0 mm_256x256x64_w2x2
+    {{5.29f, 1.046f}, {12.32f, 0.779f}, {3.73f, 1.029f}},   // 1 mm_256x128x64_w2x2
+    {{5.21f, 0.991f}, {11.72f, 0.771f}, {3.63f, 1.042f}},   // 2 mm_128x256x64_w2x2
+    {{4.60f, 1.014f}, {7.81f, 0.781f}, {2.82f, 0.975f}},   // 3 mm_128x128x64_w2x2
+    {{1.59f, 0.581f}, {1.33f, 0.713f}, {1.76f, 0.581f}},   // 4 mm_64x64x64_w2x2
+    {{4.46f, 0.640f}, {7.40f, 0.590f}, {3.02f, 0.675f}},   // 5 mm_64x256x64_w1x4
+    {{2.79f, 0.531f}, {4.80f, 0.475f}, {2.92f, 0.534f}},   // 6 mm_32x256x64_w1x4
+    {{4.55f, 0.654f}, {4.58f, 0.660f}, {3.04f, 0.671f}},   // 7 mm_256x64x64_w4x1
+    {{2.88f, 0.565f}, {3.07f, 0.564f}, {2.65f, 0.574f}},   // 8 mm_256x32x64_w4x1
+    {{4.30f, 0.731f}, {12.88f, 0.606f}, {4.01f, 0.693f}},   // 9 mmd_256x256x32_w2x4_s4
+    {{5.69f, 1.360f}, {13.28f, 1.157f}, {4.76f, 1.246f}},   // 10 mmd_256x256x64_w2x4_s2
+    {{5.06f, 0.852f}, {6.45f, 0.792f}, {3.04f, 0.956f}},   // 11 mmd_128x128x64_w2x2_s2
+    {{4.11f, 0.856f}, {9.21f, 0.824f}, {3.90f, 0.779f}},   // 12 mmd_128x256x32_w2x2_s3
+    {{4.36f, 0.904f}, {10.94f, 0.809f}, {4.15f, 0.786f}},   // 13 mmd_256x128x32_w2x2_s3
+    {{4.18f, 0.503f}, {6.10f, 0.560f}, {3.20f, 0.459f}},   // 14 mmd_128x128x32_w2x2_s3
+    {{5.55f, 1.469f}, {6.82f, 1.473f}, {4.49f, 1.352f}},   // 15 mmp_256x256x64_w2x4_s2
+    {{5.39f, 0.852f}, {6.29f, 0.847f}, {4.06f, 0.795f}},   // 16 mmp_256x256x32_w2x4_s4
+    {{5.27f, 0.871f}, {3.25f, 0.983f}, {3.08f, 0.980f}},   // 17 mmp_128x128x64_w2x2_s2
+    {{4.81f, 2.006f}, {7.24f, 1.819f}, {3.05f, 2.002f}},   // 18 mmk_256x256x64_w2x4_s2
+    {{5.52f, 0.907f}, {4.46f, 0.944f}, {3.88f, 1.003f}},   // 19 mmk_128x128x64_w2x2_s2
 };
 
 static int wgs_per_cu(const TileDesc &t, int layout) {
@@ -178,15 +178,37 @@ static int wgs_per_cu(const TileDesc &t, int layout) {
     return w < 1 ? 1 : w;
 }
 
-// Grid of a persistent launch.  Plain: one workgroup per slot, or per unit if there are
-// fewer.  Stream-K: also when tiles are fewer than slots every slot gets a run of K-blocks,
-// as long as a run stays at least four blocks long.
+// Stream-K partition of `tiles` output tiles of `kblocks` K-blocks over a grid of at most
+// `slots` resident workgroups: whole rounds, then the remaining tiles cut into `pieces`
+// equal K pieces (at least four blocks each) so that one more, partial round fills the grid.
+struct StreamK {
+    int64_t grid;
+    int full_rounds, rem_tiles, pieces;
+};
+static StreamK stream_k_partition(int64_t tiles, int64_t kblocks, int64_t slots) {
+    StreamK s;
+    int64_t cap = kblocks / 4;
+    if (cap < 1) cap = 1;
+    if (tiles < slots) {
+        int64_t pc = slots / tiles;
+        if (pc > cap) pc = cap;
+        s.grid = tiles * pc;
+    } else {
+        s.grid = slots;
+    }
+    s.full_rounds = (int)(tiles / s.grid);
+    s.rem_tiles = (int)(tiles - (int64_t)s.full_rounds * s.grid);
+    int64_t pc = s.rem_tiles ? s.grid / s.rem_tiles : 1;
+    if (pc > cap) pc = cap;
+    s.pieces = (int)(pc < 1 ? 1 : pc);
+    return s;
+}
+
+// Grid of a persistent launch: one workgroup per slot, or per unit if there are fewer.
 static int64_t persistent_grid(const TileDesc &t, int64_t tiles, int split, int64_t kblocks, int64_t slots) {
+    if (t.persistent == 2 && split == 1) return stream_k_partition(tiles, kblocks, slots).grid;
     const int64_t units = tiles * split;
-    if (t.persistent != 2 || units >= slots) return units < slots ? units : slots;
-    int64_t g = tiles * kblocks / 4;
-    if (g < tiles) g = tiles;
-    return g < slots ? g : slots;
+    return units < slots ? units : slots;
 }
 
 // Estimated time (microseconds) of one (tile, split) choice: rounds of co-resident
@@ -199,18 +221,19 @@ static double plan_cost_us(const mg_gemm_args &a, const TileDesc &t, int split, 
     const int64_t slots = (int64_t)cus * wpc;
     double rounds = t.persistent ? (double)units / (double)slots : (double)cdiv(units, slots);
     if (t.persistent == 2) {
-        // stream-K: every workgroup gets the same number of K-blocks, plus the meeting of the pieces
+        // stream-K: whole rounds, then one round of K pieces and their meeting
         const int64_t kblocks = cdiv(a.k, t.bk);
-        const int64_t g = persistent_grid(t, gm * gn, 1, kblocks, slots);
-        const double per_wg = (double)(gm * gn) * (double)kblocks / (double)g;   // blocks per workgroup
+        const StreamK sk = stream_k_partition(gm * gn, kblocks, slots);
         const int lay2 = a.layout == MG_NN ? 0 : (a.layout == MG_NT ? 1 : 2);
-        double occ = (double)cdiv(g, cus) / wpc;
+        double occ = (double)cdiv(sk.grid, cus) / wpc;
         if (occ > 1.0) occ = 1.0;
         if (occ < 0.6) occ = 0.6;
-        double tiles_per_wg = (double)(gm * gn) / (double)g;
-        if (tiles_per_wg < 1.0) tiles_per_wg = 1.0;
-        return 1.5 + tiles_per_wg * g_cost[t.id][lay2][0] + per_wg * occ * g_cost[t.id][lay2][1] +
-               ((gm * gn) % g != 0 ? 4.0 : 0.0);
+        const double blocks = (double)sk.full_rounds * kblocks + (sk.rem_tiles ? (double)cdiv(kblocks, sk.pieces) : 0.0);
+        const double units_wg = sk.full_rounds + (sk.rem_tiles ? 1 : 0);
+        // meeting of the pieces: about 5.2 us per piece of a 256 x 256 tile, 1.4 us of a 128 x 128 one
+        const double per_piece = t.bm * t.bn > 128 * 128 ? 5.2 : 1.4;
+        return 1.5 + units_wg * g_cost[t.id][lay2][0] + blocks * occ * g_cost[t.id][lay2][1] +
+               (sk.pieces > 1 ? sk.pieces * per_piece : 0.0);
     }
     if (rounds < 1.0) rounds = 1.0;
     const int64_t resident = cdiv(units, cus) < wpc ? cdiv(units, cus) : wpc;
@@ -602,7 +625,8 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     p.ws = nullptr;
     p.cnt = nullptr;
     p.stream_k = 0;
-    p.sk_full_rounds = p.sk_rem_wgs = p.sk_q = p.sk_r = 0;
+    p.sk_full_rounds = p.sk_rem_tiles = 0;
+    p.sk_pieces = 1;
     if (pl.split_k > 1) {
         // partial tiles go through the workspace when they fit
         const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n * a.nbatch;
@@ -639,16 +663,16 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
         const int64_t slots = (int64_t)ctx->prop.multiProcessorCount * wgs_per_cu(t, a.layout);
         int64_t g = persistent_grid(t, tiles, pl.split_k, a.k / t.bk, slots);
         if (t.persistent == 2 && pl.split_k == 1) {
-            // two workspace slots per workgroup and batch; without them the tile runs as plain persistent
-            const int64_t need = 2 * g * a.nbatch * t.bm * t.bn * (int64_t)sizeof(float);
-            const int64_t rem_blocks = (tiles % g) * (a.k / t.bk);
-            if (ctx->ws && need <= ctx->ws_bytes && tiles * a.nbatch <= MG_MAX_COUNTED_TILES &&
-                rem_blocks < 0x7fffffffLL) {
+            // one workspace slot per piece; without the workspace the tile runs as plain persistent
+            const StreamK sk = stream_k_partition(tiles, a.k / t.bk, slots);
+            const int64_t need = (int64_t)sk.pieces * sk.rem_tiles * a.nbatch * t.bm * t.bn * (int64_t)sizeof(float);
+            if (sk.pieces == 1) {
+                g = tiles < slots ? tiles : slots;   // nothing to cut
+            } else if (ctx->ws && need <= ctx->ws_bytes && tiles * a.nbatch <= MG_MAX_COUNTED_TILES) {
                 p.stream_k = 1;
-                p.sk_full_rounds = (int)(tiles / g);
-                p.sk_rem_wgs = (int)(rem_blocks < g ? rem_blocks : g);
-                p.sk_q = p.sk_rem_wgs ? (int)(rem_blocks / p.sk_rem_wgs) : 0;
-                p.sk_r = p.sk_rem_wgs ? (int)(rem_blocks % p.sk_rem_wgs) : 0;
+                p.sk_full_rounds = sk.full_rounds;
+                p.sk_rem_tiles = sk.rem_tiles;
+                p.sk_pieces = sk.pieces;
                 p.ws = ctx->ws;
                 p.cnt = ctx->cnt;
             } else {

@@ -11,8 +11,8 @@
 //     P(id, BM, BN, BK, WGM, WGN, NSTAGE, fallback_id) — falls back to the
 //     one-tile-per-workgroup direct-to-LDS tile of the same shape.
 //   stream-K: the persistent kernel again, but the tiles that do not fill a whole
-//     round of the resident grid are cut along K into one equal run per workgroup
-//     (pieces meet in the context's workspace), so every CU finishes together.
+//     round of the resident grid are cut along K into equal pieces, one per workgroup
+//     (pieces meet in the context's workspace), so the last round fills the chip too.
 //     S(id, BM, BN, BK, WGM, WGN, NSTAGE, fallback_id) — falls back to the
 //     persistent tile of the same shape (no workspace, or ragged K).
 // WGM x WGN wavefronts of 64 lanes per workgroup.
