@@ -378,9 +378,6 @@ struct mg_ctx {
     int *cnt;
 };
 static const int64_t MG_MAX_COUNTED_TILES = 1 << 18;
-// Above this many bytes of partial tiles the slices add with atomics even though the
-// workspace could hold them: measured on MI355X, the gather loses once C is that large.
-static const int64_t MG_WS_AUTO_LIMIT = 96ll << 20;
 
 struct mg_graph {
     hipGraph_t graph;
@@ -631,8 +628,7 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
         // partial tiles go through the workspace when they fit
         const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n * a.nbatch;
         const int64_t need = tiles * pl.split_k * t.bm * t.bn * (int64_t)sizeof(float);
-        if (ctx->ws && need <= ctx->ws_bytes && need <= MG_WS_AUTO_LIMIT && tiles <= MG_MAX_COUNTED_TILES &&
-            !(a.flags & MG_FLAG_SPLITK_ATOMIC)) {
+        if (ctx->ws && need <= ctx->ws_bytes && tiles <= MG_MAX_COUNTED_TILES && !(a.flags & MG_FLAG_SPLITK_ATOMIC)) {
             p.ws = ctx->ws;
             p.cnt = ctx->cnt;
         }

@@ -315,7 +315,7 @@ def candidate_space(m, n, k, cus=256, nbatch=1):
         kblocks = -(-k // t["bk"])
         splits = {1}
         if groups < cus and kblocks >= 4 and t.get("persistent") != 2:   # stream-K tiles cut K themselves
-            for target in (cus, 2 * cus):
+            for target in (cus, 2 * cus, 3 * cus):
                 s = max(1, min(target // groups, kblocks // 2))
                 # the neighbours too: atomic traffic grows with the split, so the
                 # fastest one is often just below what fills the chip
