@@ -259,21 +259,23 @@ def main():
     tflops = step_flops / (dt / args.steps) / 1e12
 
     # Per-shape launch durations with HIP events on the library's stream
-    # (mg_gemm_time): best of 3 batches of back-to-back launches.
+    # (mg_gemm_time_rotating): best of 3 batches of back-to-back launches that rotate
+    # through the step's buffer sets, so a layer GEMM reads its operands from HBM as
+    # it does inside the step.
     per_shape = []
     for name, layout, m, n, k, count in gemm_list():
         mm = mm_for(layout, m, n, k)
         is_head = name.startswith("head")
-        b = head if is_head else sets[0][name.split(".")[0]]
         role = name.split(".")[1]
-        a_, b_, c_ = {"fwd": (b["x"], b["w"], b["y"]), "dX": (b["dy"], b["w"], b["dx"]),
-                      "dW": (b["dy"], b["x"], b["dw"])}[role]
+        pick = {"fwd": ("x", "w", "y"), "dX": ("dy", "w", "dx"), "dW": ("dy", "x", "dw")}[role]
+        groups = [head] if is_head else [s[name.split(".")[0]] for s in sets]
+        rot = [tuple(g[x] for x in pick) for g in groups]
         kw = {}
         if is_head and vpitch != VOCAB:
             kw = {"ldc": vpitch} if role == "fwd" else {"lda": vpitch}
-        t1 = mm(a_, b_, c_, m, n, k, **kw)
-        rep = max(1, int(0.02 / max(t1, 1e-6)))
-        sec = min(mm(a_, b_, c_, m, n, k, repeat=rep, **kw) / rep for _ in range(3))
+        t1 = mm.time_rotating(rot, m, n, k, repeat=len(rot), **kw) / len(rot)
+        rep = max(1, int(0.02 / max(t1, 1e-6)) // len(rot)) * len(rot)
+        sec = min(mm.time_rotating(rot, m, n, k, repeat=rep, **kw) / rep for _ in range(3))
         fl = 2.0 * m * n * k
         by = 2.0 * (m * k + k * n) + 4.0 * m * n
         tile, split, gm = mm.plan(m, n, k, **kw)

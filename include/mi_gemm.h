@@ -152,6 +152,12 @@ int mg_gemm(mg_ctx *ctx, const mg_gemm_args *args);
  * events on the context's stream instead of host wall clock.  Launches the GEMM
  * `repeat` times back to back, waits, and returns the total seconds. */
 int mg_gemm_time(mg_ctx *ctx, const mg_gemm_args *args, int repeat, double *seconds);
+/* The same over `nargs` (1..64) argument sets used in turn: launch i runs
+ * args[i % nargs].  With operand sets that together exceed the 256 MB last-level
+ * cache, every launch finds its operands in HBM, as a training step does; the
+ * reference times a shape on one set of buffers (kernels.py:433-447), which on
+ * this chip would time small shapes out of cache. */
+int mg_gemm_time_rotating(mg_ctx *ctx, const mg_gemm_args *args, int nargs, int repeat, double *seconds);
 /* CONFIGS — kernels.py:326-331: the tile table the tuner walks. */
 int mg_tile_count(void);
 int mg_tile_info(int id, mg_tile *out);

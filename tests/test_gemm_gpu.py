@@ -231,6 +231,40 @@ def test_stream_k_tiles_exact(dev, layout):
         assert np.array_equal(got, got2)
 
 
+def test_timing_over_rotating_operand_sets(dev):
+    """The rotating timer launches argument set i % nsets on launch i: after seven
+    launches over three sets with different integer operands, every set's C holds
+    its own exact product (beta = 0 overwrites the poison), and the time is positive."""
+    from vkgrad_amd.kernels import Matmul
+    from vkgrad_amd.vk import VkError
+    m, n, k = 200, 136, 320
+    mm = Matmul(dev, trans_b=True, dtype="f16")
+    sets, refs = [], []
+    try:
+        for s in range(3):
+            a, b = O.make_operands(m, n, k, False, True, "f16", 40 + s, integer=True)
+            bias = np.arange(n, dtype=np.float32) - s
+            ba, bb, bc, bz = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), \
+                dev.buffer(m * n * 4, "device"), dev.buffer(n * 4, "device")
+            ba.upload(a); bb.upload(b); bz.upload(bias)
+            bc.upload(np.full((m, n), np.nan, np.float32))
+            sets.append((ba, bb, bc, bz))
+            refs.append(O.ref_gemm(a, b, False, True, "f16", bias, None))
+        sec = mm.time_rotating(sets, m, n, k, repeat=7)
+        assert sec > 0
+        for s in range(3):
+            assert np.array_equal(sets[s][2].download(np.float32, (m, n)), refs[s]), f"set {s}"
+        with pytest.raises(VkError):
+            mm.time_rotating([], m, n, k, repeat=1)
+        with pytest.raises(VkError):
+            mm.time_rotating(sets, m, n, k, repeat=0)
+    finally:
+        mm.destroy()
+        for st in sets:
+            for x in st:
+                x.destroy()
+
+
 def test_wrong_layout_fails(dev):
     """Negative control (idea: test_hf_gpt2.py:129-136): a square operand read
     with the wrong layout passes every shape check and must fail on values."""

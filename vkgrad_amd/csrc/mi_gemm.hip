@@ -715,6 +715,31 @@ int mg_gemm_time(mg_ctx *ctx, const mg_gemm_args *args, int repeat, double *seco
     return MG_OK;
 }
 
+int mg_gemm_time_rotating(mg_ctx *ctx, const mg_gemm_args *args, int nargs, int repeat, double *seconds) {
+    if (!ctx || !args || !seconds) return fail(MG_ERR_ARG, "mg_gemm_time_rotating: NULL argument");
+    if (nargs < 1 || nargs > 64) return fail(MG_ERR_ARG, "mg_gemm_time_rotating: nargs must be 1..64");
+    if (repeat < 1) return fail(MG_ERR_ARG, "mg_gemm_time_rotating: repeat must be >= 1");
+    if (ctx->capturing)
+        return fail(MG_ERR_STATE, "mg_gemm_time_rotating: not allowed while a graph is being recorded");
+    Plan pl[64];
+    for (int i = 0; i < nargs; i++) {
+        int rc = check_args(&args[i]);
+        if (rc != MG_OK) return rc;
+        pick_plan(args[i], ctx->prop.multiProcessorCount, pl[i]);
+    }
+    HIP_TRY(hipEventRecord(ctx->ev0, ctx->stream));
+    for (int i = 0; i < repeat; i++) {
+        int rc = enqueue_gemm(ctx, &args[i % nargs], pl[i % nargs]);
+        if (rc != MG_OK) return rc;
+    }
+    HIP_TRY(hipEventRecord(ctx->ev1, ctx->stream));
+    HIP_TRY(hipEventSynchronize(ctx->ev1));
+    float ms = 0.f;
+    HIP_TRY(hipEventElapsedTime(&ms, ctx->ev0, ctx->ev1));
+    *seconds = (double)ms * 1e-3;
+    return MG_OK;
+}
+
 int mg_graph_begin(mg_ctx *ctx) {
     if (!ctx) return fail(MG_ERR_ARG, "mg_graph_begin: ctx is NULL");
     if (ctx->capturing) return fail(MG_ERR_STATE, "mg_graph_begin: a graph is already being recorded");

@@ -162,6 +162,20 @@ class Matmul:
         _check(lib.mg_gemm_time(ctx, C.byref(ga), int(repeat), C.byref(dt)), self.name)
         return dt.value
 
+    def time_rotating(self, sets, m, n, k, repeat=1, nbatch=1, strides=(0, 0, 0), *, accumulate=False,
+                      lda=None, ldb=None, ldc=None):
+        """Seconds for `repeat` back-to-back launches that take their buffers from
+        `sets` in turn; each set is (a, b, c) or (a, b, c, bias).  Enough sets to
+        overflow the last-level cache make every launch read its operands from HBM."""
+        arr = (L.GemmArgs * len(sets))()
+        for i, st in enumerate(sets):
+            bias = st[3] if len(st) > 3 else None
+            arr[i] = self._args(st[0], st[1], st[2], m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc)
+        dt = C.c_double()
+        _check(self.dev._lib.mg_gemm_time_rotating(self.dev._ctx, arr, len(sets), int(repeat), C.byref(dt)),
+               self.name)
+        return dt.value
+
     def enqueue(self, a, b, c, m, n, k, nbatch=1, strides=(0, 0, 0), *, bias=None,
                 accumulate=False, lda=None, ldb=None, ldc=None):
         """Launch without waiting (the stream keeps order); for pipelined callers."""
@@ -296,6 +310,18 @@ def _repeat_for(t_one):
     return max(1, int(min(_MEASURE_S, _SUBMIT_CAP_S) / max(t_one, 1e-7)))
 
 
+LAST_LEVEL_CACHE_BYTES = 256 << 20
+
+
+def buffer_sets_for(footprint):
+    """How many operand sets a timing loop rotates through: one when a single set
+    already overflows the last-level cache twice over, otherwise enough that a
+    rotation spans three cache sizes (3 to 8 sets)."""
+    if footprint >= 2 * LAST_LEVEL_CACHE_BYTES:
+        return 1
+    return max(3, min(8, -(-3 * LAST_LEVEL_CACHE_BYTES // max(1, footprint))))
+
+
 def candidate_space(m, n, k, cus=256, nbatch=1):
     """(tile, split_k) pairs worth timing for a shape: every tile whose padding
     waste is tolerable, with K splits that bring an under-filled grid up to
@@ -356,20 +382,26 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
     ea, eb, ec = (k if trans_a else m) * pa, (n if trans_b else k) * pb, m * pc   # elements per matrix
     strides = (ea, eb, ec)
     call = dict(nbatch=nb, strides=strides) if batched else {}
-    bufs = None
+    sets = None
     if timer is None:
         warmup(dev)
-        bufs = (dev.buffer(nb * ea * 2, "device"), dev.buffer(nb * eb * 2, "device"),
-                dev.buffer(nb * ec * 4, "device"))
+        footprint = nb * (2 * (ea + eb) + 4 * ec)
         K = make_kernels(dev, dtype)
-        # random operands: zeros or garbage bit patterns misstate the timing (data
-        # toggling sets MFMA power and with it the clock)
-        K["fill_uniform16"]([bufs[0]], nb * ea, 1)
-        K["fill_uniform16"]([bufs[1]], nb * eb, 2)
+        sets = []
+        for s in range(buffer_sets_for(footprint)):
+            st = (dev.buffer(nb * ea * 2, "device"), dev.buffer(nb * eb * 2, "device"),
+                  dev.buffer(nb * ec * 4, "device"))
+            sets.append(st)
+            # random operands: zeros or garbage bit patterns misstate the timing (data
+            # toggling sets MFMA power and with it the clock)
+            K["fill_uniform16"]([st[0]], nb * ea, 1 + 2 * s)
+            K["fill_uniform16"]([st[1]], nb * eb, 2 + 2 * s)
 
         def timer(mm, repeat):
-            return mm(bufs[0], bufs[1], bufs[2], m, n, k, repeat=repeat, accumulate=accumulate,
-                      lda=lda, ldb=ldb, ldc=ldc, **call)
+            # operands rotate through sets that together overflow the last-level cache:
+            # a layer of a training step finds its operands in HBM, not in cache
+            return mm.time_rotating(sets, m, n, k, repeat=repeat, accumulate=accumulate,
+                                    lda=lda, ldb=ldb, ldc=ldc, **call)
 
     try:
         # a K split is timed both ways: slices meeting in the workspace, and adding atomically
@@ -385,7 +417,7 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
             best_t = {id(x): float("inf") for x in mms}
             for _ in range(reps):
                 for x in mms:   # round-robin: drift spreads evenly over candidates
-                    r = _repeat_for(warm[id(x)])
+                    r = max(_repeat_for(warm[id(x)]), len(sets) if sets else 1)
                     best_t[id(x)] = min(best_t[id(x)], timer(x, r) / r)
             return best_t
 
@@ -422,8 +454,8 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
                       dtype=dtype, split_k=best["split_k"], group_m=best["group_m"],
                       atomic_split=best["atomic_split"]), best
     finally:
-        if bufs:
-            for x in bufs:
+        for st in sets or ():
+            for x in st:
                 x.destroy()
 
 
