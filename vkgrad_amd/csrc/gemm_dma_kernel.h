@@ -733,15 +733,9 @@ template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTA
 hipError_t launch_gemm_dma(const GemmParams &p, dim3 grid, hipStream_t stream) {
     using TT = DmaTraits<LAYOUT, BM, BN, BK, WGM, WGN, NSTAGE>;
     auto kern = gemm_dma_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, NSTAGE>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        if (TT::LDS_BYTES > 65536) {
-            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               TT::LDS_BYTES);
-            if (e != hipSuccess) return e;
-        }
-        attr_done = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};
+    hipError_t e = allow_dynamic_lds((const void *)kern, TT::LDS_BYTES, lds_allowed);
+    if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, grid, dim3(TT::NTHREADS), TT::LDS_BYTES, stream, p);
     return hipGetLastError();
 }
@@ -751,15 +745,9 @@ template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTA
 hipError_t launch_gemm_dmap(const GemmParams &p, dim3 grid, hipStream_t stream) {
     using TT = DmaTraits<LAYOUT, BM, BN, BK, WGM, WGN, NSTAGE>;
     auto kern = gemm_dmap_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, NSTAGE, EPI_LOADS, STREAMK>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        if (TT::LDS_BYTES > 65536) {
-            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               TT::LDS_BYTES);
-            if (e != hipSuccess) return e;
-        }
-        attr_done = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};
+    hipError_t e = allow_dynamic_lds((const void *)kern, TT::LDS_BYTES, lds_allowed);
+    if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, grid, dim3(TT::NTHREADS), TT::LDS_BYTES, stream, p);
     return hipGetLastError();
 }

@@ -16,6 +16,7 @@
 // the MFMAs of block t and written to the other LDS stage afterwards, so there
 // is one workgroup barrier per K-block.
 #pragma once
+#include <atomic>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -535,19 +536,27 @@ gemm_kernel(const GemmParams p) {
 
 typedef hipError_t (*launch_fn)(const GemmParams &, dim3 grid, hipStream_t);
 
+// More than 64 KiB of dynamic LDS has to be allowed per kernel and per device; `done`
+// remembers, one bit per device index, where that has happened for the calling launcher.
+inline hipError_t allow_dynamic_lds(const void *kern, int bytes, std::atomic<uint64_t> &done) {
+    if (bytes <= 65536) return hipSuccess;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+    return e;
+}
+
 template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, bool GENERAL>
 hipError_t launch_gemm(const GemmParams &p, dim3 grid, hipStream_t stream) {
     using TT = TileTraits<LAYOUT, BM, BN, BK, WGM, WGN>;
     auto kern = gemm_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, GENERAL>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        if (TT::LDS_BYTES > 65536) {
-            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               TT::LDS_BYTES);
-            if (e != hipSuccess) return e;
-        }
-        attr_done = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};
+    hipError_t e = allow_dynamic_lds((const void *)kern, TT::LDS_BYTES, lds_allowed);
+    if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, grid, dim3(TT::NTHREADS), TT::LDS_BYTES, stream, p);
     return hipGetLastError();
 }

@@ -87,14 +87,15 @@ def algorithmic_bytes(c):
 
 
 class Runner:
-    def __init__(self, tune=False):
+    def __init__(self, tune=False, warm=True):
         from . import kernels
         from .vk import Device
         self.K = kernels
         self.dev = Device()
         self.tune = tune
         self.fill = {}
-        kernels.warmup(self.dev, 2.0)
+        if warm:
+            kernels.warmup(self.dev, 2.0)
 
     def _fill(self, dtype, buf, n, seed):
         if dtype not in self.fill:
@@ -179,7 +180,7 @@ def main(argv=None):
     ap.add_argument("--trace-pass", type=int, default=0, metavar="N",
                     help="no timing: launch every case N times in listed order (for a kernel trace)")
     args = ap.parse_args(argv)
-    r = Runner(tune=args.tune)
+    r = Runner(tune=args.tune, warm=not args.trace_pass)
     rows = []
     print(f"# {args.config} on {r.dev.name}", flush=True)
     if args.trace_pass:
