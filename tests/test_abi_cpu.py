@@ -116,9 +116,17 @@ def test_tile_table(lib):
         t = L.Tile()
         assert lib.mg_tile_info(i, C.byref(t)) == L.MG_OK
         assert t.id == i and t.threads == t.waves_m * t.waves_n * 64
-        assert t.bm % (32 * t.waves_m) == 0 and t.bn % (32 * t.waves_n) == 0
         assert t.lds_bytes <= 160 * 1024
         assert 0 <= t.fallback < n
+        seen.add(t.name)
+        if t.name.startswith(b"mv_"):
+            # the skinny-M streaming tile uses no matrix cores and no LDS; what it
+            # cannot run goes to a register-staged tile
+            fb = L.Tile()
+            lib.mg_tile_info(t.fallback, C.byref(fb))
+            assert t.lds_bytes == 0 and fb.stages == 0 and fb.fallback == fb.id
+            continue
+        assert t.bm % (32 * t.waves_m) == 0 and t.bn % (32 * t.waves_n) == 0
         # the fallback chain ends at a register-staged tile of the same BM x BN
         fb, hops = t, 0
         while fb.stages:
@@ -128,11 +136,16 @@ def test_tile_table(lib):
             fb, hops = nxt, hops + 1
             assert hops <= 3
         assert fb.fallback == fb.id and not fb.persistent
-        seen.add(t.name)
     assert len(seen) == n
     assert lib.mg_tile_info(n, C.byref(L.Tile())) == L.MG_ERR_ARG
     assert lib.mg_tile_fits(0, C.byref(good_args())) == 1
     assert lib.mg_tile_fits(n, C.byref(good_args())) == 0
+
+
+def tile_name(lib, i):
+    t = L.Tile()
+    lib.mg_tile_info(i, C.byref(t))
+    return t.name.decode()
 
 
 def pick(lib, cus=256, **kw):
@@ -163,6 +176,17 @@ def test_picker_properties(lib):
     # tiny problems still get a plan
     info, split, _ = pick(lib, m=1, n=1, k=1, lda=1, ldb=1, ldc=1)
     assert split == 1
+    # the skinny-M streaming tile runs NT with at most 4 rows over K <= 2048 and hands
+    # everything else to its fallback
+    mv = next(i for i in range(lib.mg_tile_count()) if tile_name(lib, i).startswith("mv_"))
+    info, split, _ = pick(lib, layout=L.MG_NT, m=3, n=50257, k=768, lda=768, ldb=768, ldc=50257, tile=mv)
+    assert info.id == mv and split == 1
+    for kw in (dict(layout=L.MG_NT, m=5, n=4096, k=768, lda=768, ldb=768, ldc=4096),
+               dict(layout=L.MG_NT, m=1, n=4096, k=4096, lda=4096, ldb=4096, ldc=4096),
+               dict(layout=L.MG_NT, m=4, n=4096, k=772, lda=772, ldb=772, ldc=4096),
+               dict(layout=L.MG_NN, m=4, n=4096, k=768, lda=768, ldb=4096, ldc=4096)):
+        info, _, _ = pick(lib, tile=mv, **kw)
+        assert not info.name.startswith(b"mv_"), kw
 
 
 # ---------------------------------------------------------------------------

@@ -13,12 +13,14 @@ namespace mg {
 #define P(id, bm, bn, bk, wgm, wgn, ns, fb)                          \
     {launch_gemm_dmap<L_NT, D_F16, bm, bn, bk, wgm, wgn, ns, false, false>, \
      launch_gemm_dmap<L_NT, D_F16, bm, bn, bk, wgm, wgn, ns, true, false>},
+#define G(id, bm, bn, bk, fb) {nullptr, nullptr},   // launched through gemv_table
 #define S(id, bm, bn, bk, wgm, wgn, ns, fb)                                \
     {launch_gemm_dmap<L_NT, D_F16, bm, bn, bk, wgm, wgn, ns, false, true>, \
      launch_gemm_dmap<L_NT, D_F16, bm, bn, bk, wgm, wgn, ns, true, true>},
-launch_fn launch_table_nt_f16[MG_NUM_TILES][2] = {MG_TILE_LIST(V, D, P, S)};
+launch_fn launch_table_nt_f16[MG_NUM_TILES][2] = {MG_TILE_LIST(V, D, P, S, G)};
 #undef V
 #undef D
 #undef P
 #undef S
+#undef G
 }  // namespace mg

@@ -10,6 +10,7 @@
 #include <new>
 
 #include "gemm_kernel.h"
+#include "gemv_kernel.h"
 #include "mi_gemm.h"
 #include "tiles.h"
 
@@ -46,16 +47,19 @@ struct TileDesc {
     int nstage;     // 0: register-staged kernel; >0: direct-to-LDS ring depth
     int fallback;   // tile of the same BM x BN with weaker preconditions (self: none)
     int persistent; // 1: grid of resident workgroups looping over tiles; 2: the same with stream-K balancing
+    int gemv;       // 1: the skinny-M streaming kernel (no matrix cores), NT layout only
 };
-#define V(id, bm, bn, bk, wgm, wgn) {id, bm, bn, bk, wgm, wgn, 0, id, 0},
-#define D(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 0},
-#define P(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 1},
-#define S(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 2},
-static const TileDesc g_tiles[MG_NUM_TILES] = {MG_TILE_LIST(V, D, P, S)};
+#define V(id, bm, bn, bk, wgm, wgn) {id, bm, bn, bk, wgm, wgn, 0, id, 0, 0},
+#define D(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 0, 0},
+#define P(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 1, 0},
+#define S(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 2, 0},
+#define G(id, bm, bn, bk, fb) {id, bm, bn, bk, 1, GEMV_WAVES, 0, fb, 0, 1},
+static const TileDesc g_tiles[MG_NUM_TILES] = {MG_TILE_LIST(V, D, P, S, G)};
 #undef V
 #undef D
 #undef P
 #undef S
+#undef G
 
 static thread_local char g_err[512] = "";
 
@@ -89,6 +93,7 @@ static launch_fn (*table_for(int layout, int dtype))[2] {
 }
 
 static int lds_bytes_for(const TileDesc &t, int layout) {
+    if (t.gemv) return 0;
     if (t.nstage > 0) return t.nstage * (t.bm + t.bn) * t.bk * 2;
     const bool a_kc = layout != MG_TN, b_kc = layout == MG_NT;
     const int a = a_kc ? t.bm * (t.bk + 8) : t.bk * (t.bm + 32);
@@ -118,7 +123,28 @@ struct Plan {
 // Preconditions of the direct-to-LDS kernels (gemm_dma_kernel.h): aligned bases
 // and pitches, K slices that are multiples of BK (the last may be ragged), and
 // row pitches that cover the 16-byte chunk straddling a ragged edge.
+// The skinny-M kernel holds MP >= M rows of A (1, 2 or 4) over NCH >= K / 512 chunks
+// (1, 2 or 4) in registers and reads 16-byte pieces of both operands.
+static bool gemv_shape(const mg_gemm_args &a, int *mp_log2, int *nch_log2) {
+    if (a.m > 4 || a.k > 2048) return false;
+    int lm = 0, lc = 0;
+    while ((1 << lm) < a.m) lm++;
+    while ((512 << lc) < a.k) lc++;
+    if (mp_log2) *mp_log2 = lm;
+    if (nch_log2) *nch_log2 = lc;
+    return true;
+}
+static bool gemv_eligible(const mg_gemm_args &a, int split) {
+    if (a.layout != MG_NT || split > 1) return false;
+    if (!gemv_shape(a, nullptr, nullptr)) return false;
+    if (((uintptr_t)a.a | (uintptr_t)a.b) & 15) return false;
+    if ((a.lda | a.ldb | a.k) & 7) return false;
+    if (a.nbatch > 1 && ((a.sa | a.sb) & 7)) return false;
+    return true;
+}
+
 static bool dma_eligible(const mg_gemm_args &a, const TileDesc &t, int64_t k_per_split, int split) {
+    if (t.gemv) return gemv_eligible(a, split);
     if (t.nstage == 0) return true;
     const bool a_kc = a.layout != MG_TN, b_kc = a.layout == MG_NT;
     if (((uintptr_t)a.a | (uintptr_t)a.b) & 15) return false;
@@ -167,9 +193,11 @@ static const float g_cost[MG_NUM_TILES][3][2] = {
     {{5.27f, 0.871f}, {3.25f, 0.983f}, {3.08f, 0.980f}},   // 17 mmp_128x128x64_w2x2_s2
     {{4.81f, 2.006f}, {7.24f, 1.819f}, {3.05f, 2.002f}},   // 18 mmk_256x256x64_w2x4_s2
     {{5.52f, 0.907f}, {4.46f, 0.944f}, {3.88f, 1.003f}},   // 19 mmk_128x128x64_w2x2_s2
+    {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}},                     // 20 mv_8x64x512 (priced by bytes, see plan_cost_us)
 };
 
 static int wgs_per_cu(const TileDesc &t, int layout) {
+    if (t.gemv) return 8;
     const int by_lds = 163840 / lds_bytes_for(t, layout);
     const int acc_regs = t.bm * t.bn / (t.wgm * t.wgn * 64);          // per lane
     const int waves_per_simd = acc_regs > 128 ? 1 : (acc_regs > 64 ? 2 : 4);
@@ -215,6 +243,12 @@ static int64_t persistent_grid(const TileDesc &t, int64_t tiles, int split, int6
 // workgroups, each paying its overhead plus its K-blocks; a CU that holds fewer
 // workgroups than it could runs each of them faster, down to a latency floor.
 static double plan_cost_us(const mg_gemm_args &a, const TileDesc &t, int split, int cus) {
+    if (t.gemv) {
+        // a stream over B at about 5 TB/s once enough wavefronts are in flight, plus the
+        // multiply-adds, which grow with the rows of A
+        const double bytes = 2.0 * ((double)a.m * a.k + (double)a.k * a.n) * a.nbatch + 4.0 * a.m * a.n * a.nbatch;
+        return 2.0 + 0.7 * a.m + bytes / 5.4e6 * (1.0 + 0.12 * (a.m - 1));
+    }
     const int64_t gm = cdiv(a.m, t.bm), gn = cdiv(a.n, t.bn);
     const int64_t units = gm * gn * (int64_t)a.nbatch * split;
     const int wpc = wgs_per_cu(t, a.layout);
@@ -251,7 +285,7 @@ static void finish_plan(const mg_gemm_args &a, int tile, int split, Plan &pl) {
     int64_t kblocks = cdiv(a.k, d->bk);
     if (split > kblocks) split = (int)kblocks;
     if (split < 1) split = 1;
-    if (d->persistent == 2) split = 1;
+    if (d->persistent == 2 || d->gemv) split = 1;
     int64_t kb_per = cdiv(kblocks, split);
     split = (int)cdiv(kblocks, kb_per);   // no empty slices
     while (!dma_eligible(a, *d, kb_per * d->bk, split) && d->fallback != tile) {
@@ -559,7 +593,9 @@ int mg_tile_info(int id, mg_tile *out) {
     out->threads = t.wgm * t.wgn * 64;
     out->lds_bytes = lds_bytes_for(t, MG_NT);
     out->min_m = 1;
-    if (t.persistent)
+    if (t.gemv)
+        snprintf(out->name, sizeof(out->name), "mv_%dx%dx%d", t.bm, t.bn, t.bk);
+    else if (t.persistent)
         snprintf(out->name, sizeof(out->name), "%s_%dx%dx%d_w%dx%d_s%d", t.persistent == 2 ? "mmk" : "mmp", t.bm, t.bn, t.bk,
                  t.wgm, t.wgn, t.nstage);
     else if (t.nstage > 0)
@@ -617,6 +653,20 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     p.k_per_split = pl.k_per_split;
     p.xcd_remap = pl.xcd_remap;
     if ((int64_t)pl.grid_m * pl.grid_n > 0x7fffffffLL) return fail(MG_ERR_ARG, "mg_gemm: grid too large");
+    if (t.gemv) {
+        int lm = 0, lc = 0;
+        if (!gemv_eligible(a, pl.split_k) || !gemv_shape(a, &lm, &lc) || !gemv_table[a.dtype][lm][lc])
+            return fail(MG_ERR_STATE, "mg_gemm: the skinny-M tile cannot run this call");
+        GemvParams g;
+        g.A = p.A; g.B = p.B; g.C = p.C; g.bias = p.bias;
+        g.lda = p.lda; g.ldb = p.ldb; g.ldc = p.ldc;
+        g.sa = p.sa; g.sb = p.sb; g.sc = p.sc;
+        g.M = p.M; g.N = p.N; g.K = p.K; g.beta = p.beta;
+        const dim3 grid((unsigned)cdiv(a.n, GEMV_ROWS_PER_WG), 1, (unsigned)a.nbatch);
+        hipError_t e = gemv_table[a.dtype][lm][lc](g, grid, ctx->stream);
+        if (e != hipSuccess) return hip_fail(e, "mg_gemm: kernel launch");
+        return MG_OK;
+    }
     if (lds_bytes_for(t, a.layout) > (int)ctx->prop.maxSharedMemoryPerMultiProcessor)
         return fail(MG_ERR_ARG, "mg_gemm: tile %d needs %d bytes of LDS", pl.tile, lds_bytes_for(t, a.layout));
     p.ws = nullptr;

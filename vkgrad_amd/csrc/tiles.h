@@ -15,10 +15,15 @@
 //     (pieces meet in the context's workspace), so the last round fills the chip too.
 //     S(id, BM, BN, BK, WGM, WGN, NSTAGE, fallback_id) — falls back to the
 //     persistent tile of the same shape (no workspace, or ragged K).
+//   skinny-M stream (gemv_kernel.h): NT layout with at most 4 rows of A and K <= 2048;
+//     no matrix cores, B is read once as it lies in memory.
+//     G(id, BM, BN, BK, fallback_id) — BM rows of A at most, BN output columns per
+//     workgroup, BK elements of K per register chunk; falls back to a skinny
+//     register-staged tile.
 // WGM x WGN wavefronts of 64 lanes per workgroup.
 #pragma once
 
-#define MG_TILE_LIST(V, D, P, S)   \
+#define MG_TILE_LIST(V, D, P, S, G) \
     V(0, 256, 256, 64, 2, 2)       \
     V(1, 256, 128, 64, 2, 2)       \
     V(2, 128, 256, 64, 2, 2)       \
@@ -38,6 +43,7 @@
     P(16, 256, 256, 32, 2, 4, 4, 9) \
     P(17, 128, 128, 64, 2, 2, 2, 11) \
     S(18, 256, 256, 64, 2, 4, 2, 15) \
-    S(19, 128, 128, 64, 2, 2, 2, 17)
+    S(19, 128, 128, 64, 2, 2, 2, 17) \
+    G(20, 4, 64, 512, 4)
 
-#define MG_NUM_TILES 20
+#define MG_NUM_TILES 21

@@ -322,7 +322,13 @@ def buffer_sets_for(footprint):
     return max(3, min(8, -(-3 * LAST_LEVEL_CACHE_BYTES // max(1, footprint))))
 
 
-def candidate_space(m, n, k, cus=256, nbatch=1):
+def skinny_stream_fits(m, k, layout):
+    """The skinny-M streaming tile (name mv_*): NT layout, at most 4 rows of A and
+    K <= 2048 in whole 8-element pieces."""
+    return layout == L.MG_NT and m <= 4 and k <= 2048 and k % 8 == 0
+
+
+def candidate_space(m, n, k, cus=256, nbatch=1, layout=None):
     """(tile, split_k) pairs worth timing for a shape: every tile whose padding
     waste is tolerable, with K splits that bring an under-filled grid up to
     about one or two workgroups per CU."""
@@ -330,12 +336,13 @@ def candidate_space(m, n, k, cus=256, nbatch=1):
         gm, gn = -(-m // t["bm"]), -(-n // t["bn"])
         return (m * n) / (gm * t["bm"] * gn * t["bn"])
 
+    tiled = [t for t in CONFIGS if not t["name"].startswith("mv_")]
     # skinny problems waste most of every tile: keep the tiles that waste least
-    floor = min(0.45, 0.7 * max(useful_of(t) for t in CONFIGS))
-    out = []
-    for t in CONFIGS:
+    floor = min(0.45, 0.45 * max(useful_of(t) for t in tiled))
+    out = [(t["id"], 1) for t in CONFIGS if t["name"].startswith("mv_") and skinny_stream_fits(m, k, layout)]
+    for t in tiled:
         gm, gn = -(-m // t["bm"]), -(-n // t["bn"])
-        if useful_of(t) < floor and len(CONFIGS) > 1:
+        if useful_of(t) < floor and len(tiled) > 1:
             continue
         groups = gm * gn * nbatch
         kblocks = -(-k // t["bk"])
@@ -407,7 +414,8 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
         # a K split is timed both ways: slices meeting in the workspace, and adding atomically
         cands = [Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=t, dtype=dtype,
                         split_k=s, group_m=0, atomic_split=at)
-                 for t, s in candidate_space(m, n, k, getattr(dev, "compute_units", 256), nb)
+                 for t, s in candidate_space(m, n, k, getattr(dev, "compute_units", 256), nb,
+                                             layout_of(trans_a, trans_b))
                  for at in ((False, True) if s > 1 else (False,))]
         if not cands:
             raise VkError(f"no matmul config fits {m}x{n}x{k}")
