@@ -193,7 +193,7 @@ static const float g_cost[MG_NUM_TILES][3][2] = {
     {{5.27f, 0.871f}, {3.25f, 0.983f}, {3.08f, 0.980f}},   // 17 mmp_128x128x64_w2x2_s2
     {{4.81f, 2.006f}, {7.24f, 1.819f}, {3.05f, 2.002f}},   // 18 mmk_256x256x64_w2x4_s2
     {{5.52f, 0.907f}, {4.46f, 0.944f}, {3.88f, 1.003f}},   // 19 mmk_128x128x64_w2x2_s2
-    {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}},                     // 20 mv_8x64x512 (priced by bytes, see plan_cost_us)
+    {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}},                     // 20 mv_4x64x512 (priced by bytes, see plan_cost_us)
 };
 
 static int wgs_per_cu(const TileDesc &t, int layout) {
