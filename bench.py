@@ -7,7 +7,10 @@ proj 768->768, MLP 768->3072->768, plus the tied LM head 768->50257; for every
 linear the forward, dX and dW products (147 GEMMs, 6.07 TFLOP), bf16 inputs,
 fp32 accumulate and fp32 outputs, synthetic operands already resident in HBM.
 Weights are stored out x in (the tied-head convention), so the kernel layouts
-are NT forward, NN dX, TN dW.
+are NT forward, NN dX, TN dW.  Every GEMM runs behind the previous one;
+--overlap-dw runs the forward pass first and then the backward pass with the dW
+GEMMs on the library's second stream beside the dX chain (measured 1-2 % slower
+for the whole step).
 
 Prints ONE JSON line: whole-step TFLOP/s, the MFMA roofline of the dominant
 GEMM measured with HIP events on the library's stream, and the numpy oracle
@@ -127,6 +130,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--eager", action="store_true", help="enqueue GEMMs one by one instead of replaying a graph")
+    ap.add_argument("--overlap-dw", action="store_true",
+                    help="forward pass, then the backward pass with the dW GEMMs of the layers on the library's "
+                         "second stream beside the dX chain; default: every GEMM behind the previous one on one "
+                         "stream (forward, dX, dW per linear), which measured 1-2 %% faster for the whole step")
     ap.add_argument("--dense-head", action="store_true",
                     help="row pitch of logits/dlogits = 50257 exactly (rows then start at odd addresses) instead of "
                          "the next multiple of 64")
@@ -234,14 +241,52 @@ def main():
         dev.destroy()
         return
 
+    # Order of one step.  Default: forward, dX, dW of each linear in turn, every GEMM
+    # behind the previous one.
+    # --overlap-dw: the forward pass (layer 0 .. 11, LM head), then the backward pass from
+    # the head down; dW of a linear depends on nothing that follows it
+    # (autograd.py:218-227), so the dW GEMMs of a layer go to the library's second stream
+    # once that layer's dX chain is done and overlap the next layer's dX chain; the
+    # streams join at the end of the step.
+    # schedule entries: ("gemm", call, on_side_stream) | ("fork",) | ("join",)
+    per_linear = [calls[i:i + 3] for i in range(0, len(calls), 3)]     # (fwd, dX, dW) per linear, head last
+    if not args.overlap_dw:
+        schedule = [("gemm", c, False) for c in calls]
+    else:
+        schedule = [("gemm", fwd, False) for fwd, _, _ in per_linear]
+        # backward: groups of linears from the top down (the LM head, then layer 11 .. 0);
+        # the dW GEMMs of a group go to the side stream when the group's dX chain is done
+        # (all their operands are complete then) and run beside the next group's dX chain
+        # (the LM head's two products stay on the main stream: each fills the chip with
+        # resident workgroups and two such kernels only take CUs from each other)
+        schedule += [("gemm", per_linear[-1][1], False), ("gemm", per_linear[-1][2], False)]
+        groups = [per_linear[l * len(LINEARS):(l + 1) * len(LINEARS)][::-1] for l in reversed(range(LAYERS))]
+        for g in groups:
+            schedule += [("gemm", dx, False) for _, dx, _ in g]
+            schedule.append(("fork",))
+            schedule += [("gemm", dw, True) for _, _, dw in g]
+        schedule.append(("join",))
+
     if args.eager:
         def run_step():
-            for mm, a, b, c, m, n, k, kw in calls:
-                mm.enqueue(a, b, c, m, n, k, **kw)
+            for item in schedule:
+                if item[0] == "fork":
+                    dev.side_fork()
+                elif item[0] == "join":
+                    dev.side_join()
+                else:
+                    mm, a, b, c, m, n, k, kw = item[1]
+                    mm.enqueue(a, b, c, m, n, k, side=item[2], **kw)
     else:
         graph = dev.graph("gpt2_small_gemms")
-        for mm, a, b, c, m, n, k, kw in calls:
-            mm(a, b, c, m, n, k, graph=graph, **kw)
+        for item in schedule:
+            if item[0] == "fork":
+                graph.fork()
+            elif item[0] == "join":
+                graph.join()
+            else:
+                mm, a, b, c, m, n, k, kw = item[1]
+                mm(a, b, c, m, n, k, graph=graph, side=item[2], **kw)
         graph.finish()
 
         def run_step():
@@ -304,7 +349,10 @@ def main():
         "config": {"workload": "GPT-2-small training GEMMs: d_model 768, 12 layers, 8192 token rows, "
                                "QKV/proj/MLP + tied head 50257, fwd+dX+dW, 147 GEMMs, 6.07 TFLOP per step",
                    "rows": ROWS, "d_model": D, "layers": LAYERS, "vocab": VOCAB, "logits_row_pitch": vpitch,
-                   "launch": "eager" if args.eager else "hip-graph replay"},
+                   "launch": "eager" if args.eager else "hip-graph replay",
+                   "order": "forward, dX, dW per linear, one stream" if not args.overlap_dw else
+                            "forward pass, then backward pass with the layers' dW GEMMs on a second stream "
+                            "beside the next layer's dX chain (joined at the end)"},
         "frac_of_mfma_peak": round(tflops / PEAK_TFLOPS, 4),
         "sum_of_event_timed_gemms_ms": round(events_ms, 4),
         "roofline": roofline,

@@ -85,6 +85,10 @@ typedef struct {
  * (after a clear kernel when beta == 0), which is also what happens when the partial tiles
  * do not fit the workspace; it can be faster when C is large and the split is deep. */
 #define MG_FLAG_SPLITK_ATOMIC 2
+/* Run this GEMM on the context's side stream (see mg_side_fork): it overlaps with whatever the
+ * main stream runs until mg_side_join.  The side stream has its own half of the split-K
+ * workspace, so GEMMs of the two streams never meet there. */
+#define MG_FLAG_SIDE_STREAM 4
 
 typedef struct {
     int32_t id;
@@ -167,6 +171,21 @@ int mg_tile_fits(int id, const mg_gemm_args *args);
  * Writes tile id, split_k and group_m it would use for `args` on a device with
  * `compute_units` CUs. */
 int mg_pick(const mg_gemm_args *args, int compute_units, int *tile, int *split_k, int *group_m);
+
+/* ---- a second stream for independent GEMMs ----
+ * The reference orders every dispatch of a recorded step behind the previous one with a full
+ * compute-to-compute barrier (Graph.record, vk.py:848-851), although the dX and dW products
+ * of a linear layer (autograd.py:218-227) do not depend on each other.  Here a context owns a
+ * second stream (same, default priority): mg_side_fork makes it wait for everything enqueued
+ * on the main stream so far; GEMMs flagged MG_FLAG_SIDE_STREAM then run on it, concurrently
+ * with later main-stream work, in their own order; mg_side_join makes the main stream wait for
+ * everything enqueued on the side stream so far.  Both work eagerly and while a graph is being
+ * recorded (the branches become parallel paths of the graph; mg_graph_end joins if the caller
+ * has not).  A flagged GEMM without a preceding fork is an error; mg_sync, copies and mg_free
+ * wait for both streams.  Buffers written on one stream must not be touched on the other
+ * between fork and join. */
+int mg_side_fork(mg_ctx *ctx);
+int mg_side_join(mg_ctx *ctx);
 
 /* ---- record / replay: replaces vk.Graph (vk.py:807-889) ---- */
 

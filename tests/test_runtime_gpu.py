@@ -167,6 +167,91 @@ def test_graph_records_and_replays_gemm_with_split_k(dev):
         x.destroy()
 
 
+def _linear_backward_case(dev, rows, fin, fout, seed):
+    """Operands of one linear layer's backward pass on integer data: dY (rows, fout),
+    W (fout, fin), X (rows, fin) and the two exact products dX = dY W, dW = dY^T X."""
+    dy, w = O.make_operands(rows, fin, fout, False, False, "bf16", seed, integer=True)        # NN: (M,K), (K,N)
+    dy2, x = O.make_operands(fout, fin, rows, True, False, "bf16", seed + 1, integer=True)     # TN: (K,M), (K,N)
+    ref_dx = O.ref_gemm(dy, w, False, False, "bf16")
+    ref_dw = O.ref_gemm(dy2, x, True, False, "bf16")
+    bufs = {}
+    for name, arr in (("dy", dy), ("w", w), ("dy2", dy2), ("x", x)):
+        bufs[name] = dev.buffer(arr.nbytes, "device")
+        bufs[name].upload(arr)
+    bufs["dx"] = dev.buffer(rows * fin * 4, "device")
+    bufs["dw"] = dev.buffer(fout * fin * 4, "device")
+    return bufs, ref_dx, ref_dw
+
+
+def test_side_stream_runs_independent_gemms_concurrently(dev):
+    """dX on the main stream and dW on the side stream between fork and join, both with a
+    K split through the workspace (each stream owns its half, so the same tile numbers do
+    not collide): exact on integer data, several rounds back to back; misuse is refused."""
+    from vkgrad_amd.kernels import Matmul
+    from vkgrad_amd.vk import VkError
+    rows, fin, fout = 1024, 256, 384
+    bufs, ref_dx, ref_dw = _linear_backward_case(dev, rows, fin, fout, 21)
+    mm_dx = Matmul(dev, dtype="bf16", tile=3, split_k=3)
+    mm_dw = Matmul(dev, trans_a=True, dtype="bf16", tile=3, split_k=4)
+    try:
+        with pytest.raises(VkError):          # no fork yet
+            mm_dw.enqueue(bufs["dy2"], bufs["x"], bufs["dw"], fout, fin, rows, side=True)
+        with pytest.raises(VkError):          # an eager call waits for its result
+            mm_dw(bufs["dy2"], bufs["x"], bufs["dw"], fout, fin, rows, side=True)
+        for it in range(5):
+            bufs["dx"].upload(np.full((rows, fin), np.nan, np.float32))
+            bufs["dw"].upload(np.full((fout, fin), np.nan, np.float32))
+            dev.side_fork()
+            mm_dw.enqueue(bufs["dy2"], bufs["x"], bufs["dw"], fout, fin, rows, side=True)
+            mm_dx.enqueue(bufs["dy"], bufs["w"], bufs["dx"], rows, fin, fout)
+            dev.side_join()
+            dev.sync()
+            assert np.array_equal(bufs["dx"].download(np.float32, (rows, fin)), ref_dx), f"dX round {it}"
+            assert np.array_equal(bufs["dw"].download(np.float32, (fout, fin)), ref_dw), f"dW round {it}"
+    finally:
+        dev.side_join()
+        mm_dx.destroy()
+        mm_dw.destroy()
+        for b in bufs.values():
+            b.destroy()
+
+
+def test_graph_with_parallel_branches_replays(dev):
+    """A recorded step whose dW GEMMs sit on the side stream (fork before each, one join
+    at the end by finish()): every replay gives the exact products, with eager work and
+    synchronisations between the replays."""
+    from vkgrad_amd.kernels import Matmul
+    rows, fin, fout = 768, 512, 256
+    cases = [_linear_backward_case(dev, rows, fin, fout, 31 + 2 * i) for i in range(3)]
+    mm_dx = Matmul(dev, dtype="bf16")
+    mm_dw = Matmul(dev, trans_a=True, dtype="bf16", tile=11, split_k=3)
+    g = dev.graph("backward")
+    for bufs, _, _ in cases:
+        g.fork()
+        mm_dw(bufs["dy2"], bufs["x"], bufs["dw"], fout, fin, rows, graph=g, side=True)
+        mm_dx(bufs["dy"], bufs["w"], bufs["dx"], rows, fin, fout, graph=g)
+    g.finish()
+    try:
+        for it in range(4):
+            for bufs, _, _ in cases:
+                bufs["dx"].upload(np.full((rows, fin), np.nan, np.float32))
+                bufs["dw"].upload(np.full((fout, fin), np.nan, np.float32))
+            g.submit()
+            for j, (bufs, ref_dx, ref_dw) in enumerate(cases):
+                assert np.array_equal(bufs["dx"].download(np.float32, (rows, fin)), ref_dx), f"replay {it} dX {j}"
+                assert np.array_equal(bufs["dw"].download(np.float32, (fout, fin)), ref_dw), f"replay {it} dW {j}"
+            b0 = cases[0][0]
+            mm_dx(b0["dy"], b0["w"], b0["dx"], rows, fin, fout)      # eager work between replays
+            dev.sync()
+    finally:
+        g.destroy()
+        mm_dx.destroy()
+        mm_dw.destroy()
+        for bufs, _, _ in cases:
+            for b in bufs.values():
+                b.destroy()
+
+
 def test_elementwise_kernels(dev):
     from vkgrad_amd.kernels import make_kernels
     from oracle import ref_mlp as RM

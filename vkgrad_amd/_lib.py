@@ -13,6 +13,7 @@ MG_DEVICE, MG_SHARED, MG_CACHED, MG_BAR = 0, 1, 2, 3
 MG_ACT_NONE, MG_ACT_GELU, MG_ACT_RELU = 0, 1, 2
 MG_FLAG_TIGHT_BUFFERS = 1
 MG_FLAG_SPLITK_ATOMIC = 2
+MG_FLAG_SIDE_STREAM = 4
 
 DTYPES = {"f16": MG_F16, "bf16": MG_BF16}
 KINDS = {"device": MG_DEVICE, "shared": MG_SHARED, "cached": MG_CACHED, "bar": MG_BAR}
@@ -67,6 +68,8 @@ SIGNATURES = {
     "mg_last_error": (C.c_char_p, []),
     "mg_gemm_check": (C.c_int, [C.POINTER(GemmArgs)]),
     "mg_gemm": (C.c_int, [_P, C.POINTER(GemmArgs)]),
+    "mg_side_fork": (C.c_int, [_P]),
+    "mg_side_join": (C.c_int, [_P]),
     "mg_gemm_time": (C.c_int, [_P, C.POINTER(GemmArgs), C.c_int, C.POINTER(C.c_double)]),
     "mg_gemm_time_rotating": (C.c_int, [_P, C.POINTER(GemmArgs), C.c_int, C.c_int, C.POINTER(C.c_double)]),
     "mg_tile_count": (C.c_int, []),

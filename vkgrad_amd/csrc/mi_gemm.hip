@@ -388,7 +388,7 @@ static int check_args(const mg_gemm_args *a) {
     if (a->tile < -1 || a->tile >= MG_NUM_TILES) return fail(MG_ERR_ARG, "mg_gemm: unknown tile id %d", a->tile);
     if (a->split_k < 0 || a->split_k > 65535) return fail(MG_ERR_ARG, "mg_gemm: split_k %d out of range", a->split_k);
     if (a->group_m < 0) return fail(MG_ERR_ARG, "mg_gemm: group_m %d is negative", a->group_m);
-    if ((a->flags & ~(MG_FLAG_TIGHT_BUFFERS | MG_FLAG_SPLITK_ATOMIC)) || a->reserved)
+    if ((a->flags & ~(MG_FLAG_TIGHT_BUFFERS | MG_FLAG_SPLITK_ATOMIC | MG_FLAG_SIDE_STREAM)) || a->reserved)
         return fail(MG_ERR_ARG, "mg_gemm: unknown flags 0x%x", a->flags);
     return MG_OK;
 }
@@ -401,12 +401,17 @@ struct mg_ctx {
     int device;
     hipStream_t stream;
     hipEvent_t ev0, ev1;
+    // Side stream: GEMMs flagged MG_FLAG_SIDE_STREAM run there, concurrently with the
+    // main stream between mg_side_fork and mg_side_join.
+    hipStream_t side;
+    hipEvent_t ev_fork, ev_join;
+    bool side_forked;   // forked and not yet joined
     hipDeviceProp_t prop;
     bool capturing;
     // Split-K workspace: partial tiles of the K slices plus one arrival counter
     // per tile (zero between launches).  Allocated once, at init, so that its
     // address can be baked into captured graphs; a GEMM whose partials do not
-    // fit adds into C with atomics instead.
+    // fit adds into C with atomics instead.  Each stream owns one half of both.
     float *ws;
     int64_t ws_bytes;
     int *cnt;
@@ -438,36 +443,49 @@ int mg_init(int device_index, mg_ctx **out) {
     if (!c) return fail(MG_ERR_NOMEM, "mg_init: out of host memory");
     c->device = device_index;
     c->capturing = false;
+    c->side_forked = false;
+    c->stream = c->side = nullptr;
+    c->ev0 = c->ev1 = c->ev_fork = c->ev_join = nullptr;
+    c->ws = nullptr;
+    c->cnt = nullptr;
+    auto release = [](mg_ctx *x) {
+        if (x->ev0) (void)hipEventDestroy(x->ev0);
+        if (x->ev1) (void)hipEventDestroy(x->ev1);
+        if (x->ev_fork) (void)hipEventDestroy(x->ev_fork);
+        if (x->ev_join) (void)hipEventDestroy(x->ev_join);
+        if (x->stream) (void)hipStreamDestroy(x->stream);
+        if (x->side) (void)hipStreamDestroy(x->side);
+        if (x->ws) (void)hipFree(x->ws);
+        if (x->cnt) (void)hipFree(x->cnt);
+        delete x;
+    };
     e = hipGetDeviceProperties(&c->prop, device_index);
+    // both streams at the default priority
     if (e == hipSuccess) e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&c->side, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&c->ev0);
     if (e == hipSuccess) e = hipEventCreate(&c->ev1);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&c->ev_fork, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&c->ev_join, hipEventDisableTiming);
     if (e != hipSuccess) {
-        delete c;
+        release(c);
         return hip_fail(e, "mg_init");
     }
     if (strncmp(c->prop.gcnArchName, "gfx950", 6) != 0) {
         char arch[64];
         snprintf(arch, sizeof(arch), "%s", c->prop.gcnArchName);
-        (void)hipStreamDestroy(c->stream);
-        delete c;
+        release(c);
         return fail(MG_ERR_NODEVICE, "mg_init: device is %s; this library is built for gfx950 only", arch);
     }
-    c->ws = nullptr;
-    c->cnt = nullptr;
-    c->ws_bytes = 256ll << 20;
+    c->ws_bytes = 512ll << 20;
     if (const char *env = getenv("MIGEMM_SPLITK_WORKSPACE_MB")) c->ws_bytes = (int64_t)atoll(env) << 20;
+    c->ws_bytes &= ~(int64_t)511;   // two halves, each a multiple of 256 bytes
     if (c->ws_bytes > 0) {
         e = hipMalloc((void **)&c->ws, (size_t)c->ws_bytes);
-        if (e == hipSuccess) e = hipMalloc((void **)&c->cnt, MG_MAX_COUNTED_TILES * sizeof(int));
-        if (e == hipSuccess) e = hipMemset(c->cnt, 0, MG_MAX_COUNTED_TILES * sizeof(int));
+        if (e == hipSuccess) e = hipMalloc((void **)&c->cnt, 2 * MG_MAX_COUNTED_TILES * sizeof(int));
+        if (e == hipSuccess) e = hipMemset(c->cnt, 0, 2 * MG_MAX_COUNTED_TILES * sizeof(int));
         if (e != hipSuccess) {
-            (void)hipFree(c->ws);
-            (void)hipFree(c->cnt);
-            (void)hipEventDestroy(c->ev0);
-            (void)hipEventDestroy(c->ev1);
-            (void)hipStreamDestroy(c->stream);
-            delete c;
+            release(c);
             return hip_fail(e, "mg_init: split-K workspace");
         }
     } else {
@@ -481,9 +499,13 @@ int mg_destroy(mg_ctx *ctx) {
     if (!ctx) return MG_OK;
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
+    (void)hipStreamSynchronize(ctx->side);
     (void)hipEventDestroy(ctx->ev0);
     (void)hipEventDestroy(ctx->ev1);
+    (void)hipEventDestroy(ctx->ev_fork);
+    (void)hipEventDestroy(ctx->ev_join);
     (void)hipStreamDestroy(ctx->stream);
+    (void)hipStreamDestroy(ctx->side);
     (void)hipFree(ctx->ws);
     (void)hipFree(ctx->cnt);
     delete ctx;
@@ -543,6 +565,7 @@ int mg_free(mg_ctx *ctx, void *dev_ptr, int kind) {
     if (ctx->capturing) return fail(MG_ERR_STATE, "mg_free: not allowed while a graph is being recorded");
     HIP_TRY(hipSetDevice(ctx->device));
     HIP_TRY(hipStreamSynchronize(ctx->stream));
+    HIP_TRY(hipStreamSynchronize(ctx->side));
     if (kind == MG_DEVICE) HIP_TRY(hipFree(dev_ptr));
     else HIP_TRY(hipHostFree(dev_ptr));
     return MG_OK;
@@ -553,6 +576,7 @@ static int do_copy(mg_ctx *ctx, void *dst, const void *src, size_t nbytes, hipMe
     if (nbytes == 0) return MG_OK;
     if (ctx->capturing) return fail(MG_ERR_STATE, "%s: not allowed while a graph is being recorded", who);
     HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipStreamSynchronize(ctx->side));   // a copy sees what either stream has written
     HIP_TRY(hipMemcpyAsync(dst, src, nbytes, kind, ctx->stream));
     HIP_TRY(hipStreamSynchronize(ctx->stream));
     return MG_OK;
@@ -572,6 +596,26 @@ int mg_sync(mg_ctx *ctx) {
     if (!ctx) return fail(MG_ERR_ARG, "mg_sync: ctx is NULL");
     if (ctx->capturing) return fail(MG_ERR_STATE, "mg_sync: not allowed while a graph is being recorded");
     HIP_TRY(hipStreamSynchronize(ctx->stream));
+    HIP_TRY(hipStreamSynchronize(ctx->side));
+    return MG_OK;
+}
+
+int mg_side_fork(mg_ctx *ctx) {
+    if (!ctx) return fail(MG_ERR_ARG, "mg_side_fork: ctx is NULL");
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipEventRecord(ctx->ev_fork, ctx->stream));
+    HIP_TRY(hipStreamWaitEvent(ctx->side, ctx->ev_fork, 0));
+    ctx->side_forked = true;
+    return MG_OK;
+}
+
+int mg_side_join(mg_ctx *ctx) {
+    if (!ctx) return fail(MG_ERR_ARG, "mg_side_join: ctx is NULL");
+    if (!ctx->side_forked) return MG_OK;
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipEventRecord(ctx->ev_join, ctx->side));
+    HIP_TRY(hipStreamWaitEvent(ctx->stream, ctx->ev_join, 0));
+    ctx->side_forked = false;
     return MG_OK;
 }
 
@@ -631,6 +675,14 @@ int mg_pick(const mg_gemm_args *args, int compute_units, int *tile, int *split_k
 static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     const mg_gemm_args &a = *args;
     const TileDesc &t = g_tiles[pl.tile];
+    // the stream this GEMM runs on, and that stream's half of the split-K workspace
+    const bool on_side = (a.flags & MG_FLAG_SIDE_STREAM) != 0;
+    hipStream_t stream = on_side ? ctx->side : ctx->stream;
+    const int64_t lane_bytes = ctx->ws_bytes / 2;
+    float *lane_ws = ctx->ws ? ctx->ws + (on_side ? lane_bytes / (int64_t)sizeof(float) : 0) : nullptr;
+    int *lane_cnt = ctx->cnt ? ctx->cnt + (on_side ? MG_MAX_COUNTED_TILES : 0) : nullptr;
+    if (on_side && !ctx->side_forked)
+        return fail(MG_ERR_STATE, "mg_gemm: MG_FLAG_SIDE_STREAM needs mg_side_fork first");
     GemmParams p;
     p.A = (const uint16_t *)a.a;
     p.B = (const uint16_t *)a.b;
@@ -663,7 +715,7 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
         g.sa = p.sa; g.sb = p.sb; g.sc = p.sc;
         g.M = p.M; g.N = p.N; g.K = p.K; g.beta = p.beta;
         const dim3 grid((unsigned)cdiv(a.n, GEMV_ROWS_PER_WG), 1, (unsigned)a.nbatch);
-        hipError_t e = gemv_table[a.dtype][lm][lc](g, grid, ctx->stream);
+        hipError_t e = gemv_table[a.dtype][lm][lc](g, grid, stream);
         if (e != hipSuccess) return hip_fail(e, "mg_gemm: kernel launch");
         return MG_OK;
     }
@@ -678,9 +730,9 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
         // partial tiles go through the workspace when they fit
         const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n * a.nbatch;
         const int64_t need = tiles * pl.split_k * t.bm * t.bn * (int64_t)sizeof(float);
-        if (ctx->ws && need <= ctx->ws_bytes && tiles <= MG_MAX_COUNTED_TILES && !(a.flags & MG_FLAG_SPLITK_ATOMIC)) {
-            p.ws = ctx->ws;
-            p.cnt = ctx->cnt;
+        if (lane_ws && need <= lane_bytes && tiles <= MG_MAX_COUNTED_TILES && !(a.flags & MG_FLAG_SPLITK_ATOMIC)) {
+            p.ws = lane_ws;
+            p.cnt = lane_cnt;
         }
     }
     if (pl.split_k > 1 && a.beta == 0 && p.ws == nullptr) {
@@ -694,7 +746,7 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
         unsigned gx = (unsigned)cdiv(zn, 1024);
         unsigned gy = (unsigned)(zm < 4096 ? zm : 4096);
         if (gx > 65535u * 16u) return fail(MG_ERR_ARG, "mg_gemm: C too large for the split-K clear");
-        hipLaunchKernelGGL(zero_c_kernel, dim3(gx, gy, (unsigned)zb), dim3(256), 0, ctx->stream, a.c, a.ldc, zm, zn,
+        hipLaunchKernelGGL(zero_c_kernel, dim3(gx, gy, (unsigned)zb), dim3(256), 0, stream, a.c, a.ldc, zm, zn,
                            p.sc, vec);
         HIP_TRY(hipGetLastError());
     }
@@ -714,13 +766,13 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
             const int64_t need = (int64_t)sk.pieces * sk.rem_tiles * a.nbatch * t.bm * t.bn * (int64_t)sizeof(float);
             if (sk.pieces == 1) {
                 g = tiles < slots ? tiles : slots;   // nothing to cut
-            } else if (ctx->ws && need <= ctx->ws_bytes && tiles * a.nbatch <= MG_MAX_COUNTED_TILES) {
+            } else if (lane_ws && need <= lane_bytes && tiles * a.nbatch <= MG_MAX_COUNTED_TILES) {
                 p.stream_k = 1;
                 p.sk_full_rounds = sk.full_rounds;
                 p.sk_rem_tiles = sk.rem_tiles;
                 p.sk_pieces = sk.pieces;
-                p.ws = ctx->ws;
-                p.cnt = ctx->cnt;
+                p.ws = lane_ws;
+                p.cnt = lane_cnt;
             } else {
                 g = tiles < slots ? tiles : slots;
             }
@@ -730,7 +782,7 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     }
     launch_fn fn = table_for(a.layout, a.dtype)[pl.tile][general];
     if (!fn) return fail(MG_ERR_STATE, "mg_gemm: tile %d has no kernel for this alignment", pl.tile);
-    hipError_t e = fn(p, grid, ctx->stream);
+    hipError_t e = fn(p, grid, stream);
     if (e != hipSuccess) return hip_fail(e, "mg_gemm: kernel launch");
     return MG_OK;
 }
@@ -750,6 +802,7 @@ int mg_gemm_time(mg_ctx *ctx, const mg_gemm_args *args, int repeat, double *seco
     if (ctx->capturing) return fail(MG_ERR_STATE, "mg_gemm_time: not allowed while a graph is being recorded");
     int rc = check_args(args);
     if (rc != MG_OK) return rc;
+    if (args->flags & MG_FLAG_SIDE_STREAM) return fail(MG_ERR_ARG, "mg_gemm_time: timing runs on the main stream");
     Plan pl;
     pick_plan(*args, ctx->prop.multiProcessorCount, pl);
     HIP_TRY(hipEventRecord(ctx->ev0, ctx->stream));
@@ -775,6 +828,8 @@ int mg_gemm_time_rotating(mg_ctx *ctx, const mg_gemm_args *args, int nargs, int 
     for (int i = 0; i < nargs; i++) {
         int rc = check_args(&args[i]);
         if (rc != MG_OK) return rc;
+        if (args[i].flags & MG_FLAG_SIDE_STREAM)
+            return fail(MG_ERR_ARG, "mg_gemm_time_rotating: timing runs on the main stream");
         pick_plan(args[i], ctx->prop.multiProcessorCount, pl[i]);
     }
     HIP_TRY(hipEventRecord(ctx->ev0, ctx->stream));
@@ -793,6 +848,7 @@ int mg_gemm_time_rotating(mg_ctx *ctx, const mg_gemm_args *args, int nargs, int 
 int mg_graph_begin(mg_ctx *ctx) {
     if (!ctx) return fail(MG_ERR_ARG, "mg_graph_begin: ctx is NULL");
     if (ctx->capturing) return fail(MG_ERR_STATE, "mg_graph_begin: a graph is already being recorded");
+    if (ctx->side_forked) return fail(MG_ERR_STATE, "mg_graph_begin: join the side stream first (mg_side_join)");
     HIP_TRY(hipSetDevice(ctx->device));
     HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
     ctx->capturing = true;
@@ -803,6 +859,18 @@ int mg_graph_end(mg_ctx *ctx, mg_graph **out) {
     if (!ctx || !out) return fail(MG_ERR_ARG, "mg_graph_end: NULL argument");
     *out = nullptr;
     if (!ctx->capturing) return fail(MG_ERR_STATE, "mg_graph_end: no graph is being recorded");
+    if (ctx->side_forked) {
+        // a capture cannot end while a forked stream is still apart
+        int rc = mg_side_join(ctx);
+        if (rc != MG_OK) {
+            hipGraph_t dead = nullptr;
+            (void)hipStreamEndCapture(ctx->stream, &dead);
+            if (dead) (void)hipGraphDestroy(dead);
+            ctx->capturing = false;
+            ctx->side_forked = false;
+            return rc;
+        }
+    }
     hipGraph_t g = nullptr;
     hipError_t e = hipStreamEndCapture(ctx->stream, &g);
     ctx->capturing = false;

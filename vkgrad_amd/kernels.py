@@ -99,7 +99,7 @@ class Matmul:
         """Every tile handles ragged shapes; only positivity is required."""
         return m > 0 and n > 0 and k > 0
 
-    def _args(self, a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc):
+    def _args(self, a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side=False):
         if self.batched:
             nb = int(nbatch)
             sa, sb, sc = (int(s) for s in strides)
@@ -134,6 +134,8 @@ class Matmul:
         ga.flags = L.MG_FLAG_TIGHT_BUFFERS if (full_a > a.size or full_b > b.size) else 0
         if self.atomic_split:
             ga.flags |= L.MG_FLAG_SPLITK_ATOMIC
+        if side:
+            ga.flags |= L.MG_FLAG_SIDE_STREAM
         if m > 0 and n > 0 and k > 0:
             if need_a > a.size or need_b > b.size or need_c > c.size:
                 raise VkError(f"{self.name}: shape {m}x{n}x{k} (nbatch {nb}) needs {need_a}/{need_b}/{need_c} "
@@ -143,9 +145,14 @@ class Matmul:
         return ga
 
     def __call__(self, a, b, c, m, n, k, repeat=1, graph=None, nbatch=1, strides=(0, 0, 0),
-                 *, bias=None, accumulate=False, lda=None, ldb=None, ldc=None):
+                 *, bias=None, accumulate=False, lda=None, ldb=None, ldc=None, side=False):
+        """side=True (recorded calls only) puts the GEMM on the device's side stream:
+        it runs concurrently with the main stream between graph.fork() and graph.join()."""
         lib, ctx = self.dev._lib, self.dev._ctx
-        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc)
+        if side and graph is None:
+            raise VkError(f"{self.name}: side=True needs graph= (eager calls wait for their result); "
+                          f"use enqueue(..., side=True) between dev.side_fork() and dev.side_join()")
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side)
         if graph is not None:
             _check(lib.mg_gemm_check(C.byref(ga)), self.name)
             self._keep.append(ga)
@@ -177,9 +184,9 @@ class Matmul:
         return dt.value
 
     def enqueue(self, a, b, c, m, n, k, nbatch=1, strides=(0, 0, 0), *, bias=None,
-                accumulate=False, lda=None, ldb=None, ldc=None):
+                accumulate=False, lda=None, ldb=None, ldc=None, side=False):
         """Launch without waiting (the stream keeps order); for pipelined callers."""
-        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc)
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side)
         _check(self.dev._lib.mg_gemm(self.dev._ctx, C.byref(ga)), self.name)
 
     def plan(self, m, n, k, nbatch=1, lda=None, ldb=None, ldc=None):

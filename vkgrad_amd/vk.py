@@ -112,6 +112,23 @@ class Graph:
         self.traffic.append((name, compulsory, compulsory if bytes_hint is None else bytes_hint))
         self.n_dispatch += 1
 
+    def fork(self):
+        """From here on, launches recorded with side=True run on the device's side
+        stream, after everything recorded so far and concurrently with what the main
+        stream records next.  The reference puts a full barrier between any two
+        dispatches (vk.py:848-851); independent products (dX and dW of a linear
+        layer) need none."""
+        if self._finished:
+            raise VkError(f"{self.name}: already finished")
+        self._thunks.append(self.dev.side_fork)
+
+    def join(self):
+        """Later main-stream launches wait for the side stream's work recorded so far
+        (finish() joins by itself)."""
+        if self._finished:
+            raise VkError(f"{self.name}: already finished")
+        self._thunks.append(self.dev.side_join)
+
     def finish(self):
         if self._finished:
             raise VkError(f"{self.name}: already finished")
@@ -204,6 +221,14 @@ class Device:
         for _ in range(repeat):
             _check(self._lib.mg_copy(self._ctx, dst.ptr, src.ptr, size), "copy")
         return time.perf_counter() - t0
+
+    def side_fork(self):
+        """The side stream waits for the main stream's work so far (mg_side_fork)."""
+        _check(self._lib.mg_side_fork(self._ctx), "side_fork")
+
+    def side_join(self):
+        """The main stream waits for the side stream's work so far (mg_side_join)."""
+        _check(self._lib.mg_side_join(self._ctx), "side_join")
 
     def sync(self):
         _check(self._lib.mg_sync(self._ctx), "sync")
