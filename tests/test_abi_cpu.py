@@ -294,3 +294,25 @@ def test_product_never_imports_the_oracle():
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, f"{f} mentions the oracle"
                 assert "_work" not in text
+
+
+def test_sweep_workloads_match_the_stated_configurations():
+    """vkgrad_amd.sweep lists the GEMMs of the other workloads: the d_model-1024 decoder
+    has 1164 GEMMs and 139 TFLOP per optimiser step (4 micro-batches, dW with beta = 1 on
+    three of them), the square sweep 4 sizes x 3 layouts, the skinny sweep 5 x 3 NT cases
+    with bias, the char-LM 5 linears x 3 products."""
+    from vkgrad_amd.sweep import algorithmic_bytes, cases_for
+    dec = cases_for("decoder")
+    assert sum(c["count"] for c in dec) == 1164
+    assert abs(sum(2.0 * c["m"] * c["n"] * c["k"] * c["count"] for c in dec) / 1e12 - 138.98) < 0.01
+    acc = [c for c in dec if c["accumulate"]]
+    assert acc and all(c["layout"] == "TN" for c in acc) and sum(c["count"] for c in acc) == 3 * (24 * 4 + 1)
+    head = [c for c in dec if c["name"].startswith("head")]
+    assert {tuple(c["pitch"].items()) for c in head} == {(("ldc", 50304),), (("lda", 50304),)}
+    sq = cases_for("square")
+    assert len(sq) == 12 and {c["layout"] for c in sq} == {"NN", "NT", "TN"} and all(c["dtype"] == "f16" for c in sq)
+    sk = cases_for("skinny")
+    assert len(sk) == 15 and all(c["bias"] and c["layout"] == "NT" and c["k"] == 768 for c in sk)
+    one = next(c for c in sk if (c["m"], c["n"]) == (1, 50257))
+    assert algorithmic_bytes(one) == 2 * (768 + 768 * 50257) + 4 * 50257 + 4 * 50257
+    assert len(cases_for("charlm")) == 15
