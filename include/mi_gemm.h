@@ -63,7 +63,7 @@ typedef struct {
     int64_t m, n, k;
     const void *a;  int64_t lda;
     const void *b;  int64_t ldb;
-    float *c;       int64_t ldc;
+    float *c;       int64_t ldc;    /* may be NULL when y16 is given and beta == 0 */
     const float *bias;     /* NULL, or N floats added to every row of the result */
     int32_t nbatch;        /* >= 1; batch z uses a + z*sa, b + z*sb, c + z*sc (elements) */
     int32_t tile;          /* tile id from mg_tile_info, or -1 for the built-in picker */
@@ -71,7 +71,14 @@ typedef struct {
     int32_t split_k;       /* 0 = picker decides, 1 = none, >1 = that many K slices */
     int32_t group_m;       /* 0 = picker decides; else row-blocks per rasterisation band */
     int32_t flags;         /* MG_FLAG_* */
-    int32_t reserved;      /* must be 0 */
+    int32_t act;           /* MG_ACT_*: activation of the 16-bit output y16 (0 without y16) */
+    /* Fused forward epilogue — replaces the separate pass of bias_gelu / bias
+     * (kernels.py:709-718, 742-749): besides C = result (the pre-activation z the backward
+     * pass needs, f32), the epilogue writes y16 = narrow(act(result)) in the input dtype, the
+     * operand of the next layer's GEMM.  Layouts NN and NT, nbatch == 1; a K split goes
+     * through the workspace (MG_FLAG_SPLITK_ATOMIC is refused). */
+    void *y16;             /* NULL, or an (m, n) matrix of 16-bit elements */
+    int64_t ldy;           /* its row pitch in elements (>= n) */
 } mg_gemm_args;
 
 /* The buffers of A and B end at their last element: row padding (ld beyond the stored

@@ -258,6 +258,68 @@ def test_skinny_stream_tile_exact(dev, dtype):
     assert r["exact"]
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("layout", ["NN", "NT"])
+def test_fused_activation_output(dev, layout, dtype):
+    """Forward epilogue with the activated 16-bit output (the reference's separate
+    bias_gelu / bias pass, kernels.py:709-718, 742-749, folded into the GEMM):
+    C holds z = A.B + bias exactly (integer data), y16 = narrow(act(z)) - bit exact for
+    none and ReLU, within two 16-bit ulps of the numpy GELU (the device tanh differs in the
+    last bits); tiles with and without a fused variant, a K split through the workspace,
+    ragged and padded shapes, C omitted, and the misuse cases."""
+    from oracle import ref_mlp as R
+    from vkgrad_amd.kernels import CONFIGS, Matmul
+    from vkgrad_amd.vk import VkError
+    ta, tb = LAYOUTS[layout]
+    np16 = np.float16 if dtype == "f16" else np.uint16
+    cases = [(200, 136, 320, None, 0, "gelu"), (512, 384, 256, 11, 0, "relu"), (1000, 1016, 1024, 10, 0, "gelu"),
+             (392, 648, 2048, 11, 4, None), (129, 96, 768, 4, 3, "relu"), (300, 200, 264, 15, 0, "gelu"),
+             (64, 50, 72, 20, 0, "relu")]
+    for m, n, k, tile, split, act in cases:
+        a, b = O.make_operands(m, n, k, ta, tb, dtype, seed=m + k, integer=True)
+        bias = (np.arange(n) % 9 - 4).astype(np.float32) * 0.5
+        z_ref = O.ref_gemm(a, b, ta, tb, dtype, bias, None)
+        y_ref = O.round_to(R.act_fn(z_ref, act) if act else z_ref, dtype)
+        ldy = n + 6
+        ba, bb, bz = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), dev.buffer(n * 4, "device")
+        bc, by = dev.buffer(m * n * 4, "device"), dev.buffer(m * ldy * 2, "device")
+        ba.upload(a); bb.upload(b); bz.upload(bias)
+        mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype=dtype, tile=tile, split_k=split)
+        try:
+            for with_c in (True, False):
+                bc.upload(np.full((m, n), np.nan, np.float32))
+                by.upload(np.full((m, ldy), 0x7e01, np.uint16))
+                mm(ba, bb, bc if with_c else None, m, n, k, bias=bz, act=act, y16=by, ldy=ldy)
+                if with_c:
+                    assert np.array_equal(bc.download(np.float32, (m, n)), z_ref), (m, n, k, tile, "z")
+                yfull = by.download(np.uint16, (m, ldy))
+                assert np.all(yfull[:, n:] == 0x7e01), "the padding between rows of y16 was written"
+                got = np.ascontiguousarray(yfull[:, :n]).view(np16) if dtype == "f16" else np.ascontiguousarray(yfull[:, :n])
+                if act == "gelu":
+                    g32, w32 = O.widen(got, dtype), O.widen(y_ref, dtype)
+                    assert np.all(np.abs(g32 - w32) <= 2 * np.maximum(np.abs(w32), 2.0 ** -14) * 2.0 ** (-10 if dtype == "f16" else -7)), \
+                        (m, n, k, tile, np.abs(g32 - w32).max())
+                else:
+                    assert np.array_equal(got.view(np.uint16), y_ref.view(np.uint16)), (m, n, k, tile, act)
+        finally:
+            mm.destroy()
+            for x in (ba, bb, bz, bc, by):
+                x.destroy()
+    # misuse
+    mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype=dtype)
+    buf = dev.buffer(64 * 64 * 4, "device")
+    try:
+        with pytest.raises(VkError):
+            mm(buf, buf, buf, 64, 64, 64, act="gelu")                  # activation without y16
+        with pytest.raises(VkError):
+            mm(buf, buf, None, 64, 64, 64)                             # nothing to write
+        with pytest.raises(VkError):
+            mm(buf, buf, None, 64, 64, 64, y16=buf, accumulate=True)   # beta = 1 needs C
+    finally:
+        mm.destroy()
+        buf.destroy()
+
+
 def test_timing_over_rotating_operand_sets(dev):
     """The rotating timer launches argument set i % nsets on launch i: after seven
     launches over three sets with different integer operands, every set's C holds

@@ -31,7 +31,8 @@ class GemmArgs(C.Structure):
         ("nbatch", C.c_int32), ("tile", C.c_int32),
         ("sa", C.c_int64), ("sb", C.c_int64), ("sc", C.c_int64),
         ("split_k", C.c_int32), ("group_m", C.c_int32),
-        ("flags", C.c_int32), ("reserved", C.c_int32),
+        ("flags", C.c_int32), ("act", C.c_int32),
+        ("y16", C.c_void_p), ("ldy", C.c_int64),
     ]
 
 

@@ -173,7 +173,7 @@ struct DmaTraits {
     static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;
 };
 
-template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE>
+template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool ACT = false>
 __global__ void __launch_bounds__(WGM *WGN * 64)
 gemm_dma_kernel(const GemmParams p) {
     constexpr bool A_KC = (LAYOUT != L_TN);
@@ -316,7 +316,7 @@ gemm_dma_kernel(const GemmParams p) {
         stage = nstage;
     }
 
-    // Epilogue: identical to gemm_kernel.h.
+    // Epilogue: shared with the register-staged kernel (store_tile, gemm_kernel.h).
     bool add_bias = p.bias != nullptr && blockIdx.y == 0;
     int mode = p.split_k > 1 ? 2 : (p.beta ? 1 : 0);
     if (p.split_k > 1 && p.ws != nullptr) {
@@ -329,57 +329,7 @@ gemm_dma_kernel(const GemmParams p) {
         add_bias = p.bias != nullptr;
         mode = p.beta ? 1 : 0;
     }
-    const int row_l = m0 + wave_m * WTM + (lane >> 5) * 4;
-    const int col_l = n0 + wave_n * WTN + (lane & 31);
-    float *cl = C + (int64_t)row_l * p.ldc + col_l;
-    const int64_t ldc = p.ldc;
-    float bv[TN];
-#pragma unroll
-    for (int j = 0; j < TN; j++) bv[j] = (add_bias && col_l + j * 32 < p.N) ? p.bias[col_l + j * 32] : 0.f;
-
-    auto write_out = [&](auto mode_c, auto edge_c) {
-        constexpr int MODE = decltype(mode_c)::value;
-        constexpr bool EDGE = decltype(edge_c)::value != 0;
-#pragma unroll
-        for (int i = 0; i < TM; i++) {
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                float *ct = cl + (int64_t)(i * 32) * ldc + j * 32;
-                const bool col_ok = !EDGE || (col_l + j * 32 < p.N);
-                float old[16];
-                if constexpr (MODE == 1) {
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int ro = (r >> 2) * 8 + (r & 3);
-                        const bool ok = col_ok && (!EDGE || row_l + i * 32 + ro < p.M);
-                        old[r] = ok ? ct[ro * ldc] : 0.f;
-                    }
-                }
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int ro = (r >> 2) * 8 + (r & 3);
-                    const bool ok = col_ok && (!EDGE || row_l + i * 32 + ro < p.M);
-                    float v = acc[i][j][r] + bv[j];
-                    if constexpr (MODE == 1) v = old[r] + v;
-                    if (ok) {
-                        if constexpr (MODE == 2)
-                            __hip_atomic_fetch_add(ct + ro * ldc, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        else
-                            __builtin_nontemporal_store(v, ct + ro * ldc);   // streams past the L2
-                    }
-                }
-            }
-        }
-    };
-    if (interior) {
-        if (mode == 0) write_out(IntC<0>{}, IntC<0>{});
-        else if (mode == 1) write_out(IntC<1>{}, IntC<0>{});
-        else write_out(IntC<2>{}, IntC<0>{});
-    } else {
-        if (mode == 0) write_out(IntC<0>{}, IntC<1>{});
-        else if (mode == 1) write_out(IntC<1>{}, IntC<1>{});
-        else write_out(IntC<2>{}, IntC<1>{});
-    }
+    store_tile<DT, TM, TN, WTM, WTN, ACT>(p, C, acc, m0, n0, wave_m, wave_n, lane, add_bias, mode, interior);
 }
 
 // ---------------------------------------------------------------------------
@@ -729,10 +679,10 @@ gemm_dmap_kernel(const GemmParams p) {
     }
 }
 
-template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE>
+template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool ACT = false>
 hipError_t launch_gemm_dma(const GemmParams &p, dim3 grid, hipStream_t stream) {
     using TT = DmaTraits<LAYOUT, BM, BN, BK, WGM, WGN, NSTAGE>;
-    auto kern = gemm_dma_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, NSTAGE>;
+    auto kern = gemm_dma_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, NSTAGE, ACT>;
     static std::atomic<uint64_t> lds_allowed{0};
     hipError_t e = allow_dynamic_lds((const void *)kern, TT::LDS_BYTES, lds_allowed);
     if (e != hipSuccess) return e;

@@ -57,6 +57,11 @@ struct GemmParams {
     // tiles left over after them, and the number of equal K pieces each of those is cut into
     // (sk_rem_tiles * sk_pieces <= gridDim.x workgroups take one piece each)
     int sk_full_rounds, sk_rem_tiles, sk_pieces;
+    // fused activation output (kernels instantiated with ACT only): Y = narrow(act(result))
+    // in the input dtype; C (the pre-activation result) may then be null
+    uint16_t *Y;
+    int64_t ldy;
+    int act;              // MG_ACT_*
 };
 
 template <int DT>
@@ -326,7 +331,98 @@ __device__ __forceinline__ void interleave_group() {
     interleave_step<0, NMFMA, NDSR, NDSW, NVMEM>();
 }
 
-template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, bool GENERAL>
+// 16-bit narrowing (round to nearest even) and the activations of the fused output;
+// same formulas as the companion kernels (reference kernels.py:625-629, 709-718).
+template <int DT>
+__device__ __forceinline__ uint16_t narrow16_rne(float x) {
+    if constexpr (DT == D_F16) {
+        return __builtin_bit_cast(uint16_t, (_Float16)x);
+    } else {
+        uint32_t u = __builtin_bit_cast(uint32_t, x);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return (uint16_t)(u >> 16);
+    }
+}
+__device__ __forceinline__ float fused_act(float x, int act) {
+    if (act == 2) return fmaxf(x, 0.f);                  // MG_ACT_RELU
+    if (act == 1) {                                       // MG_ACT_GELU (tanh form)
+        const float c = 0.7978845608028654f;
+        return 0.5f * x * (1.0f + tanhf(c * (x + 0.044715f * x * x * x)));
+    }
+    return x;
+}
+
+// Writes one workgroup tile from the accumulators.  Accumulator register r of lane l holds
+//   row (r/4)*8 + (l/32)*4 + r%4,  column l%32   of its 32x32 tile,
+// so one store instruction writes two full 128-byte row segments.  mode: 0 overwrite,
+// 1 C += (read, add, store), 2 atomic +=; the mode and the edge test are uniform over the
+// workgroup and hoisted out of the element loops.  ACT: additionally Y = narrow(act(result))
+// (modes 0 and 1 only), and C is optional.
+template <int DT, int TM, int TN, int WTM, int WTN, bool ACT>
+__device__ __forceinline__ void store_tile(const GemmParams &p, float *C, f32x16 (&acc)[TM][TN], int m0, int n0,
+                                           int wave_m, int wave_n, int lane, bool add_bias, int mode,
+                                           bool interior) {
+    const int row_l = m0 + wave_m * WTM + (lane >> 5) * 4;
+    const int col_l = n0 + wave_n * WTN + (lane & 31);
+    float *cl = C + (int64_t)row_l * p.ldc + col_l;
+    const int64_t ldc = p.ldc;
+    uint16_t *yl = ACT ? p.Y + (int64_t)row_l * p.ldy + col_l : nullptr;
+    const int64_t ldy = ACT ? p.ldy : 0;
+    const bool have_c = !ACT || C != nullptr;
+    float bv[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) bv[j] = (add_bias && col_l + j * 32 < p.N) ? p.bias[col_l + j * 32] : 0.f;
+
+    auto write_out = [&](auto mode_c, auto edge_c) {
+        constexpr int MODE = decltype(mode_c)::value;   // 0 overwrite, 1 C += , 2 atomic +=
+        constexpr bool EDGE = decltype(edge_c)::value != 0;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                float *ct = cl + (int64_t)(i * 32) * ldc + j * 32;
+                uint16_t *yt = yl + (int64_t)(i * 32) * ldy + j * 32;
+                const bool col_ok = !EDGE || (col_l + j * 32 < p.N);
+                float old[16];
+                if constexpr (MODE == 1) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int ro = (r >> 2) * 8 + (r & 3);
+                        const bool ok = col_ok && (!EDGE || row_l + i * 32 + ro < p.M);
+                        old[r] = ok ? ct[ro * ldc] : 0.f;
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int ro = (r >> 2) * 8 + (r & 3);
+                    const bool ok = col_ok && (!EDGE || row_l + i * 32 + ro < p.M);
+                    float v = acc[i][j][r] + bv[j];
+                    if constexpr (MODE == 1) v = old[r] + v;
+                    if (ok) {
+                        if constexpr (MODE == 2) {
+                            __hip_atomic_fetch_add(ct + ro * ldc, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        } else {
+                            if (have_c) __builtin_nontemporal_store(v, ct + ro * ldc);   // written once: stream past the L2
+                            if constexpr (ACT) yt[ro * ldy] = narrow16_rne<DT>(fused_act(v, p.act));
+                        }
+                    }
+                }
+            }
+        }
+    };
+    if (interior) {
+        if (mode == 0) write_out(IntC<0>{}, IntC<0>{});
+        else if (mode == 1) write_out(IntC<1>{}, IntC<0>{});
+        else write_out(IntC<2>{}, IntC<0>{});
+    } else {
+        if (mode == 0) write_out(IntC<0>{}, IntC<1>{});
+        else if (mode == 1) write_out(IntC<1>{}, IntC<1>{});
+        else write_out(IntC<2>{}, IntC<1>{});
+    }
+}
+
+template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, bool GENERAL, bool ACT = false>
 __global__ void __launch_bounds__(WGM *WGN * 64)
 gemm_kernel(const GemmParams p) {
     constexpr bool A_KC = (LAYOUT != L_TN);
@@ -481,57 +577,7 @@ gemm_kernel(const GemmParams p) {
         add_bias = p.bias != nullptr;
         mode = p.beta ? 1 : 0;
     }
-    const int row_l = m0 + wave_m * WTM + (lane >> 5) * 4;
-    const int col_l = n0 + wave_n * WTN + (lane & 31);
-    float *cl = C + (int64_t)row_l * p.ldc + col_l;
-    const int64_t ldc = p.ldc;
-    float bv[TN];
-#pragma unroll
-    for (int j = 0; j < TN; j++) bv[j] = (add_bias && col_l + j * 32 < p.N) ? p.bias[col_l + j * 32] : 0.f;
-
-    auto write_out = [&](auto mode_c, auto edge_c) {
-        constexpr int MODE = decltype(mode_c)::value;   // 0 overwrite, 1 C += , 2 atomic +=
-        constexpr bool EDGE = decltype(edge_c)::value != 0;
-#pragma unroll
-        for (int i = 0; i < TM; i++) {
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                float *ct = cl + (int64_t)(i * 32) * ldc + j * 32;
-                const bool col_ok = !EDGE || (col_l + j * 32 < p.N);
-                float old[16];
-                if constexpr (MODE == 1) {
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int ro = (r >> 2) * 8 + (r & 3);
-                        const bool ok = col_ok && (!EDGE || row_l + i * 32 + ro < p.M);
-                        old[r] = ok ? ct[ro * ldc] : 0.f;
-                    }
-                }
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int ro = (r >> 2) * 8 + (r & 3);
-                    const bool ok = col_ok && (!EDGE || row_l + i * 32 + ro < p.M);
-                    float v = acc[i][j][r] + bv[j];
-                    if constexpr (MODE == 1) v = old[r] + v;
-                    if (ok) {
-                        if constexpr (MODE == 2)
-                            __hip_atomic_fetch_add(ct + ro * ldc, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        else
-                            __builtin_nontemporal_store(v, ct + ro * ldc);   // written once: stream past the L2
-                    }
-                }
-            }
-        }
-    };
-    if (interior) {
-        if (mode == 0) write_out(IntC<0>{}, IntC<0>{});
-        else if (mode == 1) write_out(IntC<1>{}, IntC<0>{});
-        else write_out(IntC<2>{}, IntC<0>{});
-    } else {
-        if (mode == 0) write_out(IntC<0>{}, IntC<1>{});
-        else if (mode == 1) write_out(IntC<1>{}, IntC<1>{});
-        else write_out(IntC<2>{}, IntC<1>{});
-    }
+    store_tile<DT, TM, TN, WTM, WTN, ACT>(p, C, acc, m0, n0, wave_m, wave_n, lane, add_bias, mode, interior);
 }
 
 typedef hipError_t (*launch_fn)(const GemmParams &, dim3 grid, hipStream_t);
@@ -550,10 +596,10 @@ inline hipError_t allow_dynamic_lds(const void *kern, int bytes, std::atomic<uin
     return e;
 }
 
-template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, bool GENERAL>
+template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, bool GENERAL, bool ACT = false>
 hipError_t launch_gemm(const GemmParams &p, dim3 grid, hipStream_t stream) {
     using TT = TileTraits<LAYOUT, BM, BN, BK, WGM, WGN>;
-    auto kern = gemm_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, GENERAL>;
+    auto kern = gemm_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, GENERAL, ACT>;
     static std::atomic<uint64_t> lds_allowed{0};
     hipError_t e = allow_dynamic_lds((const void *)kern, TT::LDS_BYTES, lds_allowed);
     if (e != hipSuccess) return e;

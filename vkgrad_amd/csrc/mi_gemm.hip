@@ -15,12 +15,12 @@
 #include "tiles.h"
 
 namespace mg {
-extern launch_fn launch_table_nn_f16[MG_NUM_TILES][2];
-extern launch_fn launch_table_nn_bf16[MG_NUM_TILES][2];
-extern launch_fn launch_table_nt_f16[MG_NUM_TILES][2];
-extern launch_fn launch_table_nt_bf16[MG_NUM_TILES][2];
-extern launch_fn launch_table_tn_f16[MG_NUM_TILES][2];
-extern launch_fn launch_table_tn_bf16[MG_NUM_TILES][2];
+extern launch_fn launch_table_nn_f16[MG_NUM_TILES][3];
+extern launch_fn launch_table_nn_bf16[MG_NUM_TILES][3];
+extern launch_fn launch_table_nt_f16[MG_NUM_TILES][3];
+extern launch_fn launch_table_nt_bf16[MG_NUM_TILES][3];
+extern launch_fn launch_table_tn_f16[MG_NUM_TILES][3];
+extern launch_fn launch_table_tn_bf16[MG_NUM_TILES][3];
 
 // ---------------------------------------------------------------------------
 // Pre-pass for split-K with beta == 0: C = 0 (a fill kernel, so the sequence can
@@ -81,7 +81,7 @@ static int hip_fail(hipError_t e, const char *what) {
         if (e_ != hipSuccess) return hip_fail(e_, #expr); \
     } while (0)
 
-static launch_fn (*table_for(int layout, int dtype))[2] {
+static launch_fn (*table_for(int layout, int dtype))[3] {
     switch (layout * 2 + dtype) {
         case 0: return launch_table_nn_f16;
         case 1: return launch_table_nn_bf16;
@@ -280,6 +280,7 @@ static double plan_cost_us(const mg_gemm_args &a, const TileDesc &t, int split, 
     return us;
 }
 
+static const int MG_ACT_FALLBACK_TILE = 3;
 static void finish_plan(const mg_gemm_args &a, int tile, int split, Plan &pl) {
     const TileDesc *d = &g_tiles[tile];
     int64_t kblocks = cdiv(a.k, d->bk);
@@ -295,6 +296,11 @@ static void finish_plan(const mg_gemm_args &a, int tile, int split, Plan &pl) {
         if (split > kblocks) split = (int)kblocks;
         kb_per = cdiv(kblocks, split);
         split = (int)cdiv(kblocks, kb_per);
+    }
+    if (a.y16 && !table_for(a.layout, a.dtype)[tile][2]) {
+        // the fused activation epilogue exists for a few tiles; the any-alignment 128 x 128 one runs everything
+        finish_plan(a, MG_ACT_FALLBACK_TILE, split, pl);
+        return;
     }
     pl.tile = tile;
     pl.grid_m = (int)cdiv(a.m, d->bm);
@@ -320,6 +326,7 @@ static void pick_plan(const mg_gemm_args &a, int cus, Plan &pl) {
         int bt = tile < 0 ? 0 : tile, bs = 1;
         for (int t = 0; t < MG_NUM_TILES; t++) {
             if (tile >= 0 && t != tile) continue;
+            if (tile < 0 && a.y16 && !table_for(a.layout, a.dtype)[t][2]) continue;
             const TileDesc &d = g_tiles[t];
             const int64_t kblocks = cdiv(a.k, d.bk);
             const int64_t groups = cdiv(a.m, d.bm) * cdiv(a.n, d.bn) * (int64_t)a.nbatch;
@@ -370,7 +377,19 @@ static int check_args(const mg_gemm_args *a) {
     if (a->m > 0x7fffffffLL - 512 || a->n > 0x7fffffffLL - 512 || a->k > 0x7fffffffLL - 512)
         return fail(MG_ERR_ARG, "mg_gemm: shape %lldx%lldx%lld exceeds 32-bit indexing", (long long)a->m,
                     (long long)a->n, (long long)a->k);
-    if (!a->a || !a->b || !a->c) return fail(MG_ERR_ARG, "mg_gemm: NULL operand pointer");
+    if (!a->a || !a->b) return fail(MG_ERR_ARG, "mg_gemm: NULL operand pointer");
+    if (!a->c && !(a->y16 && a->beta == 0))
+        return fail(MG_ERR_ARG, "mg_gemm: C may only be NULL with y16 given and beta == 0");
+    if (a->act < MG_ACT_NONE || a->act > MG_ACT_RELU) return fail(MG_ERR_ARG, "mg_gemm: unknown activation %d", a->act);
+    if (!a->y16 && a->act != MG_ACT_NONE) return fail(MG_ERR_ARG, "mg_gemm: an activation needs the y16 output");
+    if (a->y16) {
+        if (a->layout == MG_TN) return fail(MG_ERR_ARG, "mg_gemm: the fused y16 output exists for layouts NN and NT only");
+        if (a->nbatch != 1) return fail(MG_ERR_ARG, "mg_gemm: the fused y16 output needs nbatch == 1");
+        if ((uintptr_t)a->y16 & 1) return fail(MG_ERR_ARG, "mg_gemm: y16 must be 2-byte aligned");
+        if (a->ldy < a->n) return fail(MG_ERR_ARG, "mg_gemm: ldy %lld < N %lld", (long long)a->ldy, (long long)a->n);
+        if (a->flags & MG_FLAG_SPLITK_ATOMIC)
+            return fail(MG_ERR_ARG, "mg_gemm: the fused y16 output cannot be combined with MG_FLAG_SPLITK_ATOMIC");
+    }
     if (((uintptr_t)a->a | (uintptr_t)a->b) & 1) return fail(MG_ERR_ARG, "mg_gemm: A and B must be 2-byte aligned");
     if ((uintptr_t)a->c & 3) return fail(MG_ERR_ARG, "mg_gemm: C must be 4-byte aligned");
     if (a->bias && ((uintptr_t)a->bias & 3)) return fail(MG_ERR_ARG, "mg_gemm: bias must be 4-byte aligned");
@@ -378,7 +397,7 @@ static int check_args(const mg_gemm_args *a) {
     const int64_t b_cols = a->layout == MG_NT ? a->k : a->n;
     if (a->lda < a_cols) return fail(MG_ERR_ARG, "mg_gemm: lda %lld < %lld stored columns of A", (long long)a->lda, (long long)a_cols);
     if (a->ldb < b_cols) return fail(MG_ERR_ARG, "mg_gemm: ldb %lld < %lld stored columns of B", (long long)a->ldb, (long long)b_cols);
-    if (a->ldc < a->n) return fail(MG_ERR_ARG, "mg_gemm: ldc %lld < N %lld", (long long)a->ldc, (long long)a->n);
+    if (a->c && a->ldc < a->n) return fail(MG_ERR_ARG, "mg_gemm: ldc %lld < N %lld", (long long)a->ldc, (long long)a->n);
     if (a->nbatch < 1 || a->nbatch > 65535) return fail(MG_ERR_ARG, "mg_gemm: nbatch %d out of range [1, 65535]", a->nbatch);
     if (a->nbatch > 1 && (a->sa < 0 || a->sb < 0 || a->sc < 0))
         return fail(MG_ERR_ARG, "mg_gemm: negative batch stride");
@@ -388,7 +407,7 @@ static int check_args(const mg_gemm_args *a) {
     if (a->tile < -1 || a->tile >= MG_NUM_TILES) return fail(MG_ERR_ARG, "mg_gemm: unknown tile id %d", a->tile);
     if (a->split_k < 0 || a->split_k > 65535) return fail(MG_ERR_ARG, "mg_gemm: split_k %d out of range", a->split_k);
     if (a->group_m < 0) return fail(MG_ERR_ARG, "mg_gemm: group_m %d is negative", a->group_m);
-    if ((a->flags & ~(MG_FLAG_TIGHT_BUFFERS | MG_FLAG_SPLITK_ATOMIC | MG_FLAG_SIDE_STREAM)) || a->reserved)
+    if (a->flags & ~(MG_FLAG_TIGHT_BUFFERS | MG_FLAG_SPLITK_ATOMIC | MG_FLAG_SIDE_STREAM))
         return fail(MG_ERR_ARG, "mg_gemm: unknown flags 0x%x", a->flags);
     return MG_OK;
 }
@@ -721,6 +740,9 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     }
     if (lds_bytes_for(t, a.layout) > (int)ctx->prop.maxSharedMemoryPerMultiProcessor)
         return fail(MG_ERR_ARG, "mg_gemm: tile %d needs %d bytes of LDS", pl.tile, lds_bytes_for(t, a.layout));
+    p.Y = (uint16_t *)a.y16;
+    p.ldy = a.ldy;
+    p.act = a.act;
     p.ws = nullptr;
     p.cnt = nullptr;
     p.stream_k = 0;
@@ -733,6 +755,15 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
         if (lane_ws && need <= lane_bytes && tiles <= MG_MAX_COUNTED_TILES && !(a.flags & MG_FLAG_SPLITK_ATOMIC)) {
             p.ws = lane_ws;
             p.cnt = lane_cnt;
+        }
+        if (a.y16 && !p.ws) {
+            // the activation is applied once, to the finished sum: without a workspace for the
+            // slices to meet in, the same GEMM runs unsplit
+            mg_gemm_args whole = a;
+            whole.split_k = 1;
+            Plan unsplit;
+            pick_plan(whole, ctx->prop.multiProcessorCount, unsplit);
+            return enqueue_gemm(ctx, &whole, unsplit);
         }
     }
     if (pl.split_k > 1 && a.beta == 0 && p.ws == nullptr) {
@@ -753,6 +784,7 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     // direct-to-LDS tiles: eligibility was settled by the plan; register-staged
     // tiles: the any-alignment instantiation unless every chunk is aligned and whole
     int general = t.nstage > 0 ? 0 : (operands_aligned(a) ? 0 : 1);
+    if (a.y16) general = 2;   // the variant with the fused activation output
     dim3 grid((unsigned)(pl.grid_m * pl.grid_n), (unsigned)pl.split_k, (unsigned)a.nbatch);
     if (t.persistent) {
         // resident workgroups loop over (slice, tile) units; [1] = epilogue with bias

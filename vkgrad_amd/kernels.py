@@ -99,7 +99,8 @@ class Matmul:
         """Every tile handles ragged shapes; only positivity is required."""
         return m > 0 and n > 0 and k > 0
 
-    def _args(self, a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side=False):
+    def _args(self, a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side=False,
+              act=None, y16=None, ldy=None):
         if self.batched:
             nb = int(nbatch)
             sa, sb, sc = (int(s) for s in strides)
@@ -110,7 +111,7 @@ class Matmul:
         ga.layout, ga.dtype = self.layout, L.DTYPES[self.dtype]
         ga.beta = 1 if accumulate else 0
         ga.m, ga.n, ga.k = int(m), int(n), int(k)
-        ga.a, ga.b, ga.c = a.ptr, b.ptr, c.ptr
+        ga.a, ga.b, ga.c = a.ptr, b.ptr, (c.ptr if c is not None else None)
         ga.lda = int(lda) if lda is not None else (m if self.trans_a else k)
         ga.ldb = int(ldb) if ldb is not None else (k if self.trans_b else n)
         ga.ldc = int(ldc) if ldc is not None else n
@@ -136,23 +137,39 @@ class Matmul:
             ga.flags |= L.MG_FLAG_SPLITK_ATOMIC
         if side:
             ga.flags |= L.MG_FLAG_SIDE_STREAM
+        if act not in L.ACTS:
+            raise VkError(f"{self.name}: unknown activation {act!r}; use None, 'gelu' or 'relu'")
+        ga.act = L.ACTS[act]
+        if y16 is not None:
+            ga.y16 = y16.ptr
+            ga.ldy = int(ldy) if ldy is not None else n
+            if m > 0 and n > 0 and y16.size < ((m - 1) * ga.ldy + n) * 2:
+                raise VkError(f"{self.name}: y16 buffer of {y16.size} bytes is too small for {m}x{n} (pitch {ga.ldy})")
+        elif ga.act:
+            raise VkError(f"{self.name}: act= needs y16= (the activated 16-bit output)")
+        if c is None and y16 is None:
+            raise VkError(f"{self.name}: C may only be omitted when y16 is given")
         if m > 0 and n > 0 and k > 0:
-            if need_a > a.size or need_b > b.size or need_c > c.size:
+            if need_a > a.size or need_b > b.size or (c is not None and need_c > c.size):
                 raise VkError(f"{self.name}: shape {m}x{n}x{k} (nbatch {nb}) needs {need_a}/{need_b}/{need_c} "
-                              f"bytes but buffers hold {a.size}/{b.size}/{c.size}")
+                              f"bytes but buffers hold {a.size}/{b.size}/{c.size if c is not None else 0}")
             if bias is not None and bias.size < n * 4:
                 raise VkError(f"{self.name}: bias buffer of {bias.size} bytes is shorter than N={n} floats")
         return ga
 
     def __call__(self, a, b, c, m, n, k, repeat=1, graph=None, nbatch=1, strides=(0, 0, 0),
-                 *, bias=None, accumulate=False, lda=None, ldb=None, ldc=None, side=False):
+                 *, bias=None, accumulate=False, lda=None, ldb=None, ldc=None, side=False,
+                 act=None, y16=None, ldy=None):
         """side=True (recorded calls only) puts the GEMM on the device's side stream:
-        it runs concurrently with the main stream between graph.fork() and graph.join()."""
+        it runs concurrently with the main stream between graph.fork() and graph.join().
+        y16= (with act=None, 'gelu' or 'relu') makes the epilogue also write
+        narrow(act(result)) in the input dtype, the separate bias_gelu pass of the
+        reference (kernels.py:709-718) folded into the GEMM; c may then be None."""
         lib, ctx = self.dev._lib, self.dev._ctx
         if side and graph is None:
             raise VkError(f"{self.name}: side=True needs graph= (eager calls wait for their result); "
                           f"use enqueue(..., side=True) between dev.side_fork() and dev.side_join()")
-        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side)
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy)
         if graph is not None:
             _check(lib.mg_gemm_check(C.byref(ga)), self.name)
             self._keep.append(ga)
@@ -160,7 +177,7 @@ class Matmul:
             def launch(ga=ga):
                 _check(lib.mg_gemm(ctx, C.byref(ga)), self.name)
 
-            graph.record(launch, [a, b, c], name=self.name,
+            graph.record(launch, [x for x in (a, b, c, y16) if x is not None], name=self.name,
                          bytes_hint=self.traffic_bytes(m, n, k, nbatch))
             nb_ = nbatch if self.batched else 1
             graph.mm_split.append((nb_ * 2 * (m * k + k * n), nb_ * m * n * 4))
@@ -184,9 +201,9 @@ class Matmul:
         return dt.value
 
     def enqueue(self, a, b, c, m, n, k, nbatch=1, strides=(0, 0, 0), *, bias=None,
-                accumulate=False, lda=None, ldb=None, ldc=None, side=False):
+                accumulate=False, lda=None, ldb=None, ldc=None, side=False, act=None, y16=None, ldy=None):
         """Launch without waiting (the stream keeps order); for pipelined callers."""
-        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side)
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy)
         _check(self.dev._lib.mg_gemm(self.dev._ctx, C.byref(ga)), self.name)
 
     def plan(self, m, n, k, nbatch=1, lda=None, ldb=None, ldc=None):
