@@ -61,11 +61,13 @@ def test_baseline_config_loss_curve(dev, fuse_bias):
     assert got[-1] < 0.5 * got[0], "not learning"
 
 
-def test_reference_variant_loss_curve(dev):
+@pytest.mark.parametrize("fuse_bias", [False, True])
+def test_reference_variant_loss_curve(dev, fuse_bias):
     """What examples.mnist --synthetic actually runs (mnist.py:124-128, 146-147):
-    784 zero-padded to 1024 -> 256 -> 16 (10 real classes), GELU."""
+    784 zero-padded to 1024 -> 256 -> 16 (10 real classes), GELU; with fuse_bias the
+    bias, GELU and narrowing happen in the forward GEMM's epilogue."""
     got, want = run_curve(dev, steps=60, batch=128, sizes=(1024, 256), n_classes=10, pad=16,
-                          act="gelu", dtype="f16", recorded=True)
+                          act="gelu", dtype="f16", fuse_bias=fuse_bias, recorded=True)
     assert np.abs(got[:5] - want[:5]).max() < 2e-3
     assert np.abs(got - want).max() < 3e-2
 

@@ -11,7 +11,7 @@ per Linear, in the reference's storage convention (W is in_f x out_f):
 
 Extensions (all off by default keep the reference's exact kernel sequence):
     Ctx(dtype="bf16")        16-bit type of activations and weight mirrors
-    Ctx(fuse_bias=True)      bias added in the forward GEMM's epilogue
+    Ctx(fuse_bias=True)      bias, activation and 16-bit narrowing in the forward GEMM's epilogue
     MLP(activation="relu")   ReLU instead of GELU in hidden layers
     Linear.backward(accumulate=True)   dW += (beta=1 epilogue), db +=
 """
@@ -172,12 +172,14 @@ class Linear:
         n = self.batch * self.out_f
         mm = c.matmul(self.batch, self.out_f, self.in_f)
         if c.fuse_bias:
-            # z = x @ W + b straight out of the GEMM epilogue
-            mm(x16, self.W.w16, self.z, self.batch, self.out_f, self.in_f, graph=graph, bias=self.b.w32)
+            # z = x @ W + b straight out of the GEMM epilogue, and with an activation
+            # also y16 = narrow(act(z)): no separate pass over the (batch x out_f) tensor
             if self.activation:
-                K[self.act + "16"]([self.z, self.y16], n, graph=graph)
+                mm(x16, self.W.w16, self.z, self.batch, self.out_f, self.in_f, graph=graph, bias=self.b.w32,
+                   act=self.act, y16=self.y16)
                 out = self.y16
             else:
+                mm(x16, self.W.w16, self.z, self.batch, self.out_f, self.in_f, graph=graph, bias=self.b.w32)
                 out = self.z
         else:
             mm(x16, self.W.w16, self.acc, self.batch, self.out_f, self.in_f, graph=graph)
