@@ -231,6 +231,12 @@ int mg_ew_adamw(mg_ctx *ctx, float *w, const float *g, float *m, float *v, void 
                 const float *hp, int64_t n, float wd, int dtype);
 /* zero (kernels.py:853-854) */
 int mg_ew_zero(mg_ctx *ctx, float *dst, int64_t n);
+/* Device-side copy of nbytes (multiple of 4, both pointers 4-byte aligned) that can be
+ * recorded into a graph, unlike mg_copy.  The reference's recorded step reads what the CPU
+ * wrote into mapped buffers directly (inputs, labels, the optimiser's per-step scalars:
+ * vk.py:583-590, autograd.py:313-329); on a discrete card every such read crosses PCIe, so a
+ * recorded step stages them into HBM with this kernel first. */
+int mg_ew_copy(mg_ctx *ctx, void *dst, const void *src, int64_t nbytes);
 /* cast16 (kernels.py:857-860) */
 int mg_ew_cast16(mg_ctx *ctx, const float *src, void *dst, int64_t n, int dtype);
 /* Scratch operands for warm-up and tuning (kernels.py:367-375, 472-474 use uninitialised

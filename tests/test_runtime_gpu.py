@@ -294,3 +294,43 @@ def test_elementwise_kernels(dev):
     # zero
     K["zero"]([bx], 1000)
     assert not bx.download(np.float32, (1000,)).any()
+
+
+def test_column_sums_and_recordable_copy(dev):
+    """col_sum over one chunk of rows (fixed order) and over several (chunks meet through
+    atomics after a clear), overwriting and accumulating; the recordable copy kernel for
+    16-byte-aligned and merely 4-byte-aligned ends, with a tail."""
+    from vkgrad_amd.kernels import make_kernels
+    K = make_kernels(dev, "f16")
+    rng = np.random.default_rng(5)
+    for nrow, ncol in [(128, 512), (1, 10), (513, 70), (2000, 300), (5000, 64)]:
+        g = rng.standard_normal((nrow, ncol)).astype(np.float32)
+        bg, bs = dev.buffer(g.nbytes, "device"), dev.buffer(ncol * 4, "device")
+        bg.upload(g)
+        bs.upload(np.full(ncol, 7.0, np.float32))
+        want = g.astype(np.float64).sum(0)
+        K["col_sum"]([bg, bs], ncol, nrow)
+        got = bs.download(np.float32, (ncol,))
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-4 * np.sqrt(nrow)), (nrow, ncol)
+        K["col_sum_acc"]([bg, bs], ncol, nrow)
+        got2 = bs.download(np.float32, (ncol,))
+        assert np.allclose(got2, 2 * want, rtol=1e-5, atol=2e-4 * np.sqrt(nrow)), (nrow, ncol)
+        bg.destroy()
+        bs.destroy()
+    src = dev.buffer(4096, "shared")
+    dst = dev.buffer(4096, "device")
+    data = rng.integers(0, 2 ** 32, 1024, dtype=np.uint64).astype(np.uint32)
+    src.array(np.uint32, (1024,))[:] = data
+    for nbytes in (32, 1000, 4096):
+        dst.upload(np.zeros(1024, np.uint32))
+        K["copy"]([src, dst], nbytes)
+        out = dst.download(np.uint32, (1024,))
+        assert np.array_equal(out[:nbytes // 4], data[:nbytes // 4]) and not out[nbytes // 4:].any()
+    # ends that are only 4-byte aligned: through the C ABI with offset pointers
+    dst.upload(np.zeros(1024, np.uint32))
+    assert dev._lib.mg_ew_copy(dev._ctx, dst.ptr + 4, src.ptr + 8, 400) == 0
+    out = dst.download(np.uint32, (1024,))
+    assert np.array_equal(out[1:101], data[2:102]) and out[0] == 0 and not out[101:].any()
+    assert dev._lib.mg_ew_copy(dev._ctx, dst.ptr, src.ptr, 6) != 0     # not a multiple of 4
+    src.destroy()
+    dst.destroy()

@@ -88,6 +88,7 @@ SIGNATURES = {
     "mg_ew_softmax_ce": (C.c_int, [_P, _P, _P, _P, _P, _P, C.c_int64, C.c_int64, C.c_int64, C.c_int]),
     "mg_ew_adamw": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, C.c_int64, C.c_float, C.c_int]),
     "mg_ew_zero": (C.c_int, [_P, _P, C.c_int64]),
+    "mg_ew_copy": (C.c_int, [_P, _P, _P, C.c_int64]),
     "mg_ew_cast16": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int]),
     "mg_ew_grad_add": (C.c_int, [_P, _P, _P, C.c_int64]),
     "mg_ew_fill_uniform16": (C.c_int, [_P, _P, C.c_int64, C.c_uint32, C.c_int]),

@@ -101,7 +101,12 @@ class Ctx:
 
 
 class Param:
-    """f32 master, 16-bit mirror for the matmul, f32 grad, Adam moments."""
+    """f32 master, 16-bit mirror for the matmul, f32 grad, Adam moments (autograd.py:111-156).
+
+    The reference keeps the master in host-cached mapped memory, which on its APU is the
+    same DRAM the GPU uses; on a discrete card the optimiser (and the bias read of a GEMM
+    epilogue) would cross PCIe for every element, so the master lives in HBM and numpy() /
+    set() copy."""
 
     def __init__(self, ctx, shape, init=None, name="", no_decay=False):
         self.ctx = ctx
@@ -109,26 +114,22 @@ class Param:
         self.n = int(np.prod(shape))
         self.name = name
         self.no_decay = no_decay
-        self.w32 = ctx.buf(self.n * 4, "cached")
+        self.w32 = ctx.buf(self.n * 4, "device")
         self.w16 = ctx.buf(self.n * 2, "device")
         self.g32 = ctx.buf(self.n * 4, "device")
         self.m = ctx.zeros(self.n)
         self.v = ctx.zeros(self.n)
-        w = self.w32.array(np.float32, shape)
-        w[:] = 0 if init is None else init
-        self.w32.flush()
-        self.sync16()
+        self.set(np.zeros(shape, np.float32) if init is None else init)
 
     def sync16(self):
         self.ctx.K["cast16"]([self.w32, self.w16], self.n)
 
     def numpy(self):
-        self.w32.invalidate()
-        return self.w32.array(np.float32, self.shape)
+        """A host copy of the master weights."""
+        return self.w32.download(np.float32, self.shape)
 
     def set(self, arr):
-        self.w32.array(np.float32, self.shape)[:] = arr
-        self.w32.flush()
+        self.w32.upload(np.ascontiguousarray(np.broadcast_to(np.asarray(arr, np.float32), self.shape)))
         self.sync16()
 
     def grad_numpy(self):
@@ -235,6 +236,7 @@ class MLP:
         self.dlog16 = ctx.buf(batch * pad_classes * 2)
         self.dlog32 = ctx.buf(batch * pad_classes * 4)
         self.loss = ctx.buf(batch * 4, "cached")
+        self._stage = {}   # HBM copies of host-mapped inputs, by buffer
 
     def params(self):
         for l in self.layers:
@@ -247,9 +249,22 @@ class MLP:
             h = l.forward(h, tape if tape is not None else [], graph=graph)
         return h
 
+    def _staged(self, buf, graph):
+        """A buffer the CPU writes between replays (host-mapped, vk.py:583-590) is copied
+        into HBM by the step's first kernels: the GEMMs that read the batch twice (forward
+        and dW of the first layer) then do not fetch it over PCIe."""
+        if not buf.host_visible:
+            return buf
+        dev_copy = self._stage.get(id(buf))
+        if dev_copy is None:
+            dev_copy = self._stage[id(buf)] = self.ctx.buf((buf.size + 3) // 4 * 4, "device")
+        self.ctx.K["copy"]([buf, dev_copy], buf.size // 4 * 4, graph=graph)
+        return dev_copy
+
     def record(self, x16, labels_buf, graph, accumulate=False):
         K = self.ctx.K
         tape = []
+        x16, labels_buf = self._staged(x16, graph), self._staged(labels_buf, graph)
         logits = self.logits(x16, tape, graph=graph)
         K["softmax_ce"]([logits, labels_buf, self.dlog16, self.dlog32, self.loss],
                         self.batch, self.pad, self.n_classes, graph=graph)
@@ -290,6 +305,9 @@ class AdamW:
         self.t = 0
         self.hp = ctx.buf(8 * 4, "shared")
         self.hpv = self.hp.array(np.float32)
+        # the kernels read the scalars from HBM: one staging copy per step instead of a
+        # PCIe read of the mapped buffer from every wavefront of every parameter's kernel
+        self.hp_dev = ctx.buf(8 * 4, "device")
         self._set_hp(lr)
 
     def _set_hp(self, lr):
@@ -304,16 +322,18 @@ class AdamW:
 
     def record(self, graph):
         k = self.ctx.K["adamw"]
+        self.ctx.K["copy"]([self.hp, self.hp_dev], 8 * 4, graph=graph)
         for p in self.params:
             wd = 0.0 if p.no_decay else self.wd
-            k([p.w32, p.g32, p.m, p.v, p.w16, self.hp], p.n, wd, graph=graph)
+            k([p.w32, p.g32, p.m, p.v, p.w16, self.hp_dev], p.n, wd, graph=graph)
 
     def step(self, lr=None):
         self.advance(lr)
         k = self.ctx.K["adamw"]
+        self.ctx.K["copy"]([self.hp, self.hp_dev], 8 * 4)
         for p in self.params:
             wd = 0.0 if p.no_decay else self.wd
-            k([p.w32, p.g32, p.m, p.v, p.w16, self.hp], p.n, wd)
+            k([p.w32, p.g32, p.m, p.v, p.w16, self.hp_dev], p.n, wd)
 
 
 class TrainStep:

@@ -61,12 +61,45 @@ __global__ void k_act_bwd(const float *dy, const float *z, uint16_t *dz16, float
     if (dz32) dz32[i] = g;
 }
 
-__global__ void k_col_sum(const float *g, float *sums, int64_t ncol, int64_t nrow, int accumulate) {
-    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= ncol) return;
+// Column sums (the reference loops the rows in one thread per column, kernels.py:753-761:
+// fine at batch 128 on 12 CUs, one long chain of dependent loads here).  A block takes 64
+// columns and COL_SUM_ROWS rows: 8 threads per column stride through the rows (coalesced 256-byte
+// row pieces), LDS adds the 8 partial sums.  One chunk of rows: the block writes (or adds to) the
+// sum itself, in a fixed order.  More rows: the chunks add with atomics into sums, which the
+// host has cleared unless accumulating.
+constexpr int COL_SUM_ROWS = 512;
+__global__ void __launch_bounds__(512) k_col_sum(const float *g, float *sums, int64_t ncol, int64_t nrow,
+                                                  int accumulate, int atomic) {
+    __shared__ float part[8][64];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int64_t c = (int64_t)blockIdx.x * 64 + tx;
+    const int64_t r0 = (int64_t)blockIdx.y * COL_SUM_ROWS;
+    const int64_t r1 = r0 + COL_SUM_ROWS < nrow ? r0 + COL_SUM_ROWS : nrow;
     float s = 0.f;
-    for (int64_t r = 0; r < nrow; ++r) s += g[r * ncol + c];
-    sums[c] = accumulate ? sums[c] + s : s;
+    if (c < ncol) {
+#pragma unroll 8
+        for (int64_t r = r0 + ty; r < r1; r += 8) s += g[r * ncol + c];
+    }
+    part[ty][tx] = s;
+    __syncthreads();
+    if (ty == 0 && c < ncol) {
+        float t = part[0][tx];
+#pragma unroll
+        for (int i = 1; i < 8; i++) t += part[i][tx];
+        if (atomic) atomicAdd(sums + c, t);
+        else sums[c] = accumulate ? sums[c] + t : t;
+    }
+}
+
+// Device-side copy of nbytes (a multiple of 4; 16-byte pieces when both ends are aligned).
+__global__ void k_copy(const uint32_t *src, uint32_t *dst, int64_t nwords, int vec) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (vec) {
+        if (i * 4 + 3 < nwords) reinterpret_cast<uint4 *>(dst)[i] = reinterpret_cast<const uint4 *>(src)[i];
+        else for (int64_t j = i * 4; j < nwords; j++) dst[j] = src[j];
+    } else if (i < nwords) {
+        dst[i] = src[i];
+    }
 }
 
 __global__ void k_softmax_ce(const float *logits, const uint32_t *labels, uint16_t *dl16, float *dl32, float *loss,
@@ -178,9 +211,23 @@ int mg_ew_act_bwd(mg_ctx *ctx, const float *dy, const float *z, void *dz16, floa
 }
 
 int mg_ew_col_sum(mg_ctx *ctx, const float *g, float *sums, int64_t ncol, int64_t nrow, int accumulate) {
-    EW_PRECHECK("mg_ew_col_sum", g && sums && count_ok(ncol) && nrow > 0);
-    hipLaunchKernelGGL(k_col_sum, dim3(blocks_for(ncol)), dim3(256), 0, ctx_stream(ctx), g, sums, ncol, nrow, accumulate);
+    EW_PRECHECK("mg_ew_col_sum", g && sums && count_ok(ncol) && nrow > 0 && nrow <= (int64_t)65535 * COL_SUM_ROWS);
+    const unsigned chunks = (unsigned)((nrow + COL_SUM_ROWS - 1) / COL_SUM_ROWS);
+    if (chunks > 1 && !accumulate) hipLaunchKernelGGL(k_zero, dim3(blocks_for(ncol)), dim3(256), 0, ctx_stream(ctx), sums, ncol);
+    hipLaunchKernelGGL(k_col_sum, dim3((unsigned)((ncol + 63) / 64), chunks), dim3(512), 0, ctx_stream(ctx), g, sums, ncol,
+                       nrow, accumulate, chunks > 1 ? 1 : 0);
     EW_POSTCHECK("mg_ew_col_sum");
+}
+
+int mg_ew_copy(mg_ctx *ctx, void *dst, const void *src, int64_t nbytes) {
+    EW_PRECHECK("mg_ew_copy", dst && src && count_ok(nbytes) && nbytes % 4 == 0 &&
+                                  (((uintptr_t)dst | (uintptr_t)src) & 3) == 0);
+    const int64_t nwords = nbytes / 4;
+    const int vec = ((((uintptr_t)dst | (uintptr_t)src) & 15) == 0) ? 1 : 0;
+    const int64_t threads = vec ? (nwords + 3) / 4 : nwords;
+    hipLaunchKernelGGL(k_copy, dim3(blocks_for(threads)), dim3(256), 0, ctx_stream(ctx), (const uint32_t *)src,
+                       (uint32_t *)dst, nwords, vec);
+    EW_POSTCHECK("mg_ew_copy");
 }
 
 int mg_ew_softmax_ce(mg_ctx *ctx, const float *logits, const uint32_t *labels, void *dl16, float *dl32, float *loss,

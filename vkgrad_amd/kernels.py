@@ -565,6 +565,8 @@ def make_kernels(dev, dtype="f16"):
     add("adamw", lambda lib, ctx, p, n, wd:
         lib.mg_ew_adamw(ctx, p[0], p[1], p[2], p[3], p[4], p[5], n, float(wd), dt))
     add("zero", lambda lib, ctx, p, n: lib.mg_ew_zero(ctx, p[0], n))
+    # buffers: src, dst ; n = bytes — recordable device-side copy (stages CPU-written inputs into HBM)
+    add("copy", lambda lib, ctx, p, n: lib.mg_ew_copy(ctx, p[1], p[0], n))
     add("cast16", lambda lib, ctx, p, n: lib.mg_ew_cast16(ctx, p[0], p[1], n, dt))
     # dataparallel.py:54-58 — buffers: dst, src
     add("grad_add", lambda lib, ctx, p, n: lib.mg_ew_grad_add(ctx, p[0], p[1], n))
