@@ -176,6 +176,11 @@ def test_picker_properties(lib):
     # tiny problems still get a plan
     info, split, _ = pick(lib, m=1, n=1, k=1, lda=1, ldb=1, ldc=1)
     assert split == 1
+    # many batches of a narrow problem: the batches fill the chip, so no tile is cut along K and
+    # a tile four times wider than N is not worth its padding
+    info, split, _ = pick(lib, m=1024, n=64, k=1024, lda=1024, ldb=64, ldc=64, nbatch=96,
+                          sa=1024 * 1024, sb=1024 * 64, sc=1024 * 64)
+    assert split == 1 and info.bn <= 128
     # the skinny-M streaming tile runs NT with at most 4 rows over K <= 2048 and hands
     # everything else to its fallback
     mv = next(i for i in range(lib.mg_tile_count()) if tile_name(lib, i).startswith("mv_"))

@@ -257,16 +257,21 @@ static double plan_cost_us(const mg_gemm_args &a, const TileDesc &t, int split, 
     if (t.persistent == 2) {
         // stream-K: whole rounds, then one round of K pieces and their meeting
         const int64_t kblocks = cdiv(a.k, t.bk);
-        const StreamK sk = stream_k_partition(gm * gn, kblocks, slots);
+        // every batch is partitioned by itself (grid.z), over its share of the resident slots
+        const int64_t slots_z = slots / a.nbatch > 0 ? slots / a.nbatch : 1;
+        const StreamK sk = stream_k_partition(gm * gn, kblocks, slots_z);
         const int lay2 = a.layout == MG_NN ? 0 : (a.layout == MG_NT ? 1 : 2);
-        double occ = (double)cdiv(sk.grid, cus) / wpc;
+        double occ = (double)cdiv(sk.grid * a.nbatch, cus) / wpc;
         if (occ > 1.0) occ = 1.0;
         if (occ < 0.6) occ = 0.6;
         const double blocks = (double)sk.full_rounds * kblocks + (sk.rem_tiles ? (double)cdiv(kblocks, sk.pieces) : 0.0);
         const double units_wg = sk.full_rounds + (sk.rem_tiles ? 1 : 0);
         // meeting of the pieces: about 5.2 us per piece of a 256 x 256 tile, 1.4 us of a 128 x 128 one
         const double per_piece = t.bm * t.bn > 128 * 128 ? 5.2 : 1.4;
-        return 1.5 + units_wg * g_cost[t.id][lay2][0] + blocks * occ * g_cost[t.id][lay2][1] +
+        // more workgroups than resident slots (many batches): they take turns
+        double turns = (double)(sk.grid * a.nbatch) / (double)slots;
+        if (turns < 1.0) turns = 1.0;
+        return 1.5 + turns * (units_wg * g_cost[t.id][lay2][0] + blocks * occ * g_cost[t.id][lay2][1]) +
                (sk.pieces > 1 ? sk.pieces * per_piece : 0.0);
     }
     if (rounds < 1.0) rounds = 1.0;
@@ -791,10 +796,13 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
         general = a.bias != nullptr ? 1 : 0;
         const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n;
         const int64_t slots = (int64_t)ctx->prop.multiProcessorCount * wgs_per_cu(t, a.layout);
-        int64_t g = persistent_grid(t, tiles, pl.split_k, a.k / t.bk, slots);
+        // stream-K cuts tiles only when the batches together leave resident slots idle: every batch
+        // (one grid.z slice) is partitioned by itself, over its share of the slots
+        const int64_t slots_z = slots / a.nbatch > 0 ? slots / a.nbatch : 1;
+        int64_t g = persistent_grid(t, tiles, pl.split_k, a.k / t.bk, t.persistent == 2 ? slots_z : slots);
         if (t.persistent == 2 && pl.split_k == 1) {
             // one workspace slot per piece; without the workspace the tile runs as plain persistent
-            const StreamK sk = stream_k_partition(tiles, a.k / t.bk, slots);
+            const StreamK sk = stream_k_partition(tiles, a.k / t.bk, slots_z);
             const int64_t need = (int64_t)sk.pieces * sk.rem_tiles * a.nbatch * t.bm * t.bn * (int64_t)sizeof(float);
             if (sk.pieces == 1) {
                 g = tiles < slots ? tiles : slots;   // nothing to cut
