@@ -52,8 +52,9 @@ enum { MG_NN = 0, MG_NT = 1, MG_TN = 2 };
 enum { MG_F16 = 0, MG_BF16 = 1 };
 /* memory kinds of vk.py:1161-1175 */
 enum { MG_DEVICE = 0, MG_SHARED = 1, MG_CACHED = 2, MG_BAR = 3 };
-/* activations for the companion elementwise kernels */
-enum { MG_ACT_NONE = 0, MG_ACT_GELU = 1, MG_ACT_RELU = 2 };
+/* activations for the companion elementwise kernels and the fused GEMM epilogues; the
+ * _GRAD forms exist for mg_gemm only (result times the activation's derivative at z) */
+enum { MG_ACT_NONE = 0, MG_ACT_GELU = 1, MG_ACT_RELU = 2, MG_ACT_GELU_GRAD = 3, MG_ACT_RELU_GRAD = 4 };
 
 typedef struct {
     int32_t struct_size;   /* sizeof(mg_gemm_args), checked */
@@ -79,6 +80,13 @@ typedef struct {
      * through the workspace (MG_FLAG_SPLITK_ATOMIC is refused). */
     void *y16;             /* NULL, or an (m, n) matrix of 16-bit elements */
     int64_t ldy;           /* its row pitch in elements (>= n) */
+    /* Fused backward epilogue — replaces the separate pass of bias_gelu_bwd
+     * (kernels.py:720-739; its call site autograd.py:204-207): with act = MG_ACT_GELU_GRAD or
+     * MG_ACT_RELU_GRAD the dX GEMM of one layer hands the layer below its dz directly,
+     *   g = result * act'(z),   y16 = narrow(g),   C = g (when C is given),
+     * where z is that lower layer's pre-activation (m, n) in f32.  beta == 0 and no bias. */
+    const float *z;        /* NULL unless act is a _GRAD form */
+    int64_t ldz;           /* its row pitch in elements (>= n) */
 } mg_gemm_args;
 
 /* The buffers of A and B end at their last element: row padding (ld beyond the stored

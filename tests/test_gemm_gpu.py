@@ -320,6 +320,82 @@ def test_fused_activation_output(dev, layout, dtype):
         buf.destroy()
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("layout", ["NN", "NT"])
+def test_fused_activation_gradient_output(dev, layout, dtype):
+    """Backward epilogue (the reference's separate bias_gelu_bwd pass, kernels.py:720-739,
+    folded into the dX GEMM that feeds it, autograd.py:204-207, 224-227): with integer
+    operands the product is exact, so C and y16 must equal product * act'(z) - bit exact for
+    ReLU (the factor is 0 or 1), within 1e-5 of the product's magnitude (f32) and two 16-bit
+    ulps for GELU, whose derivative the device forms from one exponential; z has its own
+    pitch, padding of y16 stays untouched, C may be omitted, tiles with and without a fused
+    variant and a K split through the workspace."""
+    from oracle import ref_mlp as R
+    from vkgrad_amd.kernels import Matmul
+    from vkgrad_amd.vk import VkError
+    ta, tb = LAYOUTS[layout]
+    np16 = np.float16 if dtype == "f16" else np.uint16
+    cases = [(200, 136, 320, None, 0, "gelu"), (512, 384, 256, 11, 0, "relu"), (1000, 1016, 1024, 10, 0, "gelu"),
+             (392, 648, 2048, 11, 4, "relu"), (129, 96, 768, 4, 3, "gelu"), (300, 200, 264, 15, 0, "relu"),
+             (64, 50, 72, 3, 0, "gelu")]
+    for m, n, k, tile, split, act in cases:
+        a, b = O.make_operands(m, n, k, ta, tb, dtype, seed=m + k, integer=True)
+        prod = O.ref_gemm(a, b, ta, tb, dtype, None, None)
+        ldz, ldy = n + 3, n + 6
+        rng = np.random.default_rng(m * 7 + n)
+        z = np.zeros((m, ldz), np.float32)
+        z[:, :n] = rng.standard_normal((m, n)).astype(np.float32) * 2.0
+        z[:, n:] = np.nan
+        g_ref = (prod.astype(np.float64) * R.dact_fn(z[:, :n].astype(np.float64), act)).astype(np.float32)
+        ba, bb, bz = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), dev.buffer(z.nbytes, "device")
+        bc, by = dev.buffer(m * n * 4, "device"), dev.buffer(m * ldy * 2, "device")
+        ba.upload(a); bb.upload(b); bz.upload(z)
+        mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype=dtype, tile=tile, split_k=split)
+        try:
+            for with_c in (True, False):
+                bc.upload(np.full((m, n), np.nan, np.float32))
+                by.upload(np.full((m, ldy), 0x7e01, np.uint16))
+                mm(ba, bb, bc if with_c else None, m, n, k, act=act + "_grad", y16=by, ldy=ldy, z=bz, ldz=ldz)
+                yfull = by.download(np.uint16, (m, ldy))
+                assert np.all(yfull[:, n:] == 0x7e01), "the padding between rows of y16 was written"
+                got16 = np.ascontiguousarray(yfull[:, :n])
+                if dtype == "f16":
+                    got16 = got16.view(np16)
+                if act == "relu":
+                    if with_c:
+                        assert np.array_equal(bc.download(np.float32, (m, n)), g_ref), (m, n, k, tile, "dz32")
+                    assert np.array_equal(got16.view(np.uint16), O.round_to(g_ref, dtype).view(np.uint16)), (m, n, k, tile)
+                else:
+                    tol = 1e-5 * np.maximum(np.abs(prod), 1.0)
+                    if with_c:
+                        got = bc.download(np.float32, (m, n))
+                        assert np.all(np.abs(got - g_ref) <= tol), (m, n, k, tile, np.abs(got - g_ref).max())
+                    g32 = O.widen(got16, dtype)
+                    ulp = np.maximum(np.abs(g_ref), 2.0 ** -14) * 2.0 ** (-10 if dtype == "f16" else -7)
+                    assert np.all(np.abs(g32 - g_ref) <= 2 * ulp + tol), (m, n, k, tile, np.abs(g32 - g_ref).max())
+        finally:
+            mm.destroy()
+            for x in (ba, bb, bz, bc, by):
+                x.destroy()
+    # misuse
+    mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype=dtype)
+    buf = dev.buffer(64 * 64 * 4, "device")
+    try:
+        with pytest.raises(VkError):
+            mm(buf, buf, buf, 64, 64, 64, act="gelu_grad", y16=buf)                          # no z
+        with pytest.raises(VkError):
+            mm(buf, buf, buf, 64, 64, 64, act="gelu", y16=buf, z=buf)                        # z without a _grad activation
+        with pytest.raises(VkError):
+            mm(buf, buf, buf, 64, 64, 64, act="relu_grad", y16=buf, z=buf, bias=buf)         # bias
+        with pytest.raises(VkError):
+            mm(buf, buf, buf, 64, 64, 64, act="relu_grad", y16=buf, z=buf, accumulate=True)  # beta = 1
+        with pytest.raises(VkError):
+            mm(buf, buf, buf, 64, 64, 64, act="relu_grad", y16=buf, z=buf, ldz=60)           # pitch below N
+    finally:
+        mm.destroy()
+        buf.destroy()
+
+
 def test_timing_over_rotating_operand_sets(dev):
     """The rotating timer launches argument set i % nsets on launch i: after seven
     launches over three sets with different integer operands, every set's C holds

@@ -17,7 +17,9 @@ MG_FLAG_SIDE_STREAM = 4
 
 DTYPES = {"f16": MG_F16, "bf16": MG_BF16}
 KINDS = {"device": MG_DEVICE, "shared": MG_SHARED, "cached": MG_CACHED, "bar": MG_BAR}
-ACTS = {None: MG_ACT_NONE, "none": MG_ACT_NONE, "gelu": MG_ACT_GELU, "relu": MG_ACT_RELU}
+MG_ACT_GELU_GRAD, MG_ACT_RELU_GRAD = 3, 4
+ACTS = {None: MG_ACT_NONE, "none": MG_ACT_NONE, "gelu": MG_ACT_GELU, "relu": MG_ACT_RELU,
+        "gelu_grad": MG_ACT_GELU_GRAD, "relu_grad": MG_ACT_RELU_GRAD}
 
 
 class GemmArgs(C.Structure):
@@ -33,6 +35,7 @@ class GemmArgs(C.Structure):
         ("split_k", C.c_int32), ("group_m", C.c_int32),
         ("flags", C.c_int32), ("act", C.c_int32),
         ("y16", C.c_void_p), ("ldy", C.c_int64),
+        ("z", C.c_void_p), ("ldz", C.c_int64),
     ]
 
 

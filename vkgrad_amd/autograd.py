@@ -166,6 +166,7 @@ class Linear:
         self.dz32 = ctx.buf(batch * out_f * 4)
         self.dx32 = ctx.buf(batch * in_f * 4) if need_dx else None
         self.x16 = None
+        self._dz_ready = False   # set by the layer above when its dX epilogue wrote dz16 / dz32
 
     def forward(self, x16, tape, graph=None):
         c, K = self.ctx, self.ctx.K
@@ -193,10 +194,18 @@ class Linear:
         tape.append(self.backward)
         return out
 
-    def backward(self, dout16, dout32, graph=None, accumulate=False):
+    def backward(self, dout16, dout32, graph=None, accumulate=False, below=None):
+        """`below`: the Linear whose output this layer consumed.  Under fuse_bias, when
+        that layer has an activation, this layer's dX GEMM multiplies by act'(below.z) in
+        its epilogue and writes below.dz16 / below.dz32 itself: the separate
+        activation-backward pass of the reference (autograd.py:204-207) disappears, and
+        (below.dz16, below.dz32) is returned in place of dX."""
         c, K = self.ctx, self.ctx.K
         n = self.batch * self.out_f
-        if self.activation:
+        if self.activation and self._dz_ready:
+            self._dz_ready = False
+            g16, g32 = self.dz16, self.dz32
+        elif self.activation:
             K["bias_" + self.act + "_bwd"]([dout32, self.z, self.dz16, self.dz32], n, graph=graph)
             g16, g32 = self.dz16, self.dz32
         else:
@@ -211,8 +220,14 @@ class Linear:
         if not self.need_dx:
             return None, None
         # dX = dZ @ W^T.  W is stored in_f x out_f, which is N x K: trans_b.
-        c.matmul(self.batch, self.in_f, self.out_f, trans_b=True)(
-            g16, self.W.w16, self.dx32, self.batch, self.in_f, self.out_f, graph=graph)
+        mm = c.matmul(self.batch, self.in_f, self.out_f, trans_b=True)
+        if (c.fuse_bias and below is not None and below.activation
+                and (below.batch, below.out_f) == (self.batch, self.in_f)):
+            mm(g16, self.W.w16, below.dz32, self.batch, self.in_f, self.out_f, graph=graph,
+               act=below.act + "_grad", z=below.z, y16=below.dz16)
+            below._dz_ready = True
+            return below.dz16, below.dz32
+        mm(g16, self.W.w16, self.dx32, self.batch, self.in_f, self.out_f, graph=graph)
         return None, self.dx32
 
 
@@ -269,8 +284,9 @@ class MLP:
         K["softmax_ce"]([logits, labels_buf, self.dlog16, self.dlog32, self.loss],
                         self.batch, self.pad, self.n_classes, graph=graph)
         g16, g32 = self.dlog16, self.dlog32
-        for fn in reversed(tape):
-            g16, g32 = fn(g16, g32, graph=graph, accumulate=accumulate)
+        for i in reversed(range(len(tape))):
+            g16, g32 = tape[i](g16, g32, graph=graph, accumulate=accumulate,
+                               below=self.layers[i - 1] if i > 0 else None)
 
     def read_loss(self):
         self.loss.invalidate()
@@ -285,8 +301,8 @@ class MLP:
                         self.batch, self.pad, self.n_classes)
         loss = self.read_loss()
         g16, g32 = self.dlog16, self.dlog32
-        for fn in reversed(tape):
-            g16, g32 = fn(g16, g32, accumulate=accumulate)
+        for i in reversed(range(len(tape))):
+            g16, g32 = tape[i](g16, g32, accumulate=accumulate, below=self.layers[i - 1] if i > 0 else None)
         return loss
 
     def predict(self, x16):

@@ -62,6 +62,8 @@ struct GemmParams {
     uint16_t *Y;
     int64_t ldy;
     int act;              // MG_ACT_*
+    const float *Z;       // pre-activation for the _GRAD activations
+    int64_t ldz;
 };
 
 template <int DT>
@@ -353,7 +355,17 @@ __device__ __forceinline__ float fused_act(float x, int act) {
         const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
         return x * __frcp_rn(1.0f + __expf(-2.0f * u));
     }
-    return x;
+    return x;   // none, and the _GRAD forms (their factor is applied before)
+}
+// derivative of the activation at pre-activation x, for MG_ACT_GELU_GRAD (3) / MG_ACT_RELU_GRAD (4)
+// (reference kernels.py:630-635).  With s = 1 / (1 + exp(-2u)) = (1 + tanh u) / 2:
+//   gelu'(x) = s + x * 2 s (1 - s) * c (1 + 3 * 0.044715 x^2)
+__device__ __forceinline__ float fused_dact(float x, int act) {
+    if (act == 4) return x > 0.f ? 1.f : 0.f;
+    const float c = 0.7978845608028654f;
+    const float u = c * (x + 0.044715f * x * x * x);
+    const float s = __frcp_rn(1.0f + __expf(-2.0f * u));
+    return s + x * (2.0f * s * (1.0f - s)) * (c * (1.0f + 0.134145f * x * x));
 }
 
 // Writes one workgroup tile from the accumulators.  Accumulator register r of lane l holds
@@ -361,7 +373,8 @@ __device__ __forceinline__ float fused_act(float x, int act) {
 // so one store instruction writes two full 128-byte row segments.  mode: 0 overwrite,
 // 1 C += (read, add, store), 2 atomic +=; the mode and the edge test are uniform over the
 // workgroup and hoisted out of the element loops.  ACT: additionally Y = narrow(act(result))
-// (modes 0 and 1 only), and C is optional.
+// (modes 0 and 1 only), and C is optional; with a _GRAD activation (mode 0 only) the result
+// is first multiplied by act'(Z) and goes to both outputs that way.
 template <int DT, int TM, int TN, int WTM, int WTN, bool ACT>
 __device__ __forceinline__ void store_tile(const GemmParams &p, float *C, f32x16 (&acc)[TM][TN], int m0, int n0,
                                            int wave_m, int wave_n, int lane, bool add_bias, int mode,
@@ -373,6 +386,9 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, float *C, f32x16
     uint16_t *yl = ACT ? p.Y + (int64_t)row_l * p.ldy + col_l : nullptr;
     const int64_t ldy = ACT ? p.ldy : 0;
     const bool have_c = !ACT || C != nullptr;
+    const bool grad = ACT && p.act >= 3;
+    const float *zl = grad ? p.Z + (int64_t)row_l * p.ldz + col_l : nullptr;
+    const int64_t ldz = grad ? p.ldz : 0;
     float bv[TN];
 #pragma unroll
     for (int j = 0; j < TN; j++) bv[j] = (add_bias && col_l + j * 32 < p.N) ? p.bias[col_l + j * 32] : 0.f;
@@ -396,12 +412,26 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, float *C, f32x16
                         old[r] = ok ? ct[ro * ldc] : 0.f;
                     }
                 }
+                if constexpr (ACT && MODE == 0) {
+                    if (grad) {
+                        const float *zt = zl + (int64_t)(i * 32) * ldz + j * 32;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const int ro = (r >> 2) * 8 + (r & 3);
+                            const bool ok = col_ok && (!EDGE || row_l + i * 32 + ro < p.M);
+                            old[r] = ok ? __builtin_nontemporal_load(zt + ro * ldz) : 0.f;
+                        }
+                    }
+                }
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int ro = (r >> 2) * 8 + (r & 3);
                     const bool ok = col_ok && (!EDGE || row_l + i * 32 + ro < p.M);
                     float v = acc[i][j][r] + bv[j];
                     if constexpr (MODE == 1) v = old[r] + v;
+                    if constexpr (ACT && MODE == 0) {
+                        if (grad) v *= fused_dact(old[r], p.act);
+                    }
                     if (ok) {
                         if constexpr (MODE == 2) {
                             __hip_atomic_fetch_add(ct + ro * ldc, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -385,8 +385,16 @@ static int check_args(const mg_gemm_args *a) {
     if (!a->a || !a->b) return fail(MG_ERR_ARG, "mg_gemm: NULL operand pointer");
     if (!a->c && !(a->y16 && a->beta == 0))
         return fail(MG_ERR_ARG, "mg_gemm: C may only be NULL with y16 given and beta == 0");
-    if (a->act < MG_ACT_NONE || a->act > MG_ACT_RELU) return fail(MG_ERR_ARG, "mg_gemm: unknown activation %d", a->act);
+    if (a->act < MG_ACT_NONE || a->act > MG_ACT_RELU_GRAD) return fail(MG_ERR_ARG, "mg_gemm: unknown activation %d", a->act);
     if (!a->y16 && a->act != MG_ACT_NONE) return fail(MG_ERR_ARG, "mg_gemm: an activation needs the y16 output");
+    if (a->act >= MG_ACT_GELU_GRAD) {
+        if (!a->z) return fail(MG_ERR_ARG, "mg_gemm: a _GRAD activation needs the pre-activation z");
+        if ((uintptr_t)a->z & 3) return fail(MG_ERR_ARG, "mg_gemm: z must be 4-byte aligned");
+        if (a->ldz < a->n) return fail(MG_ERR_ARG, "mg_gemm: ldz %lld < N %lld", (long long)a->ldz, (long long)a->n);
+        if (a->beta != 0 || a->bias) return fail(MG_ERR_ARG, "mg_gemm: a _GRAD activation needs beta == 0 and no bias");
+    } else if (a->z) {
+        return fail(MG_ERR_ARG, "mg_gemm: z is only read by the _GRAD activations");
+    }
     if (a->y16) {
         if (a->layout == MG_TN) return fail(MG_ERR_ARG, "mg_gemm: the fused y16 output exists for layouts NN and NT only");
         if (a->nbatch != 1) return fail(MG_ERR_ARG, "mg_gemm: the fused y16 output needs nbatch == 1");
@@ -748,6 +756,8 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     p.Y = (uint16_t *)a.y16;
     p.ldy = a.ldy;
     p.act = a.act;
+    p.Z = a.z;
+    p.ldz = a.ldz;
     p.ws = nullptr;
     p.cnt = nullptr;
     p.stream_k = 0;

@@ -100,7 +100,7 @@ class Matmul:
         return m > 0 and n > 0 and k > 0
 
     def _args(self, a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side=False,
-              act=None, y16=None, ldy=None):
+              act=None, y16=None, ldy=None, z=None, ldz=None):
         if self.batched:
             nb = int(nbatch)
             sa, sb, sc = (int(s) for s in strides)
@@ -138,8 +138,18 @@ class Matmul:
         if side:
             ga.flags |= L.MG_FLAG_SIDE_STREAM
         if act not in L.ACTS:
-            raise VkError(f"{self.name}: unknown activation {act!r}; use None, 'gelu' or 'relu'")
+            raise VkError(f"{self.name}: unknown activation {act!r}; use None, 'gelu', 'relu', "
+                          f"'gelu_grad' or 'relu_grad'")
         ga.act = L.ACTS[act]
+        if ga.act >= L.MG_ACT_GELU_GRAD:
+            if z is None:
+                raise VkError(f"{self.name}: act={act!r} needs z= (the pre-activation, f32)")
+            ga.z = z.ptr
+            ga.ldz = int(ldz) if ldz is not None else n
+            if m > 0 and n > 0 and z.size < ((m - 1) * ga.ldz + n) * 4:
+                raise VkError(f"{self.name}: z buffer of {z.size} bytes is too small for {m}x{n} (pitch {ga.ldz})")
+        elif z is not None:
+            raise VkError(f"{self.name}: z= is only read with act='gelu_grad' or 'relu_grad'")
         if y16 is not None:
             ga.y16 = y16.ptr
             ga.ldy = int(ldy) if ldy is not None else n
@@ -159,17 +169,20 @@ class Matmul:
 
     def __call__(self, a, b, c, m, n, k, repeat=1, graph=None, nbatch=1, strides=(0, 0, 0),
                  *, bias=None, accumulate=False, lda=None, ldb=None, ldc=None, side=False,
-                 act=None, y16=None, ldy=None):
+                 act=None, y16=None, ldy=None, z=None, ldz=None):
         """side=True (recorded calls only) puts the GEMM on the device's side stream:
         it runs concurrently with the main stream between graph.fork() and graph.join().
         y16= (with act=None, 'gelu' or 'relu') makes the epilogue also write
         narrow(act(result)) in the input dtype, the separate bias_gelu pass of the
-        reference (kernels.py:709-718) folded into the GEMM; c may then be None."""
+        reference (kernels.py:709-718) folded into the GEMM; c may then be None.
+        act='gelu_grad' / 'relu_grad' with z= (f32 pre-activation of the layer below)
+        folds bias_gelu_bwd (kernels.py:720-739) into a dX GEMM instead: y16 and c
+        receive result * act'(z)."""
         lib, ctx = self.dev._lib, self.dev._ctx
         if side and graph is None:
             raise VkError(f"{self.name}: side=True needs graph= (eager calls wait for their result); "
                           f"use enqueue(..., side=True) between dev.side_fork() and dev.side_join()")
-        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy)
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz)
         if graph is not None:
             _check(lib.mg_gemm_check(C.byref(ga)), self.name)
             self._keep.append(ga)
@@ -177,7 +190,7 @@ class Matmul:
             def launch(ga=ga):
                 _check(lib.mg_gemm(ctx, C.byref(ga)), self.name)
 
-            graph.record(launch, [x for x in (a, b, c, y16) if x is not None], name=self.name,
+            graph.record(launch, [x for x in (a, b, c, y16, z) if x is not None], name=self.name,
                          bytes_hint=self.traffic_bytes(m, n, k, nbatch))
             nb_ = nbatch if self.batched else 1
             graph.mm_split.append((nb_ * 2 * (m * k + k * n), nb_ * m * n * 4))
@@ -201,9 +214,10 @@ class Matmul:
         return dt.value
 
     def enqueue(self, a, b, c, m, n, k, nbatch=1, strides=(0, 0, 0), *, bias=None,
-                accumulate=False, lda=None, ldb=None, ldc=None, side=False, act=None, y16=None, ldy=None):
+                accumulate=False, lda=None, ldb=None, ldc=None, side=False, act=None, y16=None, ldy=None,
+                z=None, ldz=None):
         """Launch without waiting (the stream keeps order); for pipelined callers."""
-        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy)
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz)
         _check(self.dev._lib.mg_gemm(self.dev._ctx, C.byref(ga)), self.name)
 
     def plan(self, m, n, k, nbatch=1, lda=None, ldb=None, ldc=None):
