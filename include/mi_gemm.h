@@ -87,6 +87,12 @@ typedef struct {
      * where z is that lower layer's pre-activation (m, n) in f32.  beta == 0 and no bias. */
     const float *z;        /* NULL unless act is a _GRAD form */
     int64_t ldz;           /* its row pitch in elements (>= n) */
+    /* With a _GRAD activation: NULL, or N floats that receive the column sums of g, the bias
+     * gradient of the layer below — col_sum (kernels.py:753-761; autograd.py:215) folded into
+     * the same epilogue.  colsum[c] += sum over rows of g[r][c], added with float atomics once
+     * per wavefront and column: clear it first unless accumulating over micro-batches; the
+     * order of the additions, and so the last bits, vary from run to run. */
+    float *colsum;
 } mg_gemm_args;
 
 /* The buffers of A and B end at their last element: row padding (ld beyond the stored

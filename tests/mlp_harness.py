@@ -6,9 +6,9 @@ from oracle import ref_mlp
 
 
 def build_pair(dev, batch, sizes, n_classes, pad, act="gelu", dtype="f16", seed=0, fuse_bias=False,
-               bias_std=0.1):
+               bias_std=0.1, fuse_colsum=False):
     from vkgrad_amd.autograd import MLP, Ctx
-    ctx = Ctx(dev, dtype=dtype, fuse_bias=fuse_bias)
+    ctx = Ctx(dev, dtype=dtype, fuse_bias=fuse_bias, fuse_colsum=fuse_colsum)
     model = MLP(ctx, batch, list(sizes), n_classes, pad_classes=pad, activation=act)
     Ws, bs = ref_mlp.he_init(list(sizes) + [pad], seed)
     rng = np.random.default_rng(seed + 77)
@@ -32,10 +32,11 @@ def upload_batch(ctx, batch, n_in, n_classes, seed, dtype):
 
 
 def run_curve(dev, steps=20, batch=128, sizes=(784, 512, 512), n_classes=10, pad=10, act="relu",
-              dtype="f16", fuse_bias=False, recorded=True, lr=1e-3):
+              dtype="f16", fuse_bias=False, recorded=True, lr=1e-3, fuse_colsum=False):
     """Train both models on one fixed synthetic batch; returns (device losses, numpy losses)."""
     from vkgrad_amd.autograd import AdamW, TrainStep
-    ctx, model, ref = build_pair(dev, batch, sizes, n_classes, pad, act, dtype, fuse_bias=fuse_bias)
+    ctx, model, ref = build_pair(dev, batch, sizes, n_classes, pad, act, dtype, fuse_bias=fuse_bias,
+                                 fuse_colsum=fuse_colsum)
     try:
         xb, yb, xf, y = upload_batch(ctx, batch, sizes[0], n_classes, 0, dtype)
         opt = AdamW(ctx, model.params(), lr=lr)

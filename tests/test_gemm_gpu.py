@@ -329,7 +329,9 @@ def test_fused_activation_gradient_output(dev, layout, dtype):
     ReLU (the factor is 0 or 1), within 1e-5 of the product's magnitude (f32) and two 16-bit
     ulps for GELU, whose derivative the device forms from one exponential; z has its own
     pitch, padding of y16 stays untouched, C may be omitted, tiles with and without a fused
-    variant and a K split through the workspace."""
+    variant and a K split through the workspace.  colsum (the reference's col_sum pass,
+    kernels.py:753-761, in the same epilogue) receives the column sums of that result on top
+    of what it held: exact for ReLU, where every term is an integer."""
     from oracle import ref_mlp as R
     from vkgrad_amd.kernels import Matmul
     from vkgrad_amd.vk import VkError
@@ -349,13 +351,28 @@ def test_fused_activation_gradient_output(dev, layout, dtype):
         g_ref = (prod.astype(np.float64) * R.dact_fn(z[:, :n].astype(np.float64), act)).astype(np.float32)
         ba, bb, bz = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), dev.buffer(z.nbytes, "device")
         bc, by = dev.buffer(m * n * 4, "device"), dev.buffer(m * ldy * 2, "device")
+        bs = dev.buffer(n * 4 + 8, "device")
         ba.upload(a); bb.upload(b); bz.upload(z)
+        s0 = np.concatenate([(np.arange(n) % 5 - 2).astype(np.float32), [np.float32(77.0), np.float32(78.0)]])
         mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype=dtype, tile=tile, split_k=split)
         try:
             for with_c in (True, False):
                 bc.upload(np.full((m, n), np.nan, np.float32))
                 by.upload(np.full((m, ldy), 0x7e01, np.uint16))
-                mm(ba, bb, bc if with_c else None, m, n, k, act=act + "_grad", y16=by, ldy=ldy, z=bz, ldz=ldz)
+                bs.upload(s0)
+                mm(ba, bb, bc if with_c else None, m, n, k, act=act + "_grad", y16=by, ldy=ldy, z=bz, ldz=ldz,
+                   colsum=bs if with_c else None)
+                sums = bs.download(np.float32, (n + 2,))
+                assert sums[n] == 77.0 and sums[n + 1] == 78.0, "wrote beyond N column sums"
+                if not with_c:
+                    assert np.array_equal(sums, s0), "column sums written although none were asked for"
+                elif act == "relu":
+                    # integers: exact in any order of addition
+                    assert np.array_equal(sums[:n], s0[:n] + g_ref.astype(np.float64).sum(0)), (m, n, k, tile, "colsum")
+                else:
+                    want = s0[:n] + g_ref.astype(np.float64).sum(0)
+                    bound = 1e-5 * np.maximum(np.abs(prod), 1.0).sum(0) + 1e-6 * np.abs(g_ref).sum(0)
+                    assert np.all(np.abs(sums[:n] - want) <= bound), (m, n, k, tile, np.abs(sums[:n] - want).max())
                 yfull = by.download(np.uint16, (m, ldy))
                 assert np.all(yfull[:, n:] == 0x7e01), "the padding between rows of y16 was written"
                 got16 = np.ascontiguousarray(yfull[:, :n])
@@ -375,7 +392,7 @@ def test_fused_activation_gradient_output(dev, layout, dtype):
                     assert np.all(np.abs(g32 - g_ref) <= 2 * ulp + tol), (m, n, k, tile, np.abs(g32 - g_ref).max())
         finally:
             mm.destroy()
-            for x in (ba, bb, bz, bc, by):
+            for x in (ba, bb, bz, bc, by, bs):
                 x.destroy()
     # misuse
     mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype=dtype)
@@ -383,6 +400,8 @@ def test_fused_activation_gradient_output(dev, layout, dtype):
     try:
         with pytest.raises(VkError):
             mm(buf, buf, buf, 64, 64, 64, act="gelu_grad", y16=buf)                          # no z
+        with pytest.raises(VkError):
+            mm(buf, buf, buf, 64, 64, 64, act="relu", y16=buf, colsum=buf)                   # column sums of a forward GEMM
         with pytest.raises(VkError):
             mm(buf, buf, buf, 64, 64, 64, act="gelu", y16=buf, z=buf)                        # z without a _grad activation
         with pytest.raises(VkError):

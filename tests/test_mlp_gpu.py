@@ -19,16 +19,20 @@ def relerr(a, b):
     return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-8))
 
 
+@pytest.mark.parametrize("fuse", ["separate passes", "epilogues", "epilogues + column sums"])
 @pytest.mark.parametrize("act", ["gelu", "relu"])
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-def test_loss_and_gradients(dev, act, dtype):
+def test_loss_and_gradients(dev, act, dtype, fuse):
+    """Two hidden layers, so that a dX GEMM with the activation derivative (and the bias
+    column sums) of the layer below in its epilogue is on the path when fused."""
     batch, n_in, n_hid, n_cls, pad = 16, 32, 16, 4, 16
-    ctx, model, ref = build_pair(dev, batch, (n_in, n_hid), n_cls, pad, act, dtype, seed=0)
+    ctx, model, ref = build_pair(dev, batch, (n_in, n_hid, n_hid), n_cls, pad, act, dtype, seed=0,
+                                 fuse_bias=fuse != "separate passes", fuse_colsum=fuse.endswith("sums"))
     try:
         xb, yb, xf, y = upload_batch(ctx, batch, n_in, n_cls, 0, dtype)
         loss = model.forward_backward(xb, yb)
         # independent float32 model (no 16-bit rounding): the reference's tolerances
-        pure = ref_mlp.RefMLP((n_in, n_hid), n_cls, pad, act=act, pure_f32=True)
+        pure = ref_mlp.RefMLP((n_in, n_hid, n_hid), n_cls, pad, act=act, pure_f32=True)
         pure.set_params(ref.W, ref.b)
         ploss, dW, db = pure.loss_and_grads(xf, y)
         tol_loss, tol_grad = (2e-3, 2e-2) if dtype == "f16" else (2e-2, 6e-2)   # bf16 has 3 fewer mantissa bits
@@ -61,13 +65,14 @@ def test_baseline_config_loss_curve(dev, fuse_bias):
     assert got[-1] < 0.5 * got[0], "not learning"
 
 
-@pytest.mark.parametrize("fuse_bias", [False, True])
-def test_reference_variant_loss_curve(dev, fuse_bias):
+@pytest.mark.parametrize("fuse_bias,fuse_colsum", [(False, False), (True, False), (True, True)])
+def test_reference_variant_loss_curve(dev, fuse_bias, fuse_colsum):
     """What examples.mnist --synthetic actually runs (mnist.py:124-128, 146-147):
     784 zero-padded to 1024 -> 256 -> 16 (10 real classes), GELU; with fuse_bias the
-    bias, GELU and narrowing happen in the forward GEMM's epilogue."""
+    bias, GELU and narrowing happen in the forward GEMM's epilogue and GELU' in the head's
+    dX epilogue, with fuse_colsum the hidden layer's bias gradient too."""
     got, want = run_curve(dev, steps=60, batch=128, sizes=(1024, 256), n_classes=10, pad=16,
-                          act="gelu", dtype="f16", fuse_bias=fuse_bias, recorded=True)
+                          act="gelu", dtype="f16", fuse_bias=fuse_bias, recorded=True, fuse_colsum=fuse_colsum)
     assert np.abs(got[:5] - want[:5]).max() < 2e-3
     assert np.abs(got - want).max() < 3e-2
 

@@ -35,7 +35,7 @@ class GemmArgs(C.Structure):
         ("split_k", C.c_int32), ("group_m", C.c_int32),
         ("flags", C.c_int32), ("act", C.c_int32),
         ("y16", C.c_void_p), ("ldy", C.c_int64),
-        ("z", C.c_void_p), ("ldz", C.c_int64),
+        ("z", C.c_void_p), ("ldz", C.c_int64), ("colsum", C.c_void_p),
     ]
 
 

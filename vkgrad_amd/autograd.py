@@ -49,12 +49,17 @@ def pick_config(m, n, k, trans_a=False, trans_b=False, min_groups=256):
 class Ctx:
     """Owns the device, the elementwise kernels and a matmul cache keyed by shape."""
 
-    def __init__(self, dev, tune=False, scalar_only=None, *, dtype="f16", fuse_bias=False):
+    def __init__(self, dev, tune=False, scalar_only=None, *, dtype="f16", fuse_bias=False, fuse_colsum=False):
+        """fuse_bias: bias, activation and narrowing (forward) and the activation derivative
+        (backward) run in the GEMM epilogues instead of separate passes.  fuse_colsum (with
+        fuse_bias): the bias gradients of the hidden layers are summed in the same backward
+        epilogue with float atomics - one pass less, last bits not reproducible."""
         if scalar_only:
             raise VkError("there is no scalar GEMM path on MI355X: MFMA is always present")
         self.dev = dev
         self.dtype = dtype
         self.fuse_bias = fuse_bias
+        self.fuse_colsum = bool(fuse_colsum and fuse_bias)
         self.K = make_kernels(dev, dtype)
         self.tune = tune
         self.scalar_only = False
@@ -167,6 +172,7 @@ class Linear:
         self.dx32 = ctx.buf(batch * in_f * 4) if need_dx else None
         self.x16 = None
         self._dz_ready = False   # set by the layer above when its dX epilogue wrote dz16 / dz32
+        self._db_ready = False   # ... and when it also summed this layer's bias gradient
 
     def forward(self, x16, tape, graph=None):
         c, K = self.ctx, self.ctx.K
@@ -215,7 +221,10 @@ class Linear:
         c.matmul(self.in_f, self.out_f, self.batch, trans_a=True)(
             self.x16, g16, self.W.g32, self.in_f, self.out_f, self.batch, graph=graph,
             accumulate=accumulate)
-        K["col_sum_acc" if accumulate else "col_sum"]([g32, self.b.g32], self.out_f, self.batch, graph=graph)
+        if self._db_ready:
+            self._db_ready = False
+        else:
+            K["col_sum_acc" if accumulate else "col_sum"]([g32, self.b.g32], self.out_f, self.batch, graph=graph)
 
         if not self.need_dx:
             return None, None
@@ -223,8 +232,16 @@ class Linear:
         mm = c.matmul(self.batch, self.in_f, self.out_f, trans_b=True)
         if (c.fuse_bias and below is not None and below.activation
                 and (below.batch, below.out_f) == (self.batch, self.in_f)):
-            mm(g16, self.W.w16, below.dz32, self.batch, self.in_f, self.out_f, graph=graph,
-               act=below.act + "_grad", z=below.z, y16=below.dz16)
+            if c.fuse_colsum:
+                # db of the layer below comes out of the same epilogue; dz32 is then not needed
+                if not accumulate:
+                    K["zero"]([below.b.g32], below.out_f, graph=graph)
+                mm(g16, self.W.w16, None, self.batch, self.in_f, self.out_f, graph=graph,
+                   act=below.act + "_grad", z=below.z, y16=below.dz16, colsum=below.b.g32)
+                below._db_ready = True
+            else:
+                mm(g16, self.W.w16, below.dz32, self.batch, self.in_f, self.out_f, graph=graph,
+                   act=below.act + "_grad", z=below.z, y16=below.dz16)
             below._dz_ready = True
             return below.dz16, below.dz32
         mm(g16, self.W.w16, self.dx32, self.batch, self.in_f, self.out_f, graph=graph)

@@ -64,6 +64,7 @@ struct GemmParams {
     int act;              // MG_ACT_*
     const float *Z;       // pre-activation for the _GRAD activations
     int64_t ldz;
+    float *colsum;        // column sums of the _GRAD result are added here (or NULL)
 };
 
 template <int DT>
@@ -396,6 +397,9 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, float *C, f32x16
     auto write_out = [&](auto mode_c, auto edge_c) {
         constexpr int MODE = decltype(mode_c)::value;   // 0 overwrite, 1 C += , 2 atomic +=
         constexpr bool EDGE = decltype(edge_c)::value != 0;
+        float cs[TN];   // this lane's share of the column sums (one column per j)
+#pragma unroll
+        for (int j = 0; j < TN; j++) cs[j] = 0.f;
 #pragma unroll
         for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -430,7 +434,10 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, float *C, f32x16
                     float v = acc[i][j][r] + bv[j];
                     if constexpr (MODE == 1) v = old[r] + v;
                     if constexpr (ACT && MODE == 0) {
-                        if (grad) v *= fused_dact(old[r], p.act);
+                        if (grad) {
+                            v *= fused_dact(old[r], p.act);
+                            cs[j] += ok ? v : 0.f;
+                        }
                     }
                     if (ok) {
                         if constexpr (MODE == 2) {
@@ -440,6 +447,17 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, float *C, f32x16
                             if constexpr (ACT) yt[ro * ldy] = narrow16_rne<DT>(fused_act(v, p.act));
                         }
                     }
+                }
+            }
+        }
+        if constexpr (ACT && MODE == 0) {
+            if (grad && p.colsum != nullptr) {
+                // the two half-waves hold different rows of the same 32 columns
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const float s = cs[j] + __shfl_xor(cs[j], 32, 64);
+                    if (lane < 32 && col_l + j * 32 < p.N)
+                        __hip_atomic_fetch_add(p.colsum + col_l + j * 32, s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
         }

@@ -392,8 +392,9 @@ static int check_args(const mg_gemm_args *a) {
         if ((uintptr_t)a->z & 3) return fail(MG_ERR_ARG, "mg_gemm: z must be 4-byte aligned");
         if (a->ldz < a->n) return fail(MG_ERR_ARG, "mg_gemm: ldz %lld < N %lld", (long long)a->ldz, (long long)a->n);
         if (a->beta != 0 || a->bias) return fail(MG_ERR_ARG, "mg_gemm: a _GRAD activation needs beta == 0 and no bias");
-    } else if (a->z) {
-        return fail(MG_ERR_ARG, "mg_gemm: z is only read by the _GRAD activations");
+        if ((uintptr_t)a->colsum & 3) return fail(MG_ERR_ARG, "mg_gemm: colsum must be 4-byte aligned");
+    } else if (a->z || a->colsum) {
+        return fail(MG_ERR_ARG, "mg_gemm: z and colsum belong to the _GRAD activations");
     }
     if (a->y16) {
         if (a->layout == MG_TN) return fail(MG_ERR_ARG, "mg_gemm: the fused y16 output exists for layouts NN and NT only");
@@ -758,6 +759,7 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     p.act = a.act;
     p.Z = a.z;
     p.ldz = a.ldz;
+    p.colsum = a.colsum;
     p.ws = nullptr;
     p.cnt = nullptr;
     p.stream_k = 0;

@@ -100,7 +100,7 @@ class Matmul:
         return m > 0 and n > 0 and k > 0
 
     def _args(self, a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side=False,
-              act=None, y16=None, ldy=None, z=None, ldz=None):
+              act=None, y16=None, ldy=None, z=None, ldz=None, colsum=None):
         if self.batched:
             nb = int(nbatch)
             sa, sb, sc = (int(s) for s in strides)
@@ -148,8 +148,12 @@ class Matmul:
             ga.ldz = int(ldz) if ldz is not None else n
             if m > 0 and n > 0 and z.size < ((m - 1) * ga.ldz + n) * 4:
                 raise VkError(f"{self.name}: z buffer of {z.size} bytes is too small for {m}x{n} (pitch {ga.ldz})")
-        elif z is not None:
-            raise VkError(f"{self.name}: z= is only read with act='gelu_grad' or 'relu_grad'")
+            if colsum is not None:
+                if colsum.size < n * 4:
+                    raise VkError(f"{self.name}: colsum buffer of {colsum.size} bytes is shorter than N={n} floats")
+                ga.colsum = colsum.ptr
+        elif z is not None or colsum is not None:
+            raise VkError(f"{self.name}: z= and colsum= belong to act='gelu_grad' or 'relu_grad'")
         if y16 is not None:
             ga.y16 = y16.ptr
             ga.ldy = int(ldy) if ldy is not None else n
@@ -169,7 +173,7 @@ class Matmul:
 
     def __call__(self, a, b, c, m, n, k, repeat=1, graph=None, nbatch=1, strides=(0, 0, 0),
                  *, bias=None, accumulate=False, lda=None, ldb=None, ldc=None, side=False,
-                 act=None, y16=None, ldy=None, z=None, ldz=None):
+                 act=None, y16=None, ldy=None, z=None, ldz=None, colsum=None):
         """side=True (recorded calls only) puts the GEMM on the device's side stream:
         it runs concurrently with the main stream between graph.fork() and graph.join().
         y16= (with act=None, 'gelu' or 'relu') makes the epilogue also write
@@ -177,12 +181,13 @@ class Matmul:
         reference (kernels.py:709-718) folded into the GEMM; c may then be None.
         act='gelu_grad' / 'relu_grad' with z= (f32 pre-activation of the layer below)
         folds bias_gelu_bwd (kernels.py:720-739) into a dX GEMM instead: y16 and c
-        receive result * act'(z)."""
+        receive g = result * act'(z), and colsum= (N floats, cleared by the caller unless
+        accumulating) has the column sums of g added to it (col_sum, kernels.py:753-761)."""
         lib, ctx = self.dev._lib, self.dev._ctx
         if side and graph is None:
             raise VkError(f"{self.name}: side=True needs graph= (eager calls wait for their result); "
                           f"use enqueue(..., side=True) between dev.side_fork() and dev.side_join()")
-        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz)
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz, colsum)
         if graph is not None:
             _check(lib.mg_gemm_check(C.byref(ga)), self.name)
             self._keep.append(ga)
@@ -190,7 +195,7 @@ class Matmul:
             def launch(ga=ga):
                 _check(lib.mg_gemm(ctx, C.byref(ga)), self.name)
 
-            graph.record(launch, [x for x in (a, b, c, y16, z) if x is not None], name=self.name,
+            graph.record(launch, [x for x in (a, b, c, y16, z, colsum) if x is not None], name=self.name,
                          bytes_hint=self.traffic_bytes(m, n, k, nbatch))
             nb_ = nbatch if self.batched else 1
             graph.mm_split.append((nb_ * 2 * (m * k + k * n), nb_ * m * n * 4))
@@ -215,9 +220,9 @@ class Matmul:
 
     def enqueue(self, a, b, c, m, n, k, nbatch=1, strides=(0, 0, 0), *, bias=None,
                 accumulate=False, lda=None, ldb=None, ldc=None, side=False, act=None, y16=None, ldy=None,
-                z=None, ldz=None):
+                z=None, ldz=None, colsum=None):
         """Launch without waiting (the stream keeps order); for pipelined callers."""
-        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz)
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz, colsum)
         _check(self.dev._lib.mg_gemm(self.dev._ctx, C.byref(ga)), self.name)
 
     def plan(self, m, n, k, nbatch=1, lda=None, ldb=None, ldc=None):
