@@ -93,6 +93,13 @@ typedef struct {
      * per wavefront and column: clear it first unless accumulating over micro-batches; the
      * order of the additions, and so the last bits, vary from run to run. */
     float *colsum;
+    /* Residual epilogue — replaces the separate pass of `residual` (tkernels.py:362-371; its
+     * call sites transformer.py:216, 223): with beta == 1 and res given,
+     *   C = res + result (+ bias),
+     * i.e. the accumulation reads another (m, n) f32 matrix than the one it writes (res == c
+     * is the plain in-place beta == 1).  nbatch == 1; MG_FLAG_SPLITK_ATOMIC is refused. */
+    const float *res;      /* NULL: beta == 1 reads C itself */
+    int64_t ldr;           /* row pitch of res in elements (>= n) */
 } mg_gemm_args;
 
 /* The buffers of A and B end at their last element: row padding (ld beyond the stored

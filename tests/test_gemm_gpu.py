@@ -415,6 +415,59 @@ def test_fused_activation_gradient_output(dev, layout, dtype):
         buf.destroy()
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
+def test_residual_epilogue(dev, layout, dtype):
+    """C = res + A.B + bias with res another matrix than C (the reference's `residual` pass,
+    tkernels.py:362-371, after the projection GEMMs, transformer.py:216, 223): exact on
+    integer data for register-staged, direct-to-LDS, persistent (which hand over: their
+    beta = 1 is an atomic add into C), stream-K and skinny tiles, with a K split through the
+    workspace, ragged shapes and a padded res pitch; res itself stays untouched, and
+    res == C is the plain in-place accumulation."""
+    from vkgrad_amd.kernels import Matmul
+    from vkgrad_amd.vk import VkError
+    ta, tb = LAYOUTS[layout]
+    cases = [(200, 136, 320, None, 0), (512, 384, 256, 11, 0), (1000, 1016, 1024, 10, 0), (392, 648, 2048, 11, 4),
+             (129, 96, 768, 4, 3), (512, 768, 512, 15, 0), (640, 384, 1024, 18, 0), (4, 300, 768, 20, 0),
+             (77, 50, 72, 0, 0), (512, 512, 4096, 17, 4)]
+    for m, n, k, tile, split in cases:
+        a, b = O.make_operands(m, n, k, ta, tb, dtype, seed=m + k, integer=True)
+        bias = (np.arange(n) % 7 - 3).astype(np.float32)
+        ldr = n + 5
+        rng = np.random.default_rng(n)
+        res = np.full((m, ldr), np.nan, np.float32)
+        res[:, :n] = rng.integers(-50, 50, (m, n)).astype(np.float32)
+        want = O.ref_gemm(a, b, ta, tb, dtype, bias, np.ascontiguousarray(res[:, :n]))
+        ba, bb, bz = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), dev.buffer(n * 4, "device")
+        bc, br = dev.buffer(m * n * 4, "device"), dev.buffer(res.nbytes, "device")
+        ba.upload(a); bb.upload(b); bz.upload(bias); br.upload(res)
+        bc.upload(np.full((m, n), np.nan, np.float32))
+        mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype=dtype, tile=tile, split_k=split)
+        try:
+            mm(ba, bb, bc, m, n, k, bias=bz, res=br, ldr=ldr)
+            assert np.array_equal(bc.download(np.float32, (m, n)), want), (layout, m, n, k, tile, split)
+            back = br.download(np.float32, (m, ldr))
+            assert np.array_equal(back[:, :n], res[:, :n]) and np.isnan(back[:, n:]).all(), "res was written"
+            # res == C: in place, the same as accumulate=True
+            bc.upload(np.ascontiguousarray(res[:, :n]))
+            mm(ba, bb, bc, m, n, k, bias=bz, res=bc)
+            assert np.array_equal(bc.download(np.float32, (m, n)), want), (layout, m, n, k, tile, "in place")
+        finally:
+            mm.destroy()
+            for x in (ba, bb, bz, bc, br):
+                x.destroy()
+    buf = dev.buffer(64 * 64 * 4, "device")
+    mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype=dtype, split_k=2, atomic_split=True)
+    try:
+        with pytest.raises(VkError):
+            mm(buf, buf, buf, 64, 64, 64, res=buf)              # atomic slices have nothing to add res once
+        with pytest.raises(VkError):
+            mm(buf, buf, buf, 64, 64, 64, res=buf, ldr=60)      # pitch below N
+    finally:
+        mm.destroy()
+        buf.destroy()
+
+
 def test_timing_over_rotating_operand_sets(dev):
     """The rotating timer launches argument set i % nsets on launch i: after seven
     launches over three sets with different integer operands, every set's C holds

@@ -36,6 +36,7 @@ class GemmArgs(C.Structure):
         ("flags", C.c_int32), ("act", C.c_int32),
         ("y16", C.c_void_p), ("ldy", C.c_int64),
         ("z", C.c_void_p), ("ldz", C.c_int64), ("colsum", C.c_void_p),
+        ("res", C.c_void_p), ("ldr", C.c_int64),
     ]
 
 

@@ -65,6 +65,8 @@ struct GemmParams {
     const float *Z;       // pre-activation for the _GRAD activations
     int64_t ldz;
     float *colsum;        // column sums of the _GRAD result are added here (or NULL)
+    const float *R;       // beta = 1 reads this matrix instead of C (or NULL)
+    int64_t ldr;
 };
 
 template <int DT>
@@ -388,6 +390,9 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, float *C, f32x16
     const int64_t ldy = ACT ? p.ldy : 0;
     const bool have_c = !ACT || C != nullptr;
     const bool grad = ACT && p.act >= 3;
+    // what beta = 1 adds to: C itself, or the residual matrix
+    const float *rl = p.R ? p.R + (int64_t)row_l * p.ldr + col_l : cl;
+    const int64_t ldr = p.R ? p.ldr : ldc;
     const float *zl = grad ? p.Z + (int64_t)row_l * p.ldz + col_l : nullptr;
     const int64_t ldz = grad ? p.ldz : 0;
     float bv[TN];
@@ -409,11 +414,12 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, float *C, f32x16
                 const bool col_ok = !EDGE || (col_l + j * 32 < p.N);
                 float old[16];
                 if constexpr (MODE == 1) {
+                    const float *rt = rl + (int64_t)(i * 32) * ldr + j * 32;
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
                         const int ro = (r >> 2) * 8 + (r & 3);
                         const bool ok = col_ok && (!EDGE || row_l + i * 32 + ro < p.M);
-                        old[r] = ok ? ct[ro * ldc] : 0.f;
+                        old[r] = ok ? rt[ro * ldr] : 0.f;
                     }
                 }
                 if constexpr (ACT && MODE == 0) {

@@ -140,6 +140,7 @@ static bool gemv_eligible(const mg_gemm_args &a, int split) {
     if (((uintptr_t)a.a | (uintptr_t)a.b) & 15) return false;
     if ((a.lda | a.ldb | a.k) & 7) return false;
     if (a.nbatch > 1 && ((a.sa | a.sb) & 7)) return false;
+    if (a.res && a.res != a.c) return false;   // its beta = 1 reads C
     return true;
 }
 
@@ -160,6 +161,7 @@ static bool dma_eligible(const mg_gemm_args &a, const TileDesc &t, int64_t k_per
     if (ragged && (a.flags & MG_FLAG_TIGHT_BUFFERS)) return false;
     if (t.persistent) {
         if (a.k % t.bk != 0 || k_per_split % t.bk != 0) return false;
+        if (a.res && a.res != a.c) return false;   // their beta = 1 is an atomic add into C
     }
     if (t.persistent == 2 && split > 1) return false;   // stream-K cuts K itself
     // the 256 x 256 stream-K kernel with the bias epilogue does not fit the register file
@@ -403,6 +405,14 @@ static int check_args(const mg_gemm_args *a) {
         if (a->ldy < a->n) return fail(MG_ERR_ARG, "mg_gemm: ldy %lld < N %lld", (long long)a->ldy, (long long)a->n);
         if (a->flags & MG_FLAG_SPLITK_ATOMIC)
             return fail(MG_ERR_ARG, "mg_gemm: the fused y16 output cannot be combined with MG_FLAG_SPLITK_ATOMIC");
+    }
+    if (a->res) {
+        if (a->beta != 1) return fail(MG_ERR_ARG, "mg_gemm: res is what beta == 1 adds to; beta is %d", a->beta);
+        if ((uintptr_t)a->res & 3) return fail(MG_ERR_ARG, "mg_gemm: res must be 4-byte aligned");
+        if (a->ldr < a->n) return fail(MG_ERR_ARG, "mg_gemm: ldr %lld < N %lld", (long long)a->ldr, (long long)a->n);
+        if (a->nbatch != 1) return fail(MG_ERR_ARG, "mg_gemm: res needs nbatch == 1");
+        if (a->flags & MG_FLAG_SPLITK_ATOMIC)
+            return fail(MG_ERR_ARG, "mg_gemm: res cannot be combined with MG_FLAG_SPLITK_ATOMIC");
     }
     if (((uintptr_t)a->a | (uintptr_t)a->b) & 1) return fail(MG_ERR_ARG, "mg_gemm: A and B must be 2-byte aligned");
     if ((uintptr_t)a->c & 3) return fail(MG_ERR_ARG, "mg_gemm: C must be 4-byte aligned");
@@ -760,6 +770,8 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     p.Z = a.z;
     p.ldz = a.ldz;
     p.colsum = a.colsum;
+    p.R = (a.res && a.res != a.c) ? a.res : nullptr;
+    p.ldr = a.ldr;
     p.ws = nullptr;
     p.cnt = nullptr;
     p.stream_k = 0;
@@ -773,9 +785,9 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
             p.ws = lane_ws;
             p.cnt = lane_cnt;
         }
-        if (a.y16 && !p.ws) {
-            // the activation is applied once, to the finished sum: without a workspace for the
-            // slices to meet in, the same GEMM runs unsplit
+        if ((a.y16 || p.R) && !p.ws) {
+            // the activation is applied once, to the finished sum, and the residual is added
+            // once: without a workspace for the slices to meet in, the same GEMM runs unsplit
             mg_gemm_args whole = a;
             whole.split_k = 1;
             Plan unsplit;

@@ -100,7 +100,7 @@ class Matmul:
         return m > 0 and n > 0 and k > 0
 
     def _args(self, a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side=False,
-              act=None, y16=None, ldy=None, z=None, ldz=None, colsum=None):
+              act=None, y16=None, ldy=None, z=None, ldz=None, colsum=None, res=None, ldr=None):
         if self.batched:
             nb = int(nbatch)
             sa, sb, sc = (int(s) for s in strides)
@@ -163,6 +163,14 @@ class Matmul:
             raise VkError(f"{self.name}: act= needs y16= (the activated 16-bit output)")
         if c is None and y16 is None:
             raise VkError(f"{self.name}: C may only be omitted when y16 is given")
+        if res is not None:
+            if c is None:
+                raise VkError(f"{self.name}: res= needs C (C = res + result)")
+            ga.beta = 1
+            ga.res = res.ptr
+            ga.ldr = int(ldr) if ldr is not None else n
+            if m > 0 and n > 0 and res.size < ((m - 1) * ga.ldr + n) * 4:
+                raise VkError(f"{self.name}: res buffer of {res.size} bytes is too small for {m}x{n} (pitch {ga.ldr})")
         if m > 0 and n > 0 and k > 0:
             if need_a > a.size or need_b > b.size or (c is not None and need_c > c.size):
                 raise VkError(f"{self.name}: shape {m}x{n}x{k} (nbatch {nb}) needs {need_a}/{need_b}/{need_c} "
@@ -173,7 +181,7 @@ class Matmul:
 
     def __call__(self, a, b, c, m, n, k, repeat=1, graph=None, nbatch=1, strides=(0, 0, 0),
                  *, bias=None, accumulate=False, lda=None, ldb=None, ldc=None, side=False,
-                 act=None, y16=None, ldy=None, z=None, ldz=None, colsum=None):
+                 act=None, y16=None, ldy=None, z=None, ldz=None, colsum=None, res=None, ldr=None):
         """side=True (recorded calls only) puts the GEMM on the device's side stream:
         it runs concurrently with the main stream between graph.fork() and graph.join().
         y16= (with act=None, 'gelu' or 'relu') makes the epilogue also write
@@ -182,12 +190,14 @@ class Matmul:
         act='gelu_grad' / 'relu_grad' with z= (f32 pre-activation of the layer below)
         folds bias_gelu_bwd (kernels.py:720-739) into a dX GEMM instead: y16 and c
         receive g = result * act'(z), and colsum= (N floats, cleared by the caller unless
-        accumulating) has the column sums of g added to it (col_sum, kernels.py:753-761)."""
+        accumulating) has the column sums of g added to it (col_sum, kernels.py:753-761).
+        res= (an (m, n) f32 matrix) makes it C = res + result (+ bias): the `residual`
+        pass of the reference's transformer (tkernels.py:362-371) in the epilogue."""
         lib, ctx = self.dev._lib, self.dev._ctx
         if side and graph is None:
             raise VkError(f"{self.name}: side=True needs graph= (eager calls wait for their result); "
                           f"use enqueue(..., side=True) between dev.side_fork() and dev.side_join()")
-        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz, colsum)
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz, colsum, res, ldr)
         if graph is not None:
             _check(lib.mg_gemm_check(C.byref(ga)), self.name)
             self._keep.append(ga)
@@ -195,7 +205,7 @@ class Matmul:
             def launch(ga=ga):
                 _check(lib.mg_gemm(ctx, C.byref(ga)), self.name)
 
-            graph.record(launch, [x for x in (a, b, c, y16, z, colsum) if x is not None], name=self.name,
+            graph.record(launch, [x for x in (a, b, c, y16, z, colsum, res) if x is not None], name=self.name,
                          bytes_hint=self.traffic_bytes(m, n, k, nbatch))
             nb_ = nbatch if self.batched else 1
             graph.mm_split.append((nb_ * 2 * (m * k + k * n), nb_ * m * n * 4))
@@ -220,9 +230,9 @@ class Matmul:
 
     def enqueue(self, a, b, c, m, n, k, nbatch=1, strides=(0, 0, 0), *, bias=None,
                 accumulate=False, lda=None, ldb=None, ldc=None, side=False, act=None, y16=None, ldy=None,
-                z=None, ldz=None, colsum=None):
+                z=None, ldz=None, colsum=None, res=None, ldr=None):
         """Launch without waiting (the stream keeps order); for pipelined callers."""
-        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz, colsum)
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz, colsum, res, ldr)
         _check(self.dev._lib.mg_gemm(self.dev._ctx, C.byref(ga)), self.name)
 
     def plan(self, m, n, k, nbatch=1, lda=None, ldb=None, ldc=None):
