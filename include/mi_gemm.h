@@ -266,6 +266,61 @@ int mg_ew_fill_uniform16(mg_ctx *ctx, void *dst, int64_t n, uint32_t seed, int d
 /* grad_add (dataparallel.py:54-58): dst[i] += src[i] */
 int mg_ew_grad_add(mg_ctx *ctx, float *dst, const float *src, int64_t n);
 
+/* ---- Row kernels of the decoder block (tkernels.py), all in f32 with 16-bit outputs where the
+ * next GEMM reads them.  `dtype` is the 16-bit type.  Head-side tensors are (B*H, T, hd),
+ * row-side tensors (B*T, D) with D = H * hd; n counts the elements of the (B*T, D) side. */
+/* layernorm (tkernels.py:32-56): y16 = narrow((x - mu) * rstd * gamma + beta), eps 1e-5 inside
+ * the root; mu and rstd (one per row) are kept for the backward pass. */
+int mg_tk_layernorm(mg_ctx *ctx, const float *x, const float *gamma, const float *beta, void *y16, float *mu,
+                    float *rstd, int64_t rows, int64_t D, int dtype);
+/* layernorm_bwd (tkernels.py:58-92): dx, plus dy * xhat and dy in 16 bits (the column sums of
+ * those two are dgamma and dbeta, transformer.py:66-73). */
+int mg_tk_layernorm_bwd(mg_ctx *ctx, const float *dy, const float *x, const float *gamma, const float *mu,
+                        const float *rstd, float *dx, void *dyxh16, void *dy16, int64_t rows, int64_t D, int dtype);
+/* attn_softmax / attn_softmax_doc (tkernels.py:105-165): rows = B*H*T rows of T scores; row r is
+ * query r % T and sees keys first..query, first = 0 or seg[(r / T / H) * T + query]; scale, max
+ * subtraction and normalisation in one kernel, masked keys get 0. */
+int mg_tk_attn_softmax(mg_ctx *ctx, const float *s, const uint32_t *seg, void *p16, int64_t rows, int64_t T, int64_t H,
+                       float scale, int dtype);
+/* attn_softmax_bwd (tkernels.py:167-187): ds16 = narrow(P * (dP - sum_j dP_j P_j) * scale) */
+int mg_tk_attn_softmax_bwd(mg_ctx *ctx, const float *dp, const void *p16, void *ds16, int64_t rows, int64_t T,
+                           float scale, int dtype);
+/* split_qkv (tkernels.py:195-213): (B*T, 3D) f32 + bias[3D] (or NULL) -> q16, k16, v16 head-side */
+int mg_tk_split_qkv(mg_ctx *ctx, const float *qkv, const float *bias, void *q16, void *k16, void *v16, int64_t n,
+                    int64_t D, int64_t T, int64_t H, int64_t hd, int dtype);
+/* merge_qkv_grad (tkernels.py:215-231): head-side dq, dk, dv f32 -> (B*T, 3D) 16-bit */
+int mg_tk_merge_qkv_grad(mg_ctx *ctx, const float *dq, const float *dk, const float *dv, void *dqkv16, int64_t n,
+                         int64_t D, int64_t T, int64_t H, int64_t hd, int dtype);
+/* merge_heads (tkernels.py:274-286): head-side f32 -> (B*T, D) 16-bit */
+int mg_tk_merge_heads(mg_ctx *ctx, const float *src, void *y16, int64_t n, int64_t D, int64_t T, int64_t H, int64_t hd,
+                      int dtype);
+/* split_heads (tkernels.py:288-300): (B*T, D) f32 -> head-side 16-bit */
+int mg_tk_split_heads(mg_ctx *ctx, const float *src, void *dst16, int64_t n, int64_t D, int64_t T, int64_t H,
+                      int64_t hd, int dtype);
+/* embed / embed_doc (tkernels.py:303-315, 334-345): x[bt, d] = tok[ids[bt], d] + pos[t, d],
+ * t = bt % T, minus seg[bt] when seg is given (positions restart at each packed sample). */
+int mg_tk_embed(mg_ctx *ctx, const float *tok, const float *pos, const uint32_t *ids, const uint32_t *seg, float *x,
+                int64_t n, int64_t D, int64_t T);
+/* embed_bwd / embed_doc_bwd (tkernels.py:317-332, 347-360): scatter-add of dx into dtok and dpos
+ * with float atomics; the caller clears (or has a GEMM overwrite) both first. */
+int mg_tk_embed_bwd(mg_ctx *ctx, const float *dx, const uint32_t *ids, const uint32_t *seg, float *dtok, float *dpos,
+                    int64_t n, int64_t D, int64_t T);
+/* residual (tkernels.py:362-371): out = res + acc + bias[i % D] — the separate-pass form of
+ * mg_gemm_args.res */
+int mg_tk_residual(mg_ctx *ctx, const float *acc, const float *bias, const float *res, float *out, int64_t n,
+                   int64_t D);
+/* add (tkernels.py:373-377) and add_bias (in place, tkernels.py:379-382) */
+int mg_tk_add(mg_ctx *ctx, const float *a, const float *b, float *out, int64_t n);
+int mg_tk_add_bias(mg_ctx *ctx, float *x, const float *bias, int64_t n, int64_t ncol);
+/* col_sum_zero + col_sum_chunk16 (tkernels.py:238-270; transformer.py:30-37): column sums of a
+ * 16-bit (nrow, ncol) matrix, f32 accumulation; accumulate != 0 adds to sums. */
+int mg_tk_col_sum16(mg_ctx *ctx, const void *g16, float *sums, int64_t ncol, int64_t nrow, int accumulate, int dtype);
+/* softmax_ce / softmax_ce_w (kernels.py:766-823) for wide rows (the LM head): one workgroup per
+ * row.  weights NULL: gradient scaled by 1 / nrows; else by weights[row], rows of weight 0 get
+ * zeros and loss 0.  dl16 or dl32 may be NULL. */
+int mg_tk_softmax_ce(mg_ctx *ctx, const float *logits, const uint32_t *labels, const float *weights, void *dl16,
+                     float *dl32, float *loss, int64_t nrows, int64_t stride, int64_t ncls, int dtype);
+
 #ifdef __cplusplus
 }
 #endif

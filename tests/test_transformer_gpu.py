@@ -1,0 +1,237 @@
+"""GPU parity of the decoder-block row kernels and of a whole GPT step.
+
+Kernels are called by the reference's names and call shapes through
+vkgrad_amd.tkernels (the C entry points mg_tk_*) and compared with
+oracle/ref_transformer.py; the whole model follows the protocol of
+/root/reference/test_transformer.py (loss within 5e-3, every gradient tensor
+within 3e-2 of its largest entry, against an independent numpy model; tied and
+untied head; packed samples with loss weights and one graph per stage)."""
+
+import numpy as np
+import pytest
+
+from oracle import ref_gemm as O
+from oracle import ref_transformer as RT
+
+pytestmark = pytest.mark.gpu
+
+ULP = {"f16": 2.0 ** -10, "bf16": 2.0 ** -7}
+
+
+def close16(got_stored, want_stored, dtype, slack=0.0):
+    """16-bit results may differ by one rounding step where the f32 values before rounding
+    differ in their last bits."""
+    g, w = O.widen(got_stored, dtype), O.widen(want_stored, dtype)
+    return bool(np.all(np.abs(g - w) <= ULP[dtype] * np.maximum(np.abs(w), 2.0 ** -14) + slack))
+
+
+def up(dev, arr):
+    b = dev.buffer(max(arr.nbytes, 4), "device")
+    b.upload(np.ascontiguousarray(arr))
+    return b
+
+
+def stored(buf, dtype, shape):
+    raw = buf.download(np.uint16, shape)
+    return raw.view(np.float16) if dtype == "f16" else raw
+
+
+@pytest.fixture(scope="module", params=["f16", "bf16"])
+def tk(request, dev):
+    from vkgrad_amd.tkernels import make_transformer_kernels
+    return request.param, make_transformer_kernels(dev, request.param)
+
+
+def test_layernorm_forward_backward(dev, tk):
+    dtype, TK = tk
+    W = dev.row_subgroup_size
+    rng = np.random.default_rng(0)
+    for rows, D in ((5, 48), (64, 768), (33, 100), (2, 1)):
+        x = (rng.standard_normal((rows, D)) * 2 + 1).astype(np.float32)
+        g = rng.uniform(0.5, 1.5, D).astype(np.float32)
+        b = rng.standard_normal(D).astype(np.float32)
+        dy = rng.standard_normal((rows, D)).astype(np.float32)
+        bx, bg, bb, bdy = up(dev, x), up(dev, g), up(dev, b), up(dev, dy)
+        by, bmu, brs = dev.buffer(rows * D * 2, "device"), dev.buffer(rows * 4, "device"), dev.buffer(rows * 4, "device")
+        bdx, bxh, bd16 = dev.buffer(rows * D * 4, "device"), dev.buffer(rows * D * 2, "device"), dev.buffer(rows * D * 2, "device")
+        bufs = [bx, bg, bb, bdy, by, bmu, brs, bdx, bxh, bd16]
+        try:
+            TK["layernorm"]([bx, bg, bb, by, bmu, brs], rows * W, D)
+            y16, mu, rstd = RT.layernorm(x, g, b, dtype)
+            gmu, grs = bmu.download(np.float32, (rows,)), brs.download(np.float32, (rows,))
+            assert np.allclose(gmu, mu, atol=1e-5) and np.allclose(grs, rstd, rtol=2e-5)
+            assert close16(stored(by, dtype, (rows, D)), y16, dtype, slack=2e-5)
+            TK["layernorm_bwd"]([bdy, bx, bg, bmu, brs, bdx, bxh, bd16], rows * W, D)
+            dx, dyxh16, dy16 = RT.layernorm_bwd(dy, x, g, gmu, grs, dtype)
+            assert np.abs(bdx.download(np.float32, (rows, D)) - dx).max() <= 1e-4 * max(1.0, np.abs(dx).max())
+            assert close16(stored(bxh, dtype, (rows, D)), dyxh16, dtype, slack=1e-5)
+            assert np.array_equal(stored(bd16, dtype, (rows, D)).view(np.uint16), dy16.view(np.uint16))
+        finally:
+            for t in bufs:
+                t.destroy()
+
+
+def test_attention_softmax_forward_backward(dev, tk):
+    dtype, TK = tk
+    W = dev.row_subgroup_size
+    rng = np.random.default_rng(1)
+    for B, H, T in ((1, 2, 16), (2, 3, 70), (1, 1, 200)):
+        rows = B * H * T
+        s = (rng.standard_normal((rows, T)) * 3).astype(np.float32)
+        s[:, T // 2:] += np.where(rng.random((rows, T - T // 2)) < 0.1, 1e4, 0).astype(np.float32)   # masked junk must not leak
+        seg = np.zeros(B * T, np.uint32)
+        for b in range(B):
+            cut = 1 + (7 * b + T // 3) % (T - 1)
+            seg[b * T + cut:(b + 1) * T] = cut
+        dp = rng.standard_normal((rows, T)).astype(np.float32)
+        scale = 1.0 / np.sqrt(8.0)
+        bs, bseg, bdp = up(dev, s), up(dev, seg), up(dev, dp)
+        bp, bds = dev.buffer(rows * T * 2, "device"), dev.buffer(rows * T * 2, "device")
+        try:
+            # junk beyond the diagonal only: keep the visible scores tame
+            tri = np.arange(T)[None, :] <= (np.arange(rows) % T)[:, None]
+            s_vis = np.where(tri, np.minimum(s, 50.0), s).astype(np.float32)
+            bs.upload(s_vis)
+            TK["attn_softmax"]([bs, bp], rows * W, T, scale)
+            want = RT.attn_softmax(s_vis, T, scale, dtype)
+            got = stored(bp, dtype, (rows, T))
+            assert close16(got, want, dtype, slack=2e-6)
+            assert not O.widen(got, dtype)[~tri].any()
+            TK["attn_softmax_bwd"]([bdp, bp, bds], rows * W, T, scale)
+            want_ds = RT.attn_softmax_bwd(dp, got, T, scale, dtype)
+            assert close16(stored(bds, dtype, (rows, T)), want_ds, dtype, slack=2e-5)
+            TK["attn_softmax_doc"]([bs, bseg, bp], rows * W, T, H, scale)
+            want = RT.attn_softmax(s_vis, T, scale, dtype, seg=seg, H=H)
+            assert close16(stored(bp, dtype, (rows, T)), want, dtype, slack=2e-6)
+        finally:
+            for t in (bs, bseg, bdp, bp, bds):
+                t.destroy()
+
+
+def test_head_permutes(dev, tk):
+    dtype, TK = tk
+    rng = np.random.default_rng(2)
+    for B, T, H, hd in ((2, 5, 3, 4), (1, 64, 12, 64)):
+        D, rows = H * hd, B * T
+        qkv = rng.standard_normal((rows, 3 * D)).astype(np.float32)
+        bias = rng.standard_normal(3 * D).astype(np.float32)
+        bq, bb = up(dev, qkv), up(dev, bias)
+        outs = [dev.buffer(rows * D * 2, "device") for _ in range(3)]
+        heads32 = [rng.standard_normal((B * H, T, hd)).astype(np.float32) for _ in range(3)]
+        hb = [up(dev, h) for h in heads32]
+        bm, bx = dev.buffer(rows * 3 * D * 2, "device"), up(dev, qkv[:, :D].copy())
+        b16 = dev.buffer(rows * D * 2, "device")
+        try:
+            TK["split_qkv"]([bq, bb] + outs, rows * D, D, T, H, hd)
+            for o, w in zip(outs, RT.split_qkv(qkv, bias, B, T, H, hd, dtype)):
+                assert np.array_equal(stored(o, dtype, (B * H, T, hd)).view(np.uint16), w.view(np.uint16))
+            TK["merge_qkv_grad"](hb + [bm], rows * D, D, T, H, hd)
+            assert np.array_equal(stored(bm, dtype, (rows, 3 * D)).view(np.uint16),
+                                  RT.merge_qkv_grad(*heads32, B, T, H, hd, dtype).view(np.uint16))
+            TK["merge_heads"]([hb[0], b16], rows * D, D, T, H, hd)
+            assert np.array_equal(stored(b16, dtype, (rows, D)).view(np.uint16),
+                                  RT.merge_heads(heads32[0], B, T, H, hd, dtype).view(np.uint16))
+            TK["split_heads"]([bx, b16], rows * D, D, T, H, hd)
+            assert np.array_equal(stored(b16, dtype, (B * H, T, hd)).view(np.uint16),
+                                  RT.split_heads(qkv[:, :D].copy(), B, T, H, hd, dtype).view(np.uint16))
+        finally:
+            for t in [bq, bb, bm, bx, b16] + outs + hb:
+                t.destroy()
+
+
+def test_embeddings_residual_and_column_sums(dev, tk):
+    dtype, TK = tk
+    rng = np.random.default_rng(3)
+    B, T, D, V = 3, 17, 24, 29
+    rows = B * T
+    tok = rng.standard_normal((V, D)).astype(np.float32)
+    pos = rng.standard_normal((T, D)).astype(np.float32)
+    ids = rng.integers(0, V, rows).astype(np.uint32)
+    seg = np.zeros(rows, np.uint32)
+    seg[5:T] = 5
+    seg[T + 9:2 * T] = 9
+    dx = rng.integers(-8, 8, (rows, D)).astype(np.float32)          # integers: the scatter-add is exact in any order
+    btok, bpos, bids, bseg, bdx = up(dev, tok), up(dev, pos), up(dev, ids), up(dev, seg), up(dev, dx)
+    bx, bdt, bdp = dev.buffer(rows * D * 4, "device"), dev.buffer(V * D * 4, "device"), dev.buffer(T * D * 4, "device")
+    try:
+        for sg, bsg in ((None, None), (seg, bseg)):
+            if sg is None:
+                TK["embed"]([btok, bpos, bids, bx], rows * D, D, T)
+            else:
+                TK["embed_doc"]([btok, bpos, bids, bsg, bx], rows * D, D, T)
+            assert np.array_equal(bx.download(np.float32, (rows, D)), RT.embed(tok, pos, ids, T, sg))
+            TK["col_sum_zero"]([bdt], V * D)
+            TK["col_sum_zero"]([bdp], T * D)
+            if sg is None:
+                TK["embed_bwd"]([bdx, bids, bdt, bdp], rows * D, D, T)
+            else:
+                TK["embed_doc_bwd"]([bdx, bids, bsg, bdt, bdp], rows * D, D, T)
+            wt, wp = RT.embed_bwd(dx, ids, T, V, sg)
+            assert np.array_equal(bdt.download(np.float32, (V, D)), wt)
+            assert np.array_equal(bdp.download(np.float32, (T, D)), wp)
+        # residual, add, add_bias, to16
+        acc, res = rng.standard_normal((rows, D)).astype(np.float32), rng.standard_normal((rows, D)).astype(np.float32)
+        bias = rng.standard_normal(D).astype(np.float32)
+        ba, br, bb, bo = up(dev, acc), up(dev, res), up(dev, bias), dev.buffer(rows * D * 4, "device")
+        b16 = dev.buffer(rows * D * 2, "device")
+        bsum = dev.buffer(D * 4, "device")
+        try:
+            TK["residual"]([ba, bb, br, bo], rows * D, D)
+            assert np.array_equal(bo.download(np.float32, (rows, D)), (res + acc) + bias[None, :]) or \
+                np.allclose(bo.download(np.float32, (rows, D)), RT.residual(acc, bias, res), atol=1e-6)
+            TK["add"]([ba, br, bo], rows * D)
+            assert np.array_equal(bo.download(np.float32, (rows, D)), acc + res)
+            TK["add_bias"]([bo, bb], rows * D, D)
+            assert np.array_equal(bo.download(np.float32, (rows, D)), (acc + res) + bias[None, :])
+            TK["to16"]([ba, b16], rows * D)
+            got16 = stored(b16, dtype, (rows, D))
+            assert np.array_equal(got16.view(np.uint16), O.round_to(acc, dtype).view(np.uint16))
+            # column sums of the 16-bit matrix, few rows (one chunk) and many (atomics between chunks)
+            TK["col_sum_zero"]([bsum], D)
+            TK["col_sum_chunk16"]([b16, bsum], 32 * D, D, rows, 32)
+            assert np.allclose(bsum.download(np.float32, (D,)), RT.col_sum16(got16, dtype), rtol=1e-6, atol=1e-5)
+            TK["col_sum_chunk16"]([b16, bsum], 32 * D, D, rows, 32)       # adds: twice the sums now
+            assert np.allclose(bsum.download(np.float32, (D,)), 2 * RT.col_sum16(got16, dtype), rtol=1e-6, atol=1e-5)
+        finally:
+            for t in (ba, br, bb, bo, b16, bsum):
+                t.destroy()
+        big = O.round_to(rng.integers(-4, 4, (1500, 70)).astype(np.float32), dtype)
+        bbig, bs2 = up(dev, big.view(np.uint16)), dev.buffer(70 * 4, "device")
+        try:
+            TK["col_sum_zero"]([bs2], 70)
+            TK["col_sum_chunk16"]([bbig, bs2], 32 * 70, 70, 1500, 32)
+            assert np.array_equal(bs2.download(np.float32, (70,)), RT.col_sum16(big, dtype))
+        finally:
+            bbig.destroy()
+            bs2.destroy()
+    finally:
+        for t in (btok, bpos, bids, bseg, bdx, bx, bdt, bdp):
+            t.destroy()
+
+
+def test_wide_softmax_cross_entropy(dev, tk):
+    dtype, TK = tk
+    rng = np.random.default_rng(4)
+    for rows, stride, ncls in ((6, 16, 10), (5, 1040, 1000), (3, 50304, 50257)):
+        logits = (rng.standard_normal((rows, stride)) * 2).astype(np.float32)
+        logits[:, ncls:] = 1e4                                      # padding must be masked
+        labels = rng.integers(0, ncls, rows).astype(np.uint32)
+        w = rng.uniform(0.5, 2.0, rows).astype(np.float32)
+        w[1] = 0
+        bl, by, bw = up(dev, logits), up(dev, labels), up(dev, w)
+        b16, b32, bloss = dev.buffer(rows * stride * 2, "device"), dev.buffer(rows * stride * 4, "device"), dev.buffer(rows * 4, "device")
+        try:
+            TK["softmax_ce"]([bl, by, b16, b32, bloss], rows, stride, ncls)
+            loss, dl16, dl32 = RT.softmax_ce_rows(logits, labels, ncls, None, dtype)
+            assert np.allclose(bloss.download(np.float32, (rows,)), loss, rtol=1e-5, atol=1e-5)
+            g32 = b32.download(np.float32, (rows, stride))
+            assert np.abs(g32 - dl32).max() <= 1e-6 and not g32[:, ncls:].any()
+            assert close16(stored(b16, dtype, (rows, stride)), dl16, dtype, slack=1e-7)
+            TK["softmax_ce_w"]([bl, by, bw, b16, bloss], rows, stride, ncls)
+            loss, dl16, dl32 = RT.softmax_ce_rows(logits, labels, ncls, w, dtype)
+            assert np.allclose(bloss.download(np.float32, (rows,)), loss, rtol=1e-5, atol=1e-5)
+            got = stored(b16, dtype, (rows, stride))
+            assert close16(got, dl16, dtype, slack=1e-6) and not O.widen(got, dtype)[1].any()
+        finally:
+            for t in (bl, by, bw, b16, b32, bloss):
+                t.destroy()

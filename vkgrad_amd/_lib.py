@@ -60,6 +60,7 @@ class DeviceInfo(C.Structure):
 
 # name -> (restype, argtypes); every symbol include/mi_gemm.h declares.
 _P = C.c_void_p
+_I = C.c_int64
 SIGNATURES = {
     "mg_init": (C.c_int, [C.c_int, C.POINTER(_P)]),
     "mg_destroy": (C.c_int, [_P]),
@@ -96,6 +97,21 @@ SIGNATURES = {
     "mg_ew_cast16": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int]),
     "mg_ew_grad_add": (C.c_int, [_P, _P, _P, C.c_int64]),
     "mg_ew_fill_uniform16": (C.c_int, [_P, _P, C.c_int64, C.c_uint32, C.c_int]),
+    "mg_tk_layernorm": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _I, _I, C.c_int]),
+    "mg_tk_layernorm_bwd": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, C.c_int]),
+    "mg_tk_attn_softmax": (C.c_int, [_P, _P, _P, _P, _I, _I, _I, C.c_float, C.c_int]),
+    "mg_tk_attn_softmax_bwd": (C.c_int, [_P, _P, _P, _P, _I, _I, C.c_float, C.c_int]),
+    "mg_tk_split_qkv": (C.c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, C.c_int]),
+    "mg_tk_merge_qkv_grad": (C.c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, C.c_int]),
+    "mg_tk_merge_heads": (C.c_int, [_P, _P, _P, _I, _I, _I, _I, _I, C.c_int]),
+    "mg_tk_split_heads": (C.c_int, [_P, _P, _P, _I, _I, _I, _I, _I, C.c_int]),
+    "mg_tk_embed": (C.c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I]),
+    "mg_tk_embed_bwd": (C.c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I]),
+    "mg_tk_residual": (C.c_int, [_P, _P, _P, _P, _P, _I, _I]),
+    "mg_tk_add": (C.c_int, [_P, _P, _P, _P, _I]),
+    "mg_tk_add_bias": (C.c_int, [_P, _P, _P, _I, _I]),
+    "mg_tk_col_sum16": (C.c_int, [_P, _P, _P, _I, _I, C.c_int, C.c_int]),
+    "mg_tk_softmax_ce": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, C.c_int]),
 }
 
 _lib = None
