@@ -235,3 +235,128 @@ def test_wide_softmax_cross_entropy(dev, tk):
         finally:
             for t in (bl, by, bw, b16, b32, bloss):
                 t.destroy()
+
+
+# --------------------------------------------------------------------------
+# whole model
+# --------------------------------------------------------------------------
+
+def _oracle_name(param_name):
+    """'b0.attn.qkv.W' -> 'b0.qkv.W' (the oracle's flat names)."""
+    return param_name.replace(".attn.", ".")
+
+
+def _shared(ctx, arr):
+    buf = ctx.buf(arr.nbytes, "shared")
+    buf.array(arr.dtype, arr.shape)[:] = arr
+    buf.flush()
+    return buf
+
+
+def _relerr(got, want):
+    return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-8))
+
+
+def _check_model(dev, B, T, D, H, L, vocab, tie, fuse, dtype, packed=False, staged=False):
+    from vkgrad_amd.transformer import GPT, TCtx
+    rows = B * T
+    ctx = TCtx(dev, dtype=dtype, fuse=fuse)
+    try:
+        model = GPT(ctx, B, T, D, H, L, vocab, tie=tie)
+        rng = np.random.default_rng(0)
+        ids = rng.integers(0, vocab, rows).astype(np.uint32)
+        tgt = rng.integers(0, vocab, rows).astype(np.uint32)
+        # non-zero biases (head.b large), or a forward pass that drops one goes unnoticed
+        # (test_transformer.py:243-254)
+        rb = np.random.default_rng(1)
+        for p in model.params():
+            if p.name.endswith(".b"):
+                p.set((rb.standard_normal(p.shape) * (1.0 if p.name == "head.b" else 0.1)).astype(np.float32))
+        seg = weights = segb = wb = None
+        if packed:
+            seg = np.zeros(rows, np.uint32)
+            for b, starts in enumerate(((0, 23, 40, 57), (0, 5, 33))):
+                for s, e in zip(starts, starts[1:] + (T,)):
+                    seg[b * T + s:b * T + e] = s
+            weights = rng.uniform(0.5, 2.0, rows).astype(np.float32)
+            weights[rng.random(rows) < 0.3] = 0.0
+            segb, wb = _shared(ctx, seg), _shared(ctx, weights)
+        idb, tgb = _shared(ctx, ids), _shared(ctx, tgt)
+        P = {_oracle_name(p.name): p.numpy() for p in model.params()}
+        graphs = {}
+
+        def stage(s):
+            if s not in graphs:
+                graphs[s] = dev.graph(f"stage{s}")
+            return graphs[s]
+
+        model.record(idb, tgb, stage if staged else stage(0), seg=segb, weights=wb)
+        if staged:
+            assert sorted(graphs) == list(range(model.n_stages()))
+        for s in sorted(graphs):
+            graphs[s].finish()
+            graphs[s].submit()
+        dev.sync()
+        model.loss.invalidate()
+        per_row = model.loss.array(np.float32, (rows,)).copy()
+        ref = RT.GPTModel(P, B, T, D, H, L, vocab, model.pad_vocab, tie=tie)
+        want_loss, G, ce = ref.loss_and_grads(ids, tgt, seg=seg, weights=weights)
+        if packed:
+            assert not per_row[weights == 0].any(), "rows of weight 0 must report loss 0"
+            loss = float((per_row * weights).sum())
+        else:
+            loss = model.read_loss()
+        tol_loss, tol_grad = (5e-3, 3e-2) if dtype == "f16" else (2e-2, 1e-1)
+        assert abs(loss - want_loss) / abs(want_loss) < tol_loss, (loss, want_loss)
+        worst = {}
+        for p in model.params():
+            e = _relerr(p.grad_numpy(), G[_oracle_name(p.name)].reshape(p.shape))
+            if e >= tol_grad:
+                worst[p.name] = e
+        assert not worst, f"gradients off: {worst}"
+        for g in graphs.values():
+            g.destroy()
+        return model, G, ref
+    finally:
+        ctx.destroy()
+
+
+@pytest.mark.parametrize("fuse", [False, True])
+@pytest.mark.parametrize("tie", [False, True])
+def test_gpt_loss_and_gradients(dev, tie, fuse):
+    _check_model(dev, 2, 16, 32, 2, 2, 16, tie, fuse, "f16")
+
+
+def test_gpt_bf16_ragged_dimensions(dev):
+    """bf16 operands, and sizes that are multiples of nothing (T = 19, hd = 9 -> D = 27,
+    vocabulary 21): no padding is needed anywhere but the logits' pitch."""
+    _check_model(dev, 2, 19, 27, 3, 1, 21, True, True, "bf16")
+
+
+@pytest.mark.parametrize("fuse", [False, True])
+def test_gpt_packed_samples_weights_and_stages(dev, fuse):
+    """Samples packed into rows (seg), per-row loss weights and one graph per stage, at once
+    (test_transformer.py:279-339): T is past one wavefront's 64 lanes and samples start
+    mid-wavefront.  The same device gradients are also compared with a model that ignores
+    seg, to show that the check can fail."""
+    from vkgrad_amd.transformer import GPT, TCtx
+    B, T, D, H, L, vocab = 2, 80, 32, 2, 2, 16
+    _check_model(dev, B, T, D, H, L, vocab, True, fuse, "f16", packed=True, staged=True)
+    # negative control on the oracle side: without seg the position gradient differs grossly
+    rng = np.random.default_rng(0)
+    rows = B * T
+    ids = rng.integers(0, vocab, rows).astype(np.uint32)
+    tgt = rng.integers(0, vocab, rows).astype(np.uint32)
+    seg = np.zeros(rows, np.uint32)
+    seg[23:T] = 23
+    Pr = {"tok": rng.standard_normal((64, D)) * 0.02, "pos": rng.standard_normal((T, D)) * 0.02,
+          "lnf.g": np.ones(D), "lnf.b": np.zeros(D)}
+    for l in range(L):
+        for n, shp in (("ln1.g", (D,)), ("ln1.b", (D,)), ("qkv.W", (D, 3 * D)), ("qkv.b", (3 * D,)),
+                       ("proj.W", (D, D)), ("proj.b", (D,)), ("ln2.g", (D,)), ("ln2.b", (D,)),
+                       ("fc1.W", (D, 4 * D)), ("fc1.b", (4 * D,)), ("fc2.W", (4 * D, D)), ("fc2.b", (D,))):
+            Pr[f"b{l}.{n}"] = np.ones(shp) if n.endswith(".g") else rng.standard_normal(shp) * 0.2
+    m = RT.GPTModel(Pr, B, T, D, H, L, vocab, 64, tie=True)
+    _, Ga, _ = m.loss_and_grads(ids, tgt, seg=seg)
+    _, Gb, _ = m.loss_and_grads(ids, tgt)
+    assert _relerr(Ga["pos"], Gb["pos"]) > 0.3
