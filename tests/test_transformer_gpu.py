@@ -75,7 +75,7 @@ def test_attention_softmax_forward_backward(dev, tk):
     dtype, TK = tk
     W = dev.row_subgroup_size
     rng = np.random.default_rng(1)
-    for B, H, T in ((1, 2, 16), (2, 3, 70), (1, 1, 200)):
+    for B, H, T in ((1, 2, 16), (2, 3, 70), (1, 1, 200), (1, 1, 512), (1, 2, 1024), (1, 1, 1100)):
         rows = B * H * T
         s = (rng.standard_normal((rows, T)) * 3).astype(np.float32)
         s[:, T // 2:] += np.where(rng.random((rows, T - T // 2)) < 0.1, 1e4, 0).astype(np.float32)   # masked junk must not leak

@@ -111,6 +111,100 @@ k_attn_softmax(const float *s, const uint32_t *seg, uint16_t *p16, int64_t rows,
     }
 }
 
+// The same two kernels for T % 4 == 0 and T <= 256 * NV: a lane holds NV groups of four
+// consecutive scores (group i covers keys 256 i + 4 lane ...), loaded once with 16-byte loads
+// - groups wholly beyond the query are never fetched - and the probabilities leave as 8-byte
+// stores.  One pass over HBM instead of three L2-assisted ones.
+template <int NV>
+__global__ void __launch_bounds__(64 * ROWS_PER_WG)
+k_attn_softmax_reg(const float *s, const uint32_t *seg, uint16_t *p16, int64_t rows, int T, int H, float scale, int dtype) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * ROWS_PER_WG + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int q = (int)(row % T);
+    const int first = seg ? (int)seg[(row / T / H) * T + q] : 0;
+    const float4 *sr = reinterpret_cast<const float4 *>(s + row * T);
+    float v[NV][4];
+    float mx = -1e30f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int j0 = i * 256 + lane * 4;
+        float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (j0 <= q && j0 + 3 >= first && j0 < T) t = sr[j0 >> 2];
+        v[i][0] = t.x * scale; v[i][1] = t.y * scale; v[i][2] = t.z * scale; v[i][3] = t.w * scale;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int j = j0 + e;
+            if (j >= first && j <= q) mx = fmaxf(mx, v[i][e]);
+        }
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int j = i * 256 + lane * 4 + e;
+            const float ex = (j >= first && j <= q) ? __expf(v[i][e] - mx) : 0.f;
+            v[i][e] = ex;
+            sum += ex;
+        }
+    const float inv = 1.0f / wave_sum(sum);
+    uint2 *pr = reinterpret_cast<uint2 *>(p16 + row * T);
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int j0 = i * 256 + lane * 4;
+        if (j0 < T) {
+            const uint32_t a = narrow16(v[i][0] * inv, dtype), b = narrow16(v[i][1] * inv, dtype);
+            const uint32_t c = narrow16(v[i][2] * inv, dtype), d = narrow16(v[i][3] * inv, dtype);
+            pr[j0 >> 2] = make_uint2(a | (b << 16), c | (d << 16));
+        }
+    }
+}
+
+template <int NV>
+__global__ void __launch_bounds__(64 * ROWS_PER_WG)
+k_attn_softmax_bwd_reg(const float *dp, const uint16_t *p16, uint16_t *ds16, int64_t rows, int T, float scale, int dtype) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * ROWS_PER_WG + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int q = (int)(row % T);
+    const float4 *dr = reinterpret_cast<const float4 *>(dp + row * T);
+    const uint2 *pr = reinterpret_cast<const uint2 *>(p16 + row * T);
+    float g[NV][4], pv[NV][4];
+    float dot = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int j0 = i * 256 + lane * 4;
+        float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+        uint2 u = make_uint2(0u, 0u);
+        if (j0 <= q && j0 < T) {
+            t = dr[j0 >> 2];
+            u = pr[j0 >> 2];
+        }
+        g[i][0] = t.x; g[i][1] = t.y; g[i][2] = t.z; g[i][3] = t.w;
+        pv[i][0] = widen16((uint16_t)(u.x & 0xffffu), dtype); pv[i][1] = widen16((uint16_t)(u.x >> 16), dtype);
+        pv[i][2] = widen16((uint16_t)(u.y & 0xffffu), dtype); pv[i][3] = widen16((uint16_t)(u.y >> 16), dtype);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            if (j0 + e > q) pv[i][e] = 0.f;       // beyond the query: P is zero there whatever the buffer holds
+            dot += g[i][e] * pv[i][e];
+        }
+    }
+    dot = wave_sum(dot);
+    uint2 *dr16 = reinterpret_cast<uint2 *>(ds16 + row * T);
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int j0 = i * 256 + lane * 4;
+        if (j0 < T) {
+            uint32_t o[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = narrow16(j0 + e <= q ? pv[i][e] * (g[i][e] - dot) * scale : 0.f, dtype);
+            dr16[j0 >> 2] = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+        }
+    }
+}
+
 // dS = P * (dP - sum_j dP_j P_j) * scale over the unmasked keys (tkernels.py:167-187); masked keys
 // hold P = 0, so only j <= q is read.
 __global__ void __launch_bounds__(64 * ROWS_PER_WG)
@@ -247,47 +341,83 @@ __global__ void k_zero_f32(float *dst, int64_t n) {
     if (i < n) dst[i] = 0.f;
 }
 
-// ---- Softmax cross-entropy over a wide row (the LM head: 50257 classes).  Same arithmetic as
-// the one-thread-per-row kernel of the MLP (kernels.py:766-791), with the row spread over a
-// 256-thread workgroup: max, sum of exponentials and the gradient sweep are each one coalesced
-// pass; weight[row] (or 1 / nrows) scales the gradient (softmax_ce_w, transformer.py:331-337).
+// ---- Softmax cross-entropy over a wide row (the LM head: 50257 classes).  Same result as the
+// one-thread-per-row kernel of the MLP (kernels.py:766-791) with the row spread over a
+// 256-thread workgroup.  Pass 1 keeps a running maximum and a sum of exponentials relative to
+// it per thread (one read of the row instead of two), the workgroup merges them; pass 2
+// re-reads the row (L2 / last-level cache) and writes the gradient.  weight[row] (or
+// 1 / nrows) scales the gradient (softmax_ce_w, kernels.py:793-823).  Rows whose pitch and
+// base are 16-byte aligned move as float4 / four 16-bit values.
+struct MaxSum {
+    float m, s;
+};
+__device__ __forceinline__ void ms_push(MaxSum &a, float x) {
+    if (x > a.m) {
+        a.s = a.s * __expf(a.m - x) + 1.0f;
+        a.m = x;
+    } else {
+        a.s += __expf(x - a.m);
+    }
+}
+__device__ __forceinline__ MaxSum ms_merge(MaxSum a, MaxSum b) {
+    const float m = fmaxf(a.m, b.m);
+    return MaxSum{m, a.s * __expf(a.m - m) + b.s * __expf(b.m - m)};
+}
 __global__ void __launch_bounds__(256)
 k_softmax_ce_wide(const float *logits, const uint32_t *labels, const float *weights, uint16_t *dl16, float *dl32,
-                  float *loss, int64_t nrows, int64_t stride, int64_t ncls, int dtype) {
-    __shared__ float red[4];
+                  float *loss, int64_t nrows, int64_t stride, int64_t ncls, int dtype, int vec) {
+    __shared__ float red_m[4], red_s[4];
     const int64_t row = blockIdx.x;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const float *lr = logits + row * stride;
+    uint16_t *g16 = dl16 ? dl16 + row * stride : nullptr;
+    float *g32 = dl32 ? dl32 + row * stride : nullptr;
     if (weights && weights[row] == 0.f) {   // masked row: no softmax, zeros (uniform over the workgroup)
         for (int64_t c = tid; c < stride; c += 256) {
-            if (dl16) dl16[row * stride + c] = 0;
-            if (dl32) dl32[row * stride + c] = 0.f;
+            if (g16) g16[c] = 0;
+            if (g32) g32[c] = 0.f;
         }
         if (tid == 0) loss[row] = 0.f;
         return;
     }
-    float mx = -1e30f;
-    for (int64_t c = tid; c < ncls; c += 256) mx = fmaxf(mx, lr[c]);
-    mx = wave_max(mx);
-    if (lane == 0) red[wave] = mx;
+    MaxSum acc{-1e30f, 0.f};
+    const int64_t n4 = vec ? ncls / 4 : 0;
+    for (int64_t c = tid; c < n4; c += 256) {
+        const float4 t = reinterpret_cast<const float4 *>(lr)[c];
+        ms_push(acc, t.x); ms_push(acc, t.y); ms_push(acc, t.z); ms_push(acc, t.w);
+    }
+    for (int64_t c = n4 * 4 + tid; c < ncls; c += 256) ms_push(acc, lr[c]);
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        MaxSum o{__shfl_xor(acc.m, m, 64), __shfl_xor(acc.s, m, 64)};
+        acc = ms_merge(acc, o);
+    }
+    if (lane == 0) {
+        red_m[wave] = acc.m;
+        red_s[wave] = acc.s;
+    }
     __syncthreads();
-    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    __syncthreads();
-    float s = 0.f;
-    for (int64_t c = tid; c < ncls; c += 256) s += __expf(lr[c] - mx);
-    s = wave_sum(s);
-    if (lane == 0) red[wave] = s;
-    __syncthreads();
-    s = (red[0] + red[1]) + (red[2] + red[3]);
-    const float logZ = mx + __logf(s);
-    const uint32_t y = labels[row];
+    MaxSum all = ms_merge(ms_merge(MaxSum{red_m[0], red_s[0]}, MaxSum{red_m[1], red_s[1]}),
+                          ms_merge(MaxSum{red_m[2], red_s[2]}, MaxSum{red_m[3], red_s[3]}));
+    const float logZ = all.m + __logf(all.s);
+    const int64_t y = labels[row];
     const float w = weights ? weights[row] : 1.0f / (float)nrows;
     if (tid == 0) loss[row] = logZ - lr[y];
-    for (int64_t c = tid; c < stride; c += 256) {
-        float gv = 0.f;
-        if (c < ncls) gv = (__expf(lr[c] - logZ) - (c == (int64_t)y ? 1.f : 0.f)) * w;
-        if (dl16) dl16[row * stride + c] = narrow16(gv, dtype);
-        if (dl32) dl32[row * stride + c] = gv;
+    auto grad = [&](int64_t c, float x) { return c < ncls ? (__expf(x - logZ) - (c == y ? 1.f : 0.f)) * w : 0.f; };
+    const int64_t s4 = vec ? stride / 4 : 0;
+    for (int64_t c = tid; c < s4; c += 256) {
+        const float4 t = reinterpret_cast<const float4 *>(lr)[c];
+        const float a = grad(4 * c, t.x), b = grad(4 * c + 1, t.y), cc = grad(4 * c + 2, t.z), d = grad(4 * c + 3, t.w);
+        if (g16)
+            reinterpret_cast<uint2 *>(g16)[c] =
+                make_uint2((uint32_t)narrow16(a, dtype) | ((uint32_t)narrow16(b, dtype) << 16),
+                           (uint32_t)narrow16(cc, dtype) | ((uint32_t)narrow16(d, dtype) << 16));
+        if (g32) reinterpret_cast<float4 *>(g32)[c] = make_float4(a, b, cc, d);
+    }
+    for (int64_t c = s4 * 4 + tid; c < stride; c += 256) {
+        const float gv = grad(c, c < ncls ? lr[c] : 0.f);
+        if (g16) g16[c] = narrow16(gv, dtype);
+        if (g32) g32[c] = gv;
     }
 }
 
@@ -324,8 +454,13 @@ int mg_tk_attn_softmax(mg_ctx *ctx, const float *s, const uint32_t *seg, void *p
                        float scale, int dtype) {
     EW_PRECHECK("mg_tk_attn_softmax", s && p16 && count_ok(rows) && T > 0 && T <= 0x7fffffff && rows % T == 0 &&
                                           H > 0 && (!seg || (rows / T) % H == 0) && dtype_ok(dtype));
-    hipLaunchKernelGGL(k_attn_softmax, dim3(row_blocks(rows)), dim3(64 * ROWS_PER_WG), 0, ctx_stream(ctx), s, seg,
-                       (uint16_t *)p16, rows, (int)T, (int)H, scale, dtype);
+    const bool vec = T % 4 == 0 && T <= 1024 && (((uintptr_t)s & 15) == 0) && (((uintptr_t)p16 & 7) == 0);
+    const dim3 grid(row_blocks(rows)), block(64 * ROWS_PER_WG);
+    uint16_t *p = (uint16_t *)p16;
+    if (vec && T <= 256) hipLaunchKernelGGL(k_attn_softmax_reg<1>, grid, block, 0, ctx_stream(ctx), s, seg, p, rows, (int)T, (int)H, scale, dtype);
+    else if (vec && T <= 512) hipLaunchKernelGGL(k_attn_softmax_reg<2>, grid, block, 0, ctx_stream(ctx), s, seg, p, rows, (int)T, (int)H, scale, dtype);
+    else if (vec) hipLaunchKernelGGL(k_attn_softmax_reg<4>, grid, block, 0, ctx_stream(ctx), s, seg, p, rows, (int)T, (int)H, scale, dtype);
+    else hipLaunchKernelGGL(k_attn_softmax, grid, block, 0, ctx_stream(ctx), s, seg, p, rows, (int)T, (int)H, scale, dtype);
     EW_POSTCHECK("mg_tk_attn_softmax");
 }
 
@@ -333,8 +468,15 @@ int mg_tk_attn_softmax_bwd(mg_ctx *ctx, const float *dp, const void *p16, void *
                            float scale, int dtype) {
     EW_PRECHECK("mg_tk_attn_softmax_bwd", dp && p16 && ds16 && count_ok(rows) && T > 0 && T <= 0x7fffffff &&
                                               rows % T == 0 && dtype_ok(dtype));
-    hipLaunchKernelGGL(k_attn_softmax_bwd, dim3(row_blocks(rows)), dim3(64 * ROWS_PER_WG), 0, ctx_stream(ctx), dp,
-                       (const uint16_t *)p16, (uint16_t *)ds16, rows, (int)T, scale, dtype);
+    const bool vec = T % 4 == 0 && T <= 1024 && (((uintptr_t)dp & 15) == 0) &&
+                     ((((uintptr_t)p16 | (uintptr_t)ds16) & 7) == 0);
+    const dim3 grid(row_blocks(rows)), block(64 * ROWS_PER_WG);
+    const uint16_t *p = (const uint16_t *)p16;
+    uint16_t *d = (uint16_t *)ds16;
+    if (vec && T <= 256) hipLaunchKernelGGL(k_attn_softmax_bwd_reg<1>, grid, block, 0, ctx_stream(ctx), dp, p, d, rows, (int)T, scale, dtype);
+    else if (vec && T <= 512) hipLaunchKernelGGL(k_attn_softmax_bwd_reg<2>, grid, block, 0, ctx_stream(ctx), dp, p, d, rows, (int)T, scale, dtype);
+    else if (vec) hipLaunchKernelGGL(k_attn_softmax_bwd_reg<4>, grid, block, 0, ctx_stream(ctx), dp, p, d, rows, (int)T, scale, dtype);
+    else hipLaunchKernelGGL(k_attn_softmax_bwd, grid, block, 0, ctx_stream(ctx), dp, p, d, rows, (int)T, scale, dtype);
     EW_POSTCHECK("mg_tk_attn_softmax_bwd");
 }
 
@@ -424,8 +566,9 @@ int mg_tk_softmax_ce(mg_ctx *ctx, const float *logits, const uint32_t *labels, c
                      float *dl32, float *loss, int64_t nrows, int64_t stride, int64_t ncls, int dtype) {
     EW_PRECHECK("mg_tk_softmax_ce", logits && labels && loss && nrows > 0 && nrows <= 0x7fffffff && ncls > 0 &&
                                         stride >= ncls && dtype_ok(dtype));
+    const int vec = stride % 4 == 0 && (((uintptr_t)logits | (uintptr_t)dl32) & 15) == 0 && ((uintptr_t)dl16 & 7) == 0;
     hipLaunchKernelGGL(k_softmax_ce_wide, dim3((unsigned)nrows), dim3(256), 0, ctx_stream(ctx), logits, labels, weights,
-                       (uint16_t *)dl16, dl32, loss, nrows, stride, ncls, dtype);
+                       (uint16_t *)dl16, dl32, loss, nrows, stride, ncls, dtype, vec);
     EW_POSTCHECK("mg_tk_softmax_ce");
 }
 

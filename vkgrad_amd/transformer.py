@@ -297,7 +297,7 @@ class GPT:
             self.logits, self.dh32 = _f32(ctx, R, V), _f32(ctx, R, D)
         else:
             self.head = Dense(ctx, R, D, V, "head", scale=0.02)
-        self.dlog16, self.dlog32 = _h16(ctx, R, V), _f32(ctx, R, V)
+        self.dlog16, self.dlog32 = _h16(ctx, R, V), None   # nothing downstream reads an f32 copy of dlogits
         self.loss = ctx.buf(R * 4, "cached")
         self.h16 = None
 
