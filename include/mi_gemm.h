@@ -265,6 +265,9 @@ int mg_ew_cast16(mg_ctx *ctx, const float *src, void *dst, int64_t n, int dtype)
 int mg_ew_fill_uniform16(mg_ctx *ctx, void *dst, int64_t n, uint32_t seed, int dtype);
 /* grad_add (dataparallel.py:54-58): dst[i] += src[i] */
 int mg_ew_grad_add(mg_ctx *ctx, float *dst, const float *src, int64_t n);
+/* grad_pull (dataparallel.py:69-73): dst[i] = src[i] * scale - the summed gradient of several
+ * micro-batches read back out of the accumulator as a mean */
+int mg_ew_scale_copy(mg_ctx *ctx, float *dst, const float *src, int64_t n, float scale);
 
 /* ---- Row kernels of the decoder block (tkernels.py), all in f32 with 16-bit outputs where the
  * next GEMM reads them.  `dtype` is the 16-bit type.  Head-side tensors are (B*H, T, hd),

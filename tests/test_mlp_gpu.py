@@ -108,3 +108,75 @@ def test_graph_replay_sees_new_inputs(dev):
         assert abs(l0 - want0) < 2e-5 and abs(l1 - want1) < 2e-5 and abs(l0 - l1) > 1e-4
     finally:
         ctx.destroy()
+
+
+@pytest.mark.parametrize("dirty", [False, True])
+def test_gradient_accumulation_equals_one_large_batch(dev, dirty):
+    """GradAccum over N micro-batches of B rows against the device's own batch of N*B rows
+    (test_accum.py:1-9, 139-168: relative error below 2e-2, also when the accumulator holds
+    stale values before it is zeroed), and one optimiser step from each lands on the same
+    weights."""
+    from vkgrad_amd.autograd import MLP, AdamW, Ctx
+    from vkgrad_amd.dataparallel import GradAccum
+    B, N, in_f, hidden, n_cls = 16, 4, 64, 32, 8
+    rng = np.random.default_rng(3)
+    data = rng.standard_normal((B * N, in_f)).astype(np.float16)
+    labels = rng.integers(0, n_cls, B * N).astype(np.uint32)
+
+    def build(batch):
+        ctx = Ctx(dev)
+        model = MLP(ctx, batch, [in_f, hidden], n_cls, pad_classes=16)
+        r = np.random.default_rng(7)                      # identical weights however the batch is split
+        for p in model.params():
+            p.set(r.standard_normal(p.shape).astype(np.float32) * 0.05)
+        xb, yb = ctx.buf(batch * in_f * 2, "shared"), ctx.buf(batch * 4, "shared")
+        return ctx, model, xb, yb
+
+    def feed(xb, yb, rows, lo):
+        xb.array(np.float16, (rows, in_f))[:] = data[lo:lo + rows]
+        yb.array(np.uint32, (rows,))[:] = labels[lo:lo + rows]
+        xb.flush()
+        yb.flush()
+
+    ctx, model, xb, yb = build(B)
+    ctx2, big, xb2, yb2 = build(B * N)
+    try:
+        params = list(model.params())
+        opt = AdamW(ctx, params, lr=1e-3)
+        ga = GradAccum(ctx, params, accum=N)
+        assert ga.total == sum(p.n for p in params) and ga.offsets[1] == params[0].n
+        if dirty:
+            ga.arena.upload(np.random.default_rng(11).standard_normal(ga.total).astype(np.float32))
+            assert np.abs(ga.arena.download(np.float32, (ga.total,))).max() > 0.5
+        g_zero, g_micro, g_apply = dev.graph("zero"), dev.graph("micro"), dev.graph("apply")
+        ga.record_zero(g_zero)
+        model.record(xb, yb, g_micro)
+        ga.record_push(g_micro)
+        ga.record_apply(g_apply, opt)
+        for g in (g_zero, g_micro, g_apply):
+            g.finish()
+        g_zero.submit()
+        for i in range(N):
+            feed(xb, yb, B, i * B)
+            g_micro.submit()
+        summed = ga.arena.download(np.float32, (ga.total,))
+        opt.advance()
+        g_apply.submit()
+
+        params2 = list(big.params())
+        opt2 = AdamW(ctx2, params2, lr=1e-3)
+        feed(xb2, yb2, B * N, 0)
+        big.forward_backward(xb2, yb2)
+        want = np.concatenate([p.grad_numpy().reshape(-1) for p in params2])
+        assert relerr(summed / N, want) < 2e-3            # the reference allows 2e-2 and measures 8.8e-06
+        pulled = np.concatenate([p.grad_numpy().reshape(-1) for p in params])
+        assert np.allclose(pulled, summed / N, rtol=1e-6, atol=0)
+        opt2.step()
+        for p, p2 in zip(params, params2):
+            assert np.abs(p.numpy() - p2.numpy()).max() < 3e-4, p.name   # |update| is about lr = 1e-3
+        for g in (g_zero, g_micro, g_apply):
+            g.destroy()
+        ga.destroy()
+    finally:
+        ctx.destroy()
+        ctx2.destroy()

@@ -96,6 +96,7 @@ SIGNATURES = {
     "mg_ew_copy": (C.c_int, [_P, _P, _P, C.c_int64]),
     "mg_ew_cast16": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int]),
     "mg_ew_grad_add": (C.c_int, [_P, _P, _P, C.c_int64]),
+    "mg_ew_scale_copy": (C.c_int, [_P, _P, _P, C.c_int64, C.c_float]),
     "mg_ew_fill_uniform16": (C.c_int, [_P, _P, C.c_int64, C.c_uint32, C.c_int]),
     "mg_tk_layernorm": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _I, _I, C.c_int]),
     "mg_tk_layernorm_bwd": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, C.c_int]),

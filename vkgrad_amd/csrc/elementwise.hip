@@ -138,6 +138,11 @@ __global__ void k_cast16(const float *src, uint16_t *dst, int64_t n, int dtype) 
     if (i < n) dst[i] = narrow16(src[i], dtype);
 }
 
+__global__ void k_scale_copy(float *dst, const float *src, int64_t n, float scale) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = src[i] * scale;
+}
+
 __global__ void k_grad_add(float *dst, const float *src, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) dst[i] += src[i];
@@ -236,6 +241,12 @@ int mg_ew_fill_uniform16(mg_ctx *ctx, void *dst, int64_t n, uint32_t seed, int d
     hipLaunchKernelGGL(k_fill_uniform16, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), (uint16_t *)dst, n, seed,
                        dtype);
     EW_POSTCHECK("mg_ew_fill_uniform16");
+}
+
+int mg_ew_scale_copy(mg_ctx *ctx, float *dst, const float *src, int64_t n, float scale) {
+    EW_PRECHECK("mg_ew_scale_copy", dst && src && count_ok(n));
+    hipLaunchKernelGGL(k_scale_copy, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), dst, src, n, scale);
+    EW_POSTCHECK("mg_ew_scale_copy");
 }
 
 int mg_ew_grad_add(mg_ctx *ctx, float *dst, const float *src, int64_t n) {
