@@ -54,6 +54,7 @@ enum { MG_F16 = 0, MG_BF16 = 1 };
 enum { MG_DEVICE = 0, MG_SHARED = 1, MG_CACHED = 2, MG_BAR = 3 };
 /* activations for the companion elementwise kernels and the fused GEMM epilogues; the
  * _GRAD forms exist for mg_gemm only (result times the activation's derivative at z) */
+enum { MG_TRI_NONE = 0, MG_TRI_C_LOWER = 1, MG_TRI_A_LOWER = 2, MG_TRI_A_UPPER = 3 };
 enum { MG_ACT_NONE = 0, MG_ACT_GELU = 1, MG_ACT_RELU = 2, MG_ACT_GELU_GRAD = 3, MG_ACT_RELU_GRAD = 4 };
 
 typedef struct {
@@ -100,6 +101,18 @@ typedef struct {
      * is the plain in-place beta == 1).  nbatch == 1; MG_FLAG_SPLITK_ATOMIC is refused. */
     const float *res;      /* NULL: beta == 1 reads C itself */
     int64_t ldr;           /* row pitch of res in elements (>= n) */
+    /* Triangular structure of causal attention (the six per-head GEMMs of transformer.py:144-182
+     * with a causal mask, tkernels.py:105-133): work that only meets masked entries is skipped.
+     *   MG_TRI_C_LOWER  only c[i][j] with j <= i is needed (scores = Q K^T, dP = dOut V^T, whose
+     *                   consumers read keys <= query): tiles wholly above the diagonal are
+     *                   neither computed nor written - C keeps its old contents there;
+     *   MG_TRI_A_LOWER  op(A)[i][k] == 0 for k > i (P V, dS K): a row block's K loop ends at
+     *                   its last row;
+     *   MG_TRI_A_UPPER  op(A)[i][k] == 0 for k < i (P^T dOut, dS^T Q with A stored (k, m)): the K
+     *                   loop starts at the block's first row.
+     * The A forms need m == k and run unsplit; every batch has the same structure. */
+    int32_t tri;           /* MG_TRI_* */
+    int32_t reserved;      /* 0 */
 } mg_gemm_args;
 
 /* The buffers of A and B end at their last element: row padding (ld beyond the stored

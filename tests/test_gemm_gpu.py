@@ -468,6 +468,81 @@ def test_residual_epilogue(dev, layout, dtype):
         buf.destroy()
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_triangular_structure_of_causal_attention(dev, dtype):
+    """tri= skips work that only meets masked entries of causal attention (the per-head
+    GEMMs of transformer.py:144-182).  'c_lower': every C[i, j <= i] equals the full product
+    (integer data: bit exact) whatever the tile, and whole tiles above the diagonal keep
+    their poison; 'a_lower' / 'a_upper': with op(A) triangular the full product comes out,
+    exactly, although part of the K range is never visited.  Batched, ragged, tiles that
+    hand over (persistent, skinny), and the misuse cases."""
+    from vkgrad_amd.kernels import Matmul
+    from vkgrad_amd.vk import VkError
+    rng = np.random.default_rng(5)
+
+    def run(layout, m, n, k, tile, tri, nb, a, b):
+        ta, tb = LAYOUTS[layout]
+        ba, bb, bc = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), dev.buffer(nb * m * n * 4, "device")
+        ba.upload(a); bb.upload(b)
+        bc.upload(np.full((nb, m, n), np.nan, np.float32))
+        mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype=dtype, tile=tile, batched=nb > 1)
+        try:
+            mm(ba, bb, bc, m, n, k, nbatch=nb, strides=(a[0].size, b[0].size, m * n), tri=tri)
+            return bc.download(np.float32, (nb, m, n))
+        finally:
+            mm.destroy()
+            for x in (ba, bb, bc):
+                x.destroy()
+
+    def operands(layout, m, n, k, nb, seed):
+        ta, tb = LAYOUTS[layout]
+        pairs = [O.make_operands(m, n, k, ta, tb, dtype, seed=seed + i, integer=True) for i in range(nb)]
+        return np.stack([p[0] for p in pairs]), np.stack([p[1] for p in pairs])
+
+    def product(layout, a, b):
+        ta, tb = LAYOUTS[layout]
+        return np.stack([O.ref_gemm(a[i], b[i], ta, tb, dtype) for i in range(a.shape[0])])
+
+    # scores-like: C = A . B^T, lower triangle needed
+    for m, n, k, tile, nb in ((200, 200, 64, None, 3), (1024, 1024, 64, None, 2), (512, 512, 64, 11, 1),
+                              (512, 512, 128, 10, 2), (300, 300, 40, 4, 1), (512, 512, 64, 15, 1), (640, 640, 64, 3, 2)):
+        a, b = operands("NT", m, n, k, nb, m + k)
+        got = run("NT", m, n, k, tile, "c_lower", nb, a, b)
+        want = product("NT", a, b)
+        low = np.tril(np.ones((m, n), bool))
+        assert np.array_equal(got[:, low], want[:, low]), (m, n, k, tile)
+        if m >= 512:
+            assert np.isnan(got[:, :256, m - 256:]).all(), "a tile wholly above the diagonal was written"
+    # P V-like (NN) and dS K: op(A) lower triangular
+    for m, n, k, tile, nb in ((256, 64, 256, None, 3), (1000, 72, 1000, None, 1), (512, 64, 512, 11, 2),
+                              (512, 128, 512, 10, 1), (1024, 64, 1024, 14, 2), (300, 64, 300, 4, 1)):
+        a, b = operands("NN", m, n, k, nb, m + n)
+        a_tri = a.copy()
+        a_tri[:, ~np.tril(np.ones((m, k), bool))] = 0
+        got = run("NN", m, n, k, tile, "a_lower", nb, a_tri, b)
+        assert np.array_equal(got, product("NN", a_tri, b)), (m, n, k, tile, "a_lower")
+        # P^T dOut-like (TN): A stored (k, m); op(A)[i, kk] = A[kk, i] is zero for kk < i
+        at, bt = operands("TN", m, n, k, nb, m + n + 1)
+        at_tri = at.copy()
+        at_tri[:, ~np.tril(np.ones((k, m), bool))] = 0          # stored A lower triangular = op(A) upper
+        got = run("TN", m, n, k, tile, "a_upper", nb, at_tri, bt)
+        assert np.array_equal(got, product("TN", at_tri, bt)), (m, n, k, tile, "a_upper")
+    buf = dev.buffer(64 * 64 * 4, "device")
+    mm = Matmul(dev, dtype=dtype)
+    mm2 = Matmul(dev, dtype=dtype, split_k=2)
+    try:
+        with pytest.raises(VkError):
+            mm(buf, buf, buf, 64, 32, 48, tri="a_lower")        # op(A) must be square
+        with pytest.raises(VkError):
+            mm2(buf, buf, buf, 64, 64, 64, tri="c_lower")       # runs unsplit
+        with pytest.raises(VkError):
+            mm(buf, buf, buf, 64, 64, 64, tri="upper")
+    finally:
+        mm.destroy()
+        mm2.destroy()
+        buf.destroy()
+
+
 def test_timing_over_rotating_operand_sets(dev):
     """The rotating timer launches argument set i % nsets on launch i: after seven
     launches over three sets with different integer operands, every set's C holds

@@ -18,6 +18,7 @@ MG_FLAG_SIDE_STREAM = 4
 DTYPES = {"f16": MG_F16, "bf16": MG_BF16}
 KINDS = {"device": MG_DEVICE, "shared": MG_SHARED, "cached": MG_CACHED, "bar": MG_BAR}
 MG_ACT_GELU_GRAD, MG_ACT_RELU_GRAD = 3, 4
+TRI = {None: 0, "c_lower": 1, "a_lower": 2, "a_upper": 3}
 ACTS = {None: MG_ACT_NONE, "none": MG_ACT_NONE, "gelu": MG_ACT_GELU, "relu": MG_ACT_RELU,
         "gelu_grad": MG_ACT_GELU_GRAD, "relu_grad": MG_ACT_RELU_GRAD}
 
@@ -37,6 +38,7 @@ class GemmArgs(C.Structure):
         ("y16", C.c_void_p), ("ldy", C.c_int64),
         ("z", C.c_void_p), ("ldz", C.c_int64), ("colsum", C.c_void_p),
         ("res", C.c_void_p), ("ldr", C.c_int64),
+        ("tri", C.c_int32), ("reserved", C.c_int32),
     ]
 
 

@@ -213,8 +213,10 @@ gemm_dma_kernel(const GemmParams p) {
     const uint16_t *A = p.A + zb * p.sa;
     const uint16_t *B = p.B + zb * p.sb;
     float *C = p.C + zb * p.sc;
-    const int kbeg = blockIdx.y * p.k_per_split;
-    const int kend = min(p.K, kbeg + p.k_per_split);
+    if (p.tri == 1 && n0 > m0 + BM - 1) return;   // tile wholly above the diagonal: nobody reads it
+    int kbeg = blockIdx.y * p.k_per_split;
+    int kend = min(p.K, kbeg + p.k_per_split);
+    tri_k_range<BM, BK>(p.tri, m0, kbeg, kend);
     const int krem = (kend - kbeg) % BK;          // K remainder, multiplied first
     const int kdma = kbeg + krem;                 // the ring covers [kdma, kend)
     const int nkb = (kend - kdma) / BK;

@@ -67,6 +67,7 @@ struct GemmParams {
     float *colsum;        // column sums of the _GRAD result are added here (or NULL)
     const float *R;       // beta = 1 reads this matrix instead of C (or NULL)
     int64_t ldr;
+    int tri;              // MG_TRI_*: causal structure (non-persistent kernels only)
 };
 
 template <int DT>
@@ -336,6 +337,14 @@ __device__ __forceinline__ void interleave_group() {
     interleave_step<0, NMFMA, NDSR, NDSW, NVMEM>();
 }
 
+// K range of a row block when op(A) is triangular (one slice, M == K): rows m0 .. m0 + BM - 1
+// meet non-zero entries of op(A) only for k <= m0 + BM - 1 (lower) or k >= m0 (upper).
+template <int BM, int BK>
+__device__ __forceinline__ void tri_k_range(int tri, int m0, int &kbeg, int &kend) {
+    if (tri == 2) kend = min(kend, m0 + BM);
+    if (tri == 3) kbeg = max(kbeg, (m0 / BK) * BK);
+}
+
 // 16-bit narrowing (round to nearest even) and the activations of the fused output;
 // same formulas as the companion kernels (reference kernels.py:625-629, 709-718).
 template <int DT>
@@ -512,8 +521,10 @@ gemm_kernel(const GemmParams p) {
     const uint16_t *B = p.B + zb * p.sb;
     float *C = p.C + zb * p.sc;
 
-    const int kbeg = blockIdx.y * p.k_per_split;
-    const int kend = min(p.K, kbeg + p.k_per_split);
+    if (p.tri == 1 && n0 > m0 + BM - 1) return;   // tile wholly above the diagonal: nobody reads it
+    int kbeg = blockIdx.y * p.k_per_split;
+    int kend = min(p.K, kbeg + p.k_per_split);
+    tri_k_range<BM, BK>(p.tri, m0, kbeg, kend);
     const int nkb = (kend - kbeg + BK - 1) / BK;
     // K-blocks that the unconditional loader may fetch: the whole block inside
     // K, and the tile inside M and N.

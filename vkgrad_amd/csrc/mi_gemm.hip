@@ -141,6 +141,7 @@ static bool gemv_eligible(const mg_gemm_args &a, int split) {
     if ((a.lda | a.ldb | a.k) & 7) return false;
     if (a.nbatch > 1 && ((a.sa | a.sb) & 7)) return false;
     if (a.res && a.res != a.c) return false;   // its beta = 1 reads C
+    if (a.tri) return false;
     return true;
 }
 
@@ -162,6 +163,7 @@ static bool dma_eligible(const mg_gemm_args &a, const TileDesc &t, int64_t k_per
     if (t.persistent) {
         if (a.k % t.bk != 0 || k_per_split % t.bk != 0) return false;
         if (a.res && a.res != a.c) return false;   // their beta = 1 is an atomic add into C
+        if (a.tri) return false;                   // the unit loop knows nothing of skipped tiles or K ranges
     }
     if (t.persistent == 2 && split > 1) return false;   // stream-K cuts K itself
     // the 256 x 256 stream-K kernel with the bias epilogue does not fit the register file
@@ -293,7 +295,7 @@ static void finish_plan(const mg_gemm_args &a, int tile, int split, Plan &pl) {
     int64_t kblocks = cdiv(a.k, d->bk);
     if (split > kblocks) split = (int)kblocks;
     if (split < 1) split = 1;
-    if (d->persistent == 2 || d->gemv) split = 1;
+    if (d->persistent == 2 || d->gemv || a.tri) split = 1;
     int64_t kb_per = cdiv(kblocks, split);
     split = (int)cdiv(kblocks, kb_per);   // no empty slices
     while (!dma_eligible(a, *d, kb_per * d->bk, split) && d->fallback != tile) {
@@ -406,6 +408,11 @@ static int check_args(const mg_gemm_args *a) {
         if (a->flags & MG_FLAG_SPLITK_ATOMIC)
             return fail(MG_ERR_ARG, "mg_gemm: the fused y16 output cannot be combined with MG_FLAG_SPLITK_ATOMIC");
     }
+    if (a->tri < MG_TRI_NONE || a->tri > MG_TRI_A_UPPER) return fail(MG_ERR_ARG, "mg_gemm: unknown tri %d", a->tri);
+    if (a->tri >= MG_TRI_A_LOWER && a->m != a->k)
+        return fail(MG_ERR_ARG, "mg_gemm: a triangular op(A) needs M == K, got %lld and %lld", (long long)a->m,
+                    (long long)a->k);
+    if (a->tri && a->split_k > 1) return fail(MG_ERR_ARG, "mg_gemm: tri runs unsplit; split_k is %d", a->split_k);
     if (a->res) {
         if (a->beta != 1) return fail(MG_ERR_ARG, "mg_gemm: res is what beta == 1 adds to; beta is %d", a->beta);
         if ((uintptr_t)a->res & 3) return fail(MG_ERR_ARG, "mg_gemm: res must be 4-byte aligned");
@@ -770,6 +777,7 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     p.Z = a.z;
     p.ldz = a.ldz;
     p.colsum = a.colsum;
+    p.tri = a.tri;
     p.R = (a.res && a.res != a.c) ? a.res : nullptr;
     p.ldr = a.ldr;
     p.ws = nullptr;

@@ -187,7 +187,10 @@ k_attn_softmax_bwd_reg(const float *dp, const uint16_t *p16, uint16_t *ds16, int
         pv[i][2] = widen16((uint16_t)(u.y & 0xffffu), dtype); pv[i][3] = widen16((uint16_t)(u.y >> 16), dtype);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            if (j0 + e > q) pv[i][e] = 0.f;       // beyond the query: P is zero there whatever the buffer holds
+            if (j0 + e > q) {                     // beyond the query P is zero and dP was never written
+                pv[i][e] = 0.f;
+                g[i][e] = 0.f;
+            }
             dot += g[i][e] * pv[i][e];
         }
     }

@@ -100,7 +100,7 @@ class Matmul:
         return m > 0 and n > 0 and k > 0
 
     def _args(self, a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side=False,
-              act=None, y16=None, ldy=None, z=None, ldz=None, colsum=None, res=None, ldr=None):
+              act=None, y16=None, ldy=None, z=None, ldz=None, colsum=None, res=None, ldr=None, tri=None):
         if self.batched:
             nb = int(nbatch)
             sa, sb, sc = (int(s) for s in strides)
@@ -163,6 +163,9 @@ class Matmul:
             raise VkError(f"{self.name}: act= needs y16= (the activated 16-bit output)")
         if c is None and y16 is None:
             raise VkError(f"{self.name}: C may only be omitted when y16 is given")
+        if tri not in L.TRI:
+            raise VkError(f"{self.name}: unknown tri {tri!r}; use None, 'c_lower', 'a_lower' or 'a_upper'")
+        ga.tri = L.TRI[tri]
         if res is not None:
             if c is None:
                 raise VkError(f"{self.name}: res= needs C (C = res + result)")
@@ -181,7 +184,7 @@ class Matmul:
 
     def __call__(self, a, b, c, m, n, k, repeat=1, graph=None, nbatch=1, strides=(0, 0, 0),
                  *, bias=None, accumulate=False, lda=None, ldb=None, ldc=None, side=False,
-                 act=None, y16=None, ldy=None, z=None, ldz=None, colsum=None, res=None, ldr=None):
+                 act=None, y16=None, ldy=None, z=None, ldz=None, colsum=None, res=None, ldr=None, tri=None):
         """side=True (recorded calls only) puts the GEMM on the device's side stream:
         it runs concurrently with the main stream between graph.fork() and graph.join().
         y16= (with act=None, 'gelu' or 'relu') makes the epilogue also write
@@ -192,12 +195,15 @@ class Matmul:
         receive g = result * act'(z), and colsum= (N floats, cleared by the caller unless
         accumulating) has the column sums of g added to it (col_sum, kernels.py:753-761).
         res= (an (m, n) f32 matrix) makes it C = res + result (+ bias): the `residual`
-        pass of the reference's transformer (tkernels.py:362-371) in the epilogue."""
+        pass of the reference's transformer (tkernels.py:362-371) in the epilogue.
+        tri= declares the causal structure of an attention GEMM so that work on masked
+        entries is skipped: 'c_lower' (only C[i, j <= i] is needed; the rest of C is left
+        as it was), 'a_lower' / 'a_upper' (op(A)[i, k] is zero for k > i / k < i)."""
         lib, ctx = self.dev._lib, self.dev._ctx
         if side and graph is None:
             raise VkError(f"{self.name}: side=True needs graph= (eager calls wait for their result); "
                           f"use enqueue(..., side=True) between dev.side_fork() and dev.side_join()")
-        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz, colsum, res, ldr)
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz, colsum, res, ldr, tri)
         if graph is not None:
             _check(lib.mg_gemm_check(C.byref(ga)), self.name)
             self._keep.append(ga)
@@ -230,9 +236,9 @@ class Matmul:
 
     def enqueue(self, a, b, c, m, n, k, nbatch=1, strides=(0, 0, 0), *, bias=None,
                 accumulate=False, lda=None, ldb=None, ldc=None, side=False, act=None, y16=None, ldy=None,
-                z=None, ldz=None, colsum=None, res=None, ldr=None):
+                z=None, ldz=None, colsum=None, res=None, ldr=None, tri=None):
         """Launch without waiting (the stream keeps order); for pipelined callers."""
-        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz, colsum, res, ldr)
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz, colsum, res, ldr, tri)
         _check(self.dev._lib.mg_gemm(self.dev._ctx, C.byref(ga)), self.name)
 
     def plan(self, m, n, k, nbatch=1, lda=None, ldb=None, ldc=None):

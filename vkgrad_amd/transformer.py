@@ -42,9 +42,10 @@ def _h16(ctx, *dims):
 class TCtx(Ctx):
     """`Ctx` + the transformer's row kernels under `.TK` (transformer.py:22-42)."""
 
-    def __init__(self, dev, tune=False, scalar_only=None, *, dtype="f16", fuse=False):
+    def __init__(self, dev, tune=False, scalar_only=None, *, dtype="f16", fuse=False, causal_gemms=True):
         super().__init__(dev, tune, scalar_only, dtype=dtype, fuse_bias=fuse)
         self.fuse = bool(fuse)
+        self.causal_gemms = bool(causal_gemms)   # attention GEMMs skip what the causal mask zeroes
         self.TK = make_transformer_kernels(dev, dtype)
         self.wave = dev.row_subgroup_size
 
@@ -156,19 +157,21 @@ class Attention:
         # per-head GEMMs as (M, N, K, trans_a, trans_b); a (T, hd) tensor advances `vec`
         # elements per head, a (T, T) tensor `sq`
         vec, sq = T * self.hd, T * T
+        # The last entry is the causal structure: scores and dP are only read at keys <= query;
+        # P and dS are zero beyond the query, so products with them stop (or start) there.
         self._head_gemms = {
-            "scores": (T, T, self.hd, False, True, (vec, vec, sq)),    # Q K^T
-            "mix":    (T, self.hd, T, False, False, (sq, vec, vec)),   # P V
-            "dV":     (T, self.hd, T, True, False, (sq, vec, vec)),    # P^T dOut
-            "dP":     (T, T, self.hd, False, True, (vec, vec, sq)),    # dOut V^T
-            "dQ":     (T, self.hd, T, False, False, (sq, vec, vec)),   # dS K
-            "dK":     (T, self.hd, T, True, False, (sq, vec, vec)),    # dS^T Q
+            "scores": (T, T, self.hd, False, True, (vec, vec, sq), "c_lower"),    # Q K^T
+            "mix":    (T, self.hd, T, False, False, (sq, vec, vec), "a_lower"),   # P V
+            "dV":     (T, self.hd, T, True, False, (sq, vec, vec), "a_upper"),    # P^T dOut
+            "dP":     (T, T, self.hd, False, True, (vec, vec, sq), "c_lower"),    # dOut V^T
+            "dQ":     (T, self.hd, T, False, False, (sq, vec, vec), "a_lower"),   # dS K
+            "dK":     (T, self.hd, T, True, False, (sq, vec, vec), "a_upper"),    # dS^T Q
         }
 
     def _heads(self, which, a, b, c, graph):
-        m, n, k, ta, tb, strides = self._head_gemms[which]
+        m, n, k, ta, tb, strides, tri = self._head_gemms[which]
         mm = self.ctx.matmul(m, n, k, trans_a=ta, trans_b=tb, batched=True, nbatch=self.nbh)
-        mm(a, b, c, m, n, k, graph=graph, nbatch=self.nbh, strides=strides)
+        mm(a, b, c, m, n, k, graph=graph, nbatch=self.nbh, strides=strides, tri=tri if self.ctx.causal_gemms else None)
 
     def _permute(self, name, buffers, graph):
         self.ctx.TK[name](buffers, self.rows * self.D, self.D, self.T, self.H, self.hd, graph=graph)
