@@ -149,137 +149,133 @@ def _seed(name):
 
 
 class Linear:
-    """y = act(x @ W + b), or the same without the activation."""
+    """One dense layer, y = act(x @ W + b) or, with activation=False, z = x @ W + b.
+
+    Buffers: `z` pre-activation (f32), `y16` activated output in the GEMM operand type,
+    `dz16` / `dz32` gradient w.r.t. z in both precisions, `dx32` gradient w.r.t. the input.
+    Two schedules (`ctx.fuse_bias`): separate passes as the reference issues them
+    (autograd.py:186-228), or the same arithmetic inside GEMM epilogues."""
+
+    ACTS = ("gelu", "relu")
 
     def __init__(self, ctx, batch, in_f, out_f, activation=True, need_dx=True, name="", act="gelu"):
-        self.ctx, self.name = ctx, name
-        self.batch, self.in_f, self.out_f = batch, in_f, out_f
-        self.activation = activation
-        if act not in ("gelu", "relu"):
+        if act not in self.ACTS:
             raise VkError(f"unknown activation {act!r}")
-        self.act = act
-        self.need_dx = need_dx
-        rng = np.random.default_rng(_seed(name))
-        w = (rng.standard_normal((in_f, out_f)) * np.sqrt(2.0 / in_f)).astype(np.float32)
-        self.W = Param(ctx, (in_f, out_f), w, name + ".W")
+        self.ctx, self.name, self.act = ctx, name, act
+        self.batch, self.in_f, self.out_f = batch, in_f, out_f
+        self.activation, self.need_dx = activation, need_dx
+        he = np.random.default_rng(_seed(name)).standard_normal((in_f, out_f)) * np.sqrt(2.0 / in_f)
+        self.W = Param(ctx, (in_f, out_f), he.astype(np.float32), name + ".W")
         self.b = Param(ctx, (out_f,), np.zeros(out_f, np.float32), name + ".b", no_decay=True)
-
-        self.acc = ctx.buf(batch * out_f * 4)
-        self.z = ctx.buf(batch * out_f * 4)
-        self.y16 = ctx.buf(batch * out_f * 2)
-        self.dz16 = ctx.buf(batch * out_f * 2)
-        self.dz32 = ctx.buf(batch * out_f * 4)
+        out_elems = batch * out_f
+        self.acc, self.z, self.dz32 = (ctx.buf(out_elems * 4) for _ in range(3))
+        self.y16, self.dz16 = ctx.buf(out_elems * 2), ctx.buf(out_elems * 2)
         self.dx32 = ctx.buf(batch * in_f * 4) if need_dx else None
         self.x16 = None
-        self._dz_ready = False   # set by the layer above when its dX epilogue wrote dz16 / dz32
-        self._db_ready = False   # ... and when it also summed this layer's bias gradient
+        # set by the layer above when its dX epilogue already produced this layer's dz (and db)
+        self._dz_ready = self._db_ready = False
 
+    # -- forward -------------------------------------------------------------------------
     def forward(self, x16, tape, graph=None):
-        c, K = self.ctx, self.ctx.K
         self.x16 = x16
-        n = self.batch * self.out_f
-        mm = c.matmul(self.batch, self.out_f, self.in_f)
-        if c.fuse_bias:
-            # z = x @ W + b straight out of the GEMM epilogue, and with an activation
-            # also y16 = narrow(act(z)): no separate pass over the (batch x out_f) tensor
-            if self.activation:
-                mm(x16, self.W.w16, self.z, self.batch, self.out_f, self.in_f, graph=graph, bias=self.b.w32,
-                   act=self.act, y16=self.y16)
-                out = self.y16
-            else:
-                mm(x16, self.W.w16, self.z, self.batch, self.out_f, self.in_f, graph=graph, bias=self.b.w32)
-                out = self.z
+        ctx, B, N, K = self.ctx, self.batch, self.out_f, self.in_f
+        gemm = ctx.matmul(B, N, K)
+        if ctx.fuse_bias:
+            # bias (and activation + narrowing) leave the GEMM's epilogue: no pass over (B, N) after it
+            extra = dict(act=self.act, y16=self.y16) if self.activation else {}
+            gemm(x16, self.W.w16, self.z, B, N, K, graph=graph, bias=self.b.w32, **extra)
         else:
-            mm(x16, self.W.w16, self.acc, self.batch, self.out_f, self.in_f, graph=graph)
+            gemm(x16, self.W.w16, self.acc, B, N, K, graph=graph)
             if self.activation:
-                K["bias_" + self.act]([self.acc, self.b.w32, self.z, self.y16], n, self.out_f, graph=graph)
-                out = self.y16
+                ctx.K["bias_" + self.act]([self.acc, self.b.w32, self.z, self.y16], B * N, N, graph=graph)
             else:
-                K["bias"]([self.acc, self.b.w32, self.z], n, self.out_f, graph=graph)
-                out = self.z
+                ctx.K["bias"]([self.acc, self.b.w32, self.z], B * N, N, graph=graph)
         tape.append(self.backward)
-        return out
+        return self.y16 if self.activation else self.z
+
+    # -- backward ------------------------------------------------------------------------
+    def _grad_wrt_z(self, dout16, dout32, graph):
+        """(16-bit, f32) gradient w.r.t. this layer's pre-activation."""
+        if not self.activation:
+            return dout16, dout32
+        if self._dz_ready:
+            self._dz_ready = False
+        else:
+            self.ctx.K["bias_" + self.act + "_bwd"]([dout32, self.z, self.dz16, self.dz32], self.batch * self.out_f,
+                                                    graph=graph)
+        return self.dz16, self.dz32
 
     def backward(self, dout16, dout32, graph=None, accumulate=False, below=None):
-        """`below`: the Linear whose output this layer consumed.  Under fuse_bias, when
-        that layer has an activation, this layer's dX GEMM multiplies by act'(below.z) in
-        its epilogue and writes below.dz16 / below.dz32 itself: the separate
-        activation-backward pass of the reference (autograd.py:204-207) disappears, and
-        (below.dz16, below.dz32) is returned in place of dX."""
-        c, K = self.ctx, self.ctx.K
-        n = self.batch * self.out_f
-        if self.activation and self._dz_ready:
-            self._dz_ready = False
-            g16, g32 = self.dz16, self.dz32
-        elif self.activation:
-            K["bias_" + self.act + "_bwd"]([dout32, self.z, self.dz16, self.dz32], n, graph=graph)
-            g16, g32 = self.dz16, self.dz32
-        else:
-            g16, g32 = dout16, dout32
+        """dout16 / dout32: dLoss/dOutput in both precisions (16-bit for the GEMMs, f32 for the
+        activation derivative and the bias sum).  Returns (g16, g32) for the layer below.
 
-        # dW = X^T @ dZ.  X is stored batch x in_f, which is K x M: trans_a.
-        c.matmul(self.in_f, self.out_f, self.batch, trans_a=True)(
-            self.x16, g16, self.W.g32, self.in_f, self.out_f, self.batch, graph=graph,
-            accumulate=accumulate)
+        `below`: the Linear whose output this layer consumed.  Under fuse_bias, when it has an
+        activation, this layer's dX GEMM multiplies by act'(below.z) in its epilogue and writes
+        below.dz16 / below.dz32 itself (with fuse_colsum also below's bias gradient), so the
+        separate activation-backward pass of the reference (autograd.py:204-207) disappears;
+        (below.dz16, below.dz32) is then returned in place of (None, dx32)."""
+        ctx, B, N, K = self.ctx, self.batch, self.out_f, self.in_f
+        g16, g32 = self._grad_wrt_z(dout16, dout32, graph)
+        # dW = x^T g : x is stored (B, K), i.e. (contraction, M) -> trans_a
+        ctx.matmul(K, N, B, trans_a=True)(self.x16, g16, self.W.g32, K, N, B, graph=graph, accumulate=accumulate)
         if self._db_ready:
             self._db_ready = False
         else:
-            K["col_sum_acc" if accumulate else "col_sum"]([g32, self.b.g32], self.out_f, self.batch, graph=graph)
-
+            ctx.K["col_sum_acc" if accumulate else "col_sum"]([g32, self.b.g32], N, B, graph=graph)
         if not self.need_dx:
             return None, None
-        # dX = dZ @ W^T.  W is stored in_f x out_f, which is N x K: trans_b.
-        mm = c.matmul(self.batch, self.in_f, self.out_f, trans_b=True)
-        if (c.fuse_bias and below is not None and below.activation
-                and (below.batch, below.out_f) == (self.batch, self.in_f)):
-            if c.fuse_colsum:
-                # db of the layer below comes out of the same epilogue; dz32 is then not needed
-                if not accumulate:
-                    K["zero"]([below.b.g32], below.out_f, graph=graph)
-                mm(g16, self.W.w16, None, self.batch, self.in_f, self.out_f, graph=graph,
-                   act=below.act + "_grad", z=below.z, y16=below.dz16, colsum=below.b.g32)
-                below._db_ready = True
-            else:
-                mm(g16, self.W.w16, below.dz32, self.batch, self.in_f, self.out_f, graph=graph,
-                   act=below.act + "_grad", z=below.z, y16=below.dz16)
-            below._dz_ready = True
-            return below.dz16, below.dz32
-        mm(g16, self.W.w16, self.dx32, self.batch, self.in_f, self.out_f, graph=graph)
-        return None, self.dx32
+        # dX = g W^T : W is stored (K, N), i.e. (N_out, contraction) -> trans_b
+        dx_gemm = ctx.matmul(B, K, N, trans_b=True)
+        fuse_down = (ctx.fuse_bias and below is not None and below.activation
+                     and (below.batch, below.out_f) == (B, K))
+        if not fuse_down:
+            dx_gemm(g16, self.W.w16, self.dx32, B, K, N, graph=graph)
+            return None, self.dx32
+        epilogue = dict(act=below.act + "_grad", z=below.z, y16=below.dz16)
+        if ctx.fuse_colsum:
+            # below's bias gradient comes out of the same epilogue; its f32 dz is then not needed
+            if not accumulate:
+                ctx.K["zero"]([below.b.g32], below.out_f, graph=graph)
+            dx_gemm(g16, self.W.w16, None, B, K, N, graph=graph, colsum=below.b.g32, **epilogue)
+            below._db_ready = True
+        else:
+            dx_gemm(g16, self.W.w16, below.dz32, B, K, N, graph=graph, **epilogue)
+        below._dz_ready = True
+        return below.dz16, below.dz32
 
 
 class MLP:
-    """Hidden layers use the activation; the head is linear and feeds softmax + CE.
-    Classes beyond n_classes (padding) are masked inside the softmax kernel.  The
-    reference pads the class count to a tile multiple (autograd.py:234-240);
-    ragged N is legal here, so pad_classes may equal n_classes."""
+    """Hidden layers with an activation, a linear head, softmax cross-entropy.  Classes
+    beyond n_classes are padding and masked inside the loss kernel.  The reference pads the
+    class count to a tile multiple (autograd.py:234-240); ragged N is legal here, so
+    pad_classes may equal n_classes."""
 
     def __init__(self, ctx, batch, sizes, n_classes, pad_classes=16, activation="gelu"):
         if pad_classes < n_classes:
             raise VkError(f"pad_classes {pad_classes} < n_classes {n_classes}")
         self.ctx, self.batch = ctx, batch
         self.n_classes, self.pad = n_classes, pad_classes
-        self.layers = []
-        for i in range(len(sizes) - 1):
-            self.layers.append(Linear(ctx, batch, sizes[i], sizes[i + 1], activation=True,
-                                      need_dx=(i > 0), name=f"fc{i}", act=activation))
-        self.layers.append(Linear(ctx, batch, sizes[-1], pad_classes, activation=False,
-                                  need_dx=True, name="head", act=activation))
+        widths = list(sizes) + [pad_classes]
+        last = len(widths) - 2
+        # hidden layers fc0, fc1, ... then the linear head; the first layer's input needs no gradient
+        self.layers = [Linear(ctx, batch, widths[i], widths[i + 1], activation=i < last, need_dx=i > 0 or i == last,
+                              name="head" if i == last else f"fc{i}", act=activation)
+                       for i in range(last + 1)]
         self.dlog16 = ctx.buf(batch * pad_classes * 2)
         self.dlog32 = ctx.buf(batch * pad_classes * 4)
         self.loss = ctx.buf(batch * 4, "cached")
         self._stage = {}   # HBM copies of host-mapped inputs, by buffer
 
     def params(self):
-        for l in self.layers:
-            yield l.W
-            yield l.b
+        for layer in self.layers:
+            yield from (layer.W, layer.b)
 
     def logits(self, x16, tape=None, graph=None):
-        h = x16
-        for l in self.layers:
-            h = l.forward(h, tape if tape is not None else [], graph=graph)
-        return h
+        tape = [] if tape is None else tape
+        out = x16
+        for layer in self.layers:
+            out = layer.forward(out, tape, graph=graph)
+        return out
 
     def _staged(self, buf, graph):
         """A buffer the CPU writes between replays (host-mapped, vk.py:583-590) is copied
@@ -287,50 +283,45 @@ class MLP:
         and dW of the first layer) then do not fetch it over PCIe."""
         if not buf.host_visible:
             return buf
-        dev_copy = self._stage.get(id(buf))
-        if dev_copy is None:
-            dev_copy = self._stage[id(buf)] = self.ctx.buf((buf.size + 3) // 4 * 4, "device")
-        self.ctx.K["copy"]([buf, dev_copy], buf.size // 4 * 4, graph=graph)
-        return dev_copy
+        if id(buf) not in self._stage:
+            self._stage[id(buf)] = self.ctx.buf((buf.size + 3) // 4 * 4, "device")
+        self.ctx.K["copy"]([buf, self._stage[id(buf)]], buf.size // 4 * 4, graph=graph)
+        return self._stage[id(buf)]
+
+    def _loss_and_backward(self, x16, labels_buf, graph, accumulate, after_loss=None):
+        tape = []
+        logits = self.logits(x16, tape, graph=graph)
+        self.ctx.K["softmax_ce"]([logits, labels_buf, self.dlog16, self.dlog32, self.loss],
+                                 self.batch, self.pad, self.n_classes, graph=graph)
+        result = after_loss() if after_loss is not None else None
+        grads = (self.dlog16, self.dlog32)
+        for depth in range(len(tape) - 1, -1, -1):
+            grads = tape[depth](*grads, graph=graph, accumulate=accumulate,
+                                below=self.layers[depth - 1] if depth else None)
+        return result
 
     def record(self, x16, labels_buf, graph, accumulate=False):
-        K = self.ctx.K
-        tape = []
-        x16, labels_buf = self._staged(x16, graph), self._staged(labels_buf, graph)
-        logits = self.logits(x16, tape, graph=graph)
-        K["softmax_ce"]([logits, labels_buf, self.dlog16, self.dlog32, self.loss],
-                        self.batch, self.pad, self.n_classes, graph=graph)
-        g16, g32 = self.dlog16, self.dlog32
-        for i in reversed(range(len(tape))):
-            g16, g32 = tape[i](g16, g32, graph=graph, accumulate=accumulate,
-                               below=self.layers[i - 1] if i > 0 else None)
+        self._loss_and_backward(self._staged(x16, graph), self._staged(labels_buf, graph), graph, accumulate)
 
     def read_loss(self):
         self.loss.invalidate()
         return float(self.loss.array(np.float32, (self.batch,)).mean())
 
     def forward_backward(self, x16, labels_buf, accumulate=False):
-        """Eager: one synchronous launch per kernel."""
-        K = self.ctx.K
-        tape = []
-        logits = self.logits(x16, tape)
-        K["softmax_ce"]([logits, labels_buf, self.dlog16, self.dlog32, self.loss],
-                        self.batch, self.pad, self.n_classes)
-        loss = self.read_loss()
-        g16, g32 = self.dlog16, self.dlog32
-        for i in reversed(range(len(tape))):
-            g16, g32 = tape[i](g16, g32, accumulate=accumulate, below=self.layers[i - 1] if i > 0 else None)
-        return loss
+        """Eager: one synchronous launch per kernel; returns the loss."""
+        return self._loss_and_backward(x16, labels_buf, None, accumulate, after_loss=self.read_loss)
 
     def predict(self, x16):
-        logits = self.logits(x16)
-        out = logits.download(np.float32, (self.batch, self.pad))[:, :self.n_classes]
-        return out.argmax(1).copy()
+        scores = self.logits(x16).download(np.float32, (self.batch, self.pad))
+        return scores[:, :self.n_classes].argmax(1).copy()
 
 
 class AdamW:
-    """One fused kernel per parameter (autograd.py:304-343); step-varying
-    scalars live in a mapped buffer so a recorded step stays valid."""
+    """Decoupled-weight-decay Adam, one fused kernel per parameter (autograd.py:304-343).
+    The scalars that change from step to step (learning rate, bias corrections) sit in a
+    mapped buffer the CPU rewrites, so a recorded step stays valid; the kernels read an HBM
+    copy of it made by the step's first launch instead of reaching over PCIe from every
+    wavefront."""
 
     def __init__(self, ctx, params, lr=1e-3, b1=0.9, b2=0.999, eps=1e-8, wd=0.01):
         self.ctx, self.params = ctx, list(params)
@@ -338,39 +329,33 @@ class AdamW:
         self.t = 0
         self.hp = ctx.buf(8 * 4, "shared")
         self.hpv = self.hp.array(np.float32)
-        # the kernels read the scalars from HBM: one staging copy per step instead of a
-        # PCIe read of the mapped buffer from every wavefront of every parameter's kernel
         self.hp_dev = ctx.buf(8 * 4, "device")
         self._set_hp(lr)
 
     def _set_hp(self, lr):
-        bc1 = 1 - self.b1 ** max(self.t, 1)
-        bc2 = 1 - self.b2 ** max(self.t, 1)
-        self.hpv[:6] = [lr, self.b1, self.b2, bc1, bc2, self.eps]
+        t = max(self.t, 1)
+        self.hpv[:6] = [lr, self.b1, self.b2, 1 - self.b1 ** t, 1 - self.b2 ** t, self.eps]
         self.hp.flush()
 
     def advance(self, lr=None):
+        """Count a step and publish its scalars (call before replaying a recorded step)."""
         self.t += 1
         self._set_hp(self.lr if lr is None else lr)
 
     def record(self, graph):
-        k = self.ctx.K["adamw"]
-        self.ctx.K["copy"]([self.hp, self.hp_dev], 8 * 4, graph=graph)
+        K = self.ctx.K
+        K["copy"]([self.hp, self.hp_dev], 8 * 4, graph=graph)
         for p in self.params:
-            wd = 0.0 if p.no_decay else self.wd
-            k([p.w32, p.g32, p.m, p.v, p.w16, self.hp_dev], p.n, wd, graph=graph)
+            K["adamw"]([p.w32, p.g32, p.m, p.v, p.w16, self.hp_dev], p.n, 0.0 if p.no_decay else self.wd, graph=graph)
 
     def step(self, lr=None):
         self.advance(lr)
-        k = self.ctx.K["adamw"]
-        self.ctx.K["copy"]([self.hp, self.hp_dev], 8 * 4)
-        for p in self.params:
-            wd = 0.0 if p.no_decay else self.wd
-            k([p.w32, p.g32, p.m, p.v, p.w16, self.hp_dev], p.n, wd)
+        self.record(None)
 
 
 class TrainStep:
-    """The whole step recorded once and replayed (autograd.py:346-366)."""
+    """Forward, loss, backward and optimiser recorded once, replayed per step
+    (autograd.py:346-366); call it after writing the batch into the mapped input buffers."""
 
     def __init__(self, model, opt, xbuf, ybuf):
         self.model, self.opt = model, opt
