@@ -46,7 +46,7 @@ def test_layernorm_forward_backward(dev, tk):
     dtype, TK = tk
     W = dev.row_subgroup_size
     rng = np.random.default_rng(0)
-    for rows, D in ((5, 48), (64, 768), (33, 100), (2, 1)):
+    for rows, D in ((5, 48), (64, 768), (33, 100), (2, 1), (9, 300), (7, 1024), (3, 1028), (6, 77)):
         x = (rng.standard_normal((rows, D)) * 2 + 1).astype(np.float32)
         g = rng.uniform(0.5, 1.5, D).astype(np.float32)
         b = rng.standard_normal(D).astype(np.float32)
@@ -111,7 +111,7 @@ def test_attention_softmax_forward_backward(dev, tk):
 def test_head_permutes(dev, tk):
     dtype, TK = tk
     rng = np.random.default_rng(2)
-    for B, T, H, hd in ((2, 5, 3, 4), (1, 64, 12, 64)):
+    for B, T, H, hd in ((2, 5, 3, 4), (1, 64, 12, 64), (2, 7, 3, 5)):      # the last: no groups of four
         D, rows = H * hd, B * T
         qkv = rng.standard_normal((rows, 3 * D)).astype(np.float32)
         bias = rng.standard_normal(3 * D).astype(np.float32)
@@ -194,6 +194,21 @@ def test_embeddings_residual_and_column_sums(dev, tk):
             assert np.allclose(bsum.download(np.float32, (D,)), 2 * RT.col_sum16(got16, dtype), rtol=1e-6, atol=1e-5)
         finally:
             for t in (ba, br, bb, bo, b16, bsum):
+                t.destroy()
+        # sizes that are not multiples of four take the element-wise forms of the same kernels
+        r2, d2 = 3, 25
+        acc2, res2 = rng.standard_normal((r2, d2)).astype(np.float32), rng.standard_normal((r2, d2)).astype(np.float32)
+        bias2 = rng.standard_normal(d2).astype(np.float32)
+        ba, br, bb, bo, b16 = up(dev, acc2), up(dev, res2), up(dev, bias2), dev.buffer(r2 * d2 * 4, "device"), dev.buffer(r2 * d2 * 2, "device")
+        try:
+            TK["residual"]([ba, bb, br, bo], r2 * d2, d2)
+            assert np.array_equal(bo.download(np.float32, (r2, d2)), (res2 + acc2) + bias2[None, :])
+            TK["add"]([ba, br, bo], r2 * d2)
+            assert np.array_equal(bo.download(np.float32, (r2, d2)), acc2 + res2)
+            TK["to16"]([ba, b16], r2 * d2)
+            assert np.array_equal(stored(b16, dtype, (r2, d2)).view(np.uint16), O.round_to(acc2, dtype).view(np.uint16))
+        finally:
+            for t in (ba, br, bb, bo, b16):
                 t.destroy()
         big = O.round_to(rng.integers(-4, 4, (1500, 70)).astype(np.float32), dtype)
         bbig, bs2 = up(dev, big.view(np.uint16)), dev.buffer(70 * 4, "device")

@@ -138,6 +138,19 @@ __global__ void k_cast16(const float *src, uint16_t *dst, int64_t n, int dtype) 
     if (i < n) dst[i] = narrow16(src[i], dtype);
 }
 
+// four elements per thread: one 16-byte load, one 8-byte store; the tail goes element by element
+__global__ void k_cast16_v4(const float *src, uint16_t *dst, int64_t n, int dtype) {
+    const int64_t i4 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i4 * 4 + 3 < n) {
+        const float4 t = reinterpret_cast<const float4 *>(src)[i4];
+        reinterpret_cast<uint2 *>(dst)[i4] =
+            make_uint2((uint32_t)narrow16(t.x, dtype) | ((uint32_t)narrow16(t.y, dtype) << 16),
+                       (uint32_t)narrow16(t.z, dtype) | ((uint32_t)narrow16(t.w, dtype) << 16));
+    } else {
+        for (int64_t i = i4 * 4; i < n; i++) dst[i] = narrow16(src[i], dtype);
+    }
+}
+
 __global__ void k_scale_copy(float *dst, const float *src, int64_t n, float scale) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) dst[i] = src[i] * scale;
@@ -232,7 +245,11 @@ int mg_ew_zero(mg_ctx *ctx, float *dst, int64_t n) {
 
 int mg_ew_cast16(mg_ctx *ctx, const float *src, void *dst, int64_t n, int dtype) {
     EW_PRECHECK("mg_ew_cast16", src && dst && count_ok(n) && dtype_ok(dtype));
-    hipLaunchKernelGGL(k_cast16, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), src, (uint16_t *)dst, n, dtype);
+    if ((((uintptr_t)src & 15) | ((uintptr_t)dst & 7)) == 0)
+        hipLaunchKernelGGL(k_cast16_v4, dim3(blocks_for((n + 3) / 4)), dim3(256), 0, ctx_stream(ctx), src, (uint16_t *)dst, n,
+                           dtype);
+    else
+        hipLaunchKernelGGL(k_cast16, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), src, (uint16_t *)dst, n, dtype);
     EW_POSTCHECK("mg_ew_cast16");
 }
 

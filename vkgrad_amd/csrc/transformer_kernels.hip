@@ -56,6 +56,104 @@ k_layernorm(const float *x, const float *gamma, const float *beta, uint16_t *y16
     for (int d = lane; d < D; d += 64) yr[d] = narrow16((xr[d] - m) * r * gamma[d] + beta[d], dtype);
 }
 
+__device__ __forceinline__ uint2 narrow16x4(float a, float b, float c, float d, int dtype) {
+    return make_uint2((uint32_t)narrow16(a, dtype) | ((uint32_t)narrow16(b, dtype) << 16),
+                      (uint32_t)narrow16(c, dtype) | ((uint32_t)narrow16(d, dtype) << 16));
+}
+
+// LayerNorm with the row in registers (D % 4 == 0, D <= 256 NV): lane l holds the float4 groups
+// l, l + 64, ...; one 16-byte load per group, statistics from registers, 8-byte stores.
+template <int NV>
+__global__ void __launch_bounds__(64 * ROWS_PER_WG)
+k_layernorm_reg(const float *x, const float *gamma, const float *beta, uint16_t *y16, float *mu, float *rstd,
+                int64_t rows, int D, int dtype) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * ROWS_PER_WG + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int ngroups = D >> 2;
+    const float4 *xr = reinterpret_cast<const float4 *>(x + row * D);
+    float4 v[NV];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int g = lane + 64 * i;
+        v[i] = g < ngroups ? xr[g] : make_float4(0.f, 0.f, 0.f, 0.f);
+        s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    }
+    const float m = wave_sum(s) / (float)D;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        if (lane + 64 * i < ngroups) {
+            const float a = v[i].x - m, b = v[i].y - m, c = v[i].z - m, d = v[i].w - m;
+            q += (a * a + b * b) + (c * c + d * d);
+        }
+    }
+    const float r = rsqrtf(wave_sum(q) / (float)D + 1e-5f);
+    if (lane == 0) {
+        mu[row] = m;
+        rstd[row] = r;
+    }
+    uint2 *yr = reinterpret_cast<uint2 *>(y16 + row * D);
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int g = lane + 64 * i;
+        if (g < ngroups) {
+            const float4 ga = reinterpret_cast<const float4 *>(gamma)[g], be = reinterpret_cast<const float4 *>(beta)[g];
+            yr[g] = narrow16x4((v[i].x - m) * r * ga.x + be.x, (v[i].y - m) * r * ga.y + be.y,
+                               (v[i].z - m) * r * ga.z + be.z, (v[i].w - m) * r * ga.w + be.w, dtype);
+        }
+    }
+}
+
+template <int NV>
+__global__ void __launch_bounds__(64 * ROWS_PER_WG)
+k_layernorm_bwd_reg(const float *dy, const float *x, const float *gamma, const float *mu, const float *rstd, float *dx,
+                    uint16_t *dyxh16, uint16_t *dy16, int64_t rows, int D, int dtype) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * ROWS_PER_WG + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int ngroups = D >> 2;
+    const float m = mu[row], r = rstd[row];
+    const float4 *xr = reinterpret_cast<const float4 *>(x + row * D);
+    const float4 *gr = reinterpret_cast<const float4 *>(dy + row * D);
+    uint2 *o1 = reinterpret_cast<uint2 *>(dyxh16 + row * D), *o2 = reinterpret_cast<uint2 *>(dy16 + row * D);
+    float xh[NV][4], dxh[NV][4];
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int g = lane + 64 * i;
+        if (g < ngroups) {
+            const float4 xv = xr[g], gv = gr[g], ga = reinterpret_cast<const float4 *>(gamma)[g];
+            const float xs[4] = {xv.x, xv.y, xv.z, xv.w}, gs[4] = {gv.x, gv.y, gv.z, gv.w};
+            const float gm[4] = {ga.x, ga.y, ga.z, ga.w};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                xh[i][e] = (xs[e] - m) * r;
+                dxh[i][e] = gs[e] * gm[e];
+                s1 += dxh[i][e];
+                s2 += dxh[i][e] * xh[i][e];
+            }
+            o1[g] = narrow16x4(gs[0] * xh[i][0], gs[1] * xh[i][1], gs[2] * xh[i][2], gs[3] * xh[i][3], dtype);
+            o2[g] = narrow16x4(gs[0], gs[1], gs[2], gs[3], dtype);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) xh[i][e] = dxh[i][e] = 0.f;
+        }
+    }
+    s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    const float inv = 1.0f / (float)D;
+    float4 *dxr = reinterpret_cast<float4 *>(dx + row * D);
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int g = lane + 64 * i;
+        if (g < ngroups)
+            dxr[g] = make_float4(r * (dxh[i][0] - s1 * inv - xh[i][0] * s2 * inv), r * (dxh[i][1] - s1 * inv - xh[i][1] * s2 * inv),
+                                 r * (dxh[i][2] - s1 * inv - xh[i][2] * s2 * inv), r * (dxh[i][3] - s1 * inv - xh[i][3] * s2 * inv));
+    }
+}
+
 // LayerNorm backward (tkernels.py:58-92): dx = rstd * (dxh - mean(dxh) - xh * mean(dxh * xh)) with
 // dxh = dy * gamma; also emits dy * xh and dy in 16 bits for the column sums of dgamma and dbeta.
 __global__ void __launch_bounds__(64 * ROWS_PER_WG)
@@ -276,6 +374,59 @@ __global__ void k_split_heads(const float *src, uint16_t *dst16, int64_t n, int 
     dst16[head_index(i, D, T, H, hd).head] = narrow16(src[i], dtype);
 }
 
+// The permutes four elements at a time (hd % 4 == 0: a group never straddles two heads).
+__global__ void k_split_qkv_v4(const float *qkv, const float *bias, uint16_t *q16, uint16_t *k16, uint16_t *v16,
+                               int64_t n4, int D, int T, int H, int hd, int dtype) {
+    const int64_t i4 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i4 >= n4) return;
+    const HeadIdx x = head_index(i4 * 4, D, T, H, hd);
+    const float *src = qkv + x.bt * 3 * D + x.d;
+    uint16_t *dst[3] = {q16, k16, v16};
+#pragma unroll
+    for (int w = 0; w < 3; w++) {
+        float4 t = *reinterpret_cast<const float4 *>(src + w * D);
+        if (bias) {
+            const float4 b = *reinterpret_cast<const float4 *>(bias + x.d + w * D);
+            t.x += b.x; t.y += b.y; t.z += b.z; t.w += b.w;
+        }
+        *reinterpret_cast<uint2 *>(dst[w] + x.head) = narrow16x4(t.x, t.y, t.z, t.w, dtype);
+    }
+}
+__global__ void k_merge_qkv_grad_v4(const float *dq, const float *dk, const float *dv, uint16_t *dqkv16, int64_t n4, int D,
+                                    int T, int H, int hd, int dtype) {
+    const int64_t i4 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i4 >= n4) return;
+    const HeadIdx x = head_index(i4 * 4, D, T, H, hd);
+    uint16_t *dst = dqkv16 + x.bt * 3 * D + x.d;
+    const float *src[3] = {dq, dk, dv};
+#pragma unroll
+    for (int w = 0; w < 3; w++) {
+        const float4 t = *reinterpret_cast<const float4 *>(src[w] + x.head);
+        *reinterpret_cast<uint2 *>(dst + w * D) = narrow16x4(t.x, t.y, t.z, t.w, dtype);
+    }
+}
+__global__ void k_heads_v4(const float *src, uint16_t *dst16, int64_t n4, int D, int T, int H, int hd, int dtype,
+                           int to_heads) {
+    const int64_t i4 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i4 >= n4) return;
+    const int64_t head = head_index(i4 * 4, D, T, H, hd).head;
+    const float4 t = *reinterpret_cast<const float4 *>(src + (to_heads ? i4 * 4 : head));
+    *reinterpret_cast<uint2 *>(dst16 + (to_heads ? head : i4 * 4)) = narrow16x4(t.x, t.y, t.z, t.w, dtype);
+}
+// out = a + b (+ bias[i % D]) and 16-bit narrowing, four elements per thread
+__global__ void k_add_v4(const float *a, const float *b, const float *bias, float *out, int64_t n4, int D) {
+    const int64_t i4 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i4 >= n4) return;
+    float4 x = reinterpret_cast<const float4 *>(a)[i4];
+    const float4 y = reinterpret_cast<const float4 *>(b)[i4];
+    x.x += y.x; x.y += y.y; x.z += y.z; x.w += y.w;
+    if (bias) {
+        const float4 c = *reinterpret_cast<const float4 *>(bias + (i4 * 4) % D);
+        x.x += c.x; x.y += c.y; x.z += c.z; x.w += c.w;
+    }
+    reinterpret_cast<float4 *>(out)[i4] = x;
+}
+
 // ---- Embeddings (tkernels.py:303-360): x = tok[ids] + pos[t]; t restarts at the sample's start
 // when seg is given.  Backward is a scatter-add (several positions share a vocabulary row).
 __global__ void k_embed(const float *tok, const float *pos, const uint32_t *ids, const uint32_t *seg, float *x, int64_t n,
@@ -424,6 +575,10 @@ k_softmax_ce_wide(const float *logits, const uint32_t *labels, const float *weig
     }
 }
 
+static inline bool aligned16(const void *a, const void *b, const void *c) {
+    return (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15) == 0;   // NULL counts as aligned
+}
+static inline bool aligned8(const void *a) { return ((uintptr_t)a & 7) == 0; }
 static inline unsigned row_blocks(int64_t rows) { return (unsigned)((rows + ROWS_PER_WG - 1) / ROWS_PER_WG); }
 static inline bool heads_ok(int64_t n, int D, int T, int H, int hd) {
     return count_ok(n) && D > 0 && T > 0 && H > 0 && hd > 0 && (int64_t)H * hd == D && n % ((int64_t)D * T) == 0;
@@ -439,8 +594,14 @@ int mg_tk_layernorm(mg_ctx *ctx, const float *x, const float *gamma, const float
                     float *rstd, int64_t rows, int64_t D, int dtype) {
     EW_PRECHECK("mg_tk_layernorm", x && gamma && beta && y16 && mu && rstd && count_ok(rows) && D > 0 &&
                                        D <= 0x7fffffff && dtype_ok(dtype));
-    hipLaunchKernelGGL(k_layernorm, dim3(row_blocks(rows)), dim3(64 * ROWS_PER_WG), 0, ctx_stream(ctx), x, gamma, beta,
-                       (uint16_t *)y16, mu, rstd, rows, (int)D, dtype);
+    const bool vec = D % 4 == 0 && D <= 1024 && aligned16(x, gamma, beta) && aligned8(y16);
+    const dim3 grid(row_blocks(rows)), block(64 * ROWS_PER_WG);
+    uint16_t *y = (uint16_t *)y16;
+    if (vec && D <= 256) hipLaunchKernelGGL(k_layernorm_reg<1>, grid, block, 0, ctx_stream(ctx), x, gamma, beta, y, mu, rstd, rows, (int)D, dtype);
+    else if (vec && D <= 512) hipLaunchKernelGGL(k_layernorm_reg<2>, grid, block, 0, ctx_stream(ctx), x, gamma, beta, y, mu, rstd, rows, (int)D, dtype);
+    else if (vec && D <= 768) hipLaunchKernelGGL(k_layernorm_reg<3>, grid, block, 0, ctx_stream(ctx), x, gamma, beta, y, mu, rstd, rows, (int)D, dtype);
+    else if (vec) hipLaunchKernelGGL(k_layernorm_reg<4>, grid, block, 0, ctx_stream(ctx), x, gamma, beta, y, mu, rstd, rows, (int)D, dtype);
+    else hipLaunchKernelGGL(k_layernorm, grid, block, 0, ctx_stream(ctx), x, gamma, beta, y, mu, rstd, rows, (int)D, dtype);
     EW_POSTCHECK("mg_tk_layernorm");
 }
 
@@ -448,8 +609,15 @@ int mg_tk_layernorm_bwd(mg_ctx *ctx, const float *dy, const float *x, const floa
                         const float *rstd, float *dx, void *dyxh16, void *dy16, int64_t rows, int64_t D, int dtype) {
     EW_PRECHECK("mg_tk_layernorm_bwd", dy && x && gamma && mu && rstd && dx && dyxh16 && dy16 && count_ok(rows) &&
                                            D > 0 && D <= 0x7fffffff && dtype_ok(dtype));
-    hipLaunchKernelGGL(k_layernorm_bwd, dim3(row_blocks(rows)), dim3(64 * ROWS_PER_WG), 0, ctx_stream(ctx), dy, x, gamma,
-                       mu, rstd, dx, (uint16_t *)dyxh16, (uint16_t *)dy16, rows, (int)D, dtype);
+    const bool vec = D % 4 == 0 && D <= 1024 && aligned16(dy, x, gamma) && aligned16(dx, dx, dx) && aligned8(dyxh16) &&
+                     aligned8(dy16);
+    const dim3 grid(row_blocks(rows)), block(64 * ROWS_PER_WG);
+    uint16_t *o1 = (uint16_t *)dyxh16, *o2 = (uint16_t *)dy16;
+    if (vec && D <= 256) hipLaunchKernelGGL(k_layernorm_bwd_reg<1>, grid, block, 0, ctx_stream(ctx), dy, x, gamma, mu, rstd, dx, o1, o2, rows, (int)D, dtype);
+    else if (vec && D <= 512) hipLaunchKernelGGL(k_layernorm_bwd_reg<2>, grid, block, 0, ctx_stream(ctx), dy, x, gamma, mu, rstd, dx, o1, o2, rows, (int)D, dtype);
+    else if (vec && D <= 768) hipLaunchKernelGGL(k_layernorm_bwd_reg<3>, grid, block, 0, ctx_stream(ctx), dy, x, gamma, mu, rstd, dx, o1, o2, rows, (int)D, dtype);
+    else if (vec) hipLaunchKernelGGL(k_layernorm_bwd_reg<4>, grid, block, 0, ctx_stream(ctx), dy, x, gamma, mu, rstd, dx, o1, o2, rows, (int)D, dtype);
+    else hipLaunchKernelGGL(k_layernorm_bwd, grid, block, 0, ctx_stream(ctx), dy, x, gamma, mu, rstd, dx, o1, o2, rows, (int)D, dtype);
     EW_POSTCHECK("mg_tk_layernorm_bwd");
 }
 
@@ -487,8 +655,12 @@ int mg_tk_split_qkv(mg_ctx *ctx, const float *qkv, const float *bias, void *q16,
                     int64_t D, int64_t T, int64_t H, int64_t hd, int dtype) {
     EW_PRECHECK("mg_tk_split_qkv", qkv && q16 && k16 && v16 && heads_ok(n, (int)D, (int)T, (int)H, (int)hd) &&
                                        dtype_ok(dtype));
-    hipLaunchKernelGGL(k_split_qkv, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), qkv, bias, (uint16_t *)q16,
-                       (uint16_t *)k16, (uint16_t *)v16, n, (int)D, (int)T, (int)H, (int)hd, dtype);
+    if (hd % 4 == 0 && aligned16(qkv, bias, bias) && aligned8(q16) && aligned8(k16) && aligned8(v16))
+        hipLaunchKernelGGL(k_split_qkv_v4, dim3(blocks_for(n / 4)), dim3(256), 0, ctx_stream(ctx), qkv, bias, (uint16_t *)q16,
+                           (uint16_t *)k16, (uint16_t *)v16, n / 4, (int)D, (int)T, (int)H, (int)hd, dtype);
+    else
+        hipLaunchKernelGGL(k_split_qkv, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), qkv, bias, (uint16_t *)q16,
+                           (uint16_t *)k16, (uint16_t *)v16, n, (int)D, (int)T, (int)H, (int)hd, dtype);
     EW_POSTCHECK("mg_tk_split_qkv");
 }
 
@@ -496,24 +668,36 @@ int mg_tk_merge_qkv_grad(mg_ctx *ctx, const float *dq, const float *dk, const fl
                          int64_t D, int64_t T, int64_t H, int64_t hd, int dtype) {
     EW_PRECHECK("mg_tk_merge_qkv_grad", dq && dk && dv && dqkv16 && heads_ok(n, (int)D, (int)T, (int)H, (int)hd) &&
                                             dtype_ok(dtype));
-    hipLaunchKernelGGL(k_merge_qkv_grad, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), dq, dk, dv,
-                       (uint16_t *)dqkv16, n, (int)D, (int)T, (int)H, (int)hd, dtype);
+    if (hd % 4 == 0 && aligned16(dq, dk, dv) && aligned8(dqkv16))
+        hipLaunchKernelGGL(k_merge_qkv_grad_v4, dim3(blocks_for(n / 4)), dim3(256), 0, ctx_stream(ctx), dq, dk, dv,
+                           (uint16_t *)dqkv16, n / 4, (int)D, (int)T, (int)H, (int)hd, dtype);
+    else
+        hipLaunchKernelGGL(k_merge_qkv_grad, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), dq, dk, dv,
+                           (uint16_t *)dqkv16, n, (int)D, (int)T, (int)H, (int)hd, dtype);
     EW_POSTCHECK("mg_tk_merge_qkv_grad");
 }
 
 int mg_tk_merge_heads(mg_ctx *ctx, const float *src, void *y16, int64_t n, int64_t D, int64_t T, int64_t H, int64_t hd,
                       int dtype) {
     EW_PRECHECK("mg_tk_merge_heads", src && y16 && heads_ok(n, (int)D, (int)T, (int)H, (int)hd) && dtype_ok(dtype));
-    hipLaunchKernelGGL(k_merge_heads, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), src, (uint16_t *)y16, n, (int)D,
-                       (int)T, (int)H, (int)hd, dtype);
+    if (hd % 4 == 0 && aligned16(src, src, src) && aligned8(y16))
+        hipLaunchKernelGGL(k_heads_v4, dim3(blocks_for(n / 4)), dim3(256), 0, ctx_stream(ctx), src, (uint16_t *)y16, n / 4,
+                           (int)D, (int)T, (int)H, (int)hd, dtype, 0);
+    else
+        hipLaunchKernelGGL(k_merge_heads, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), src, (uint16_t *)y16, n, (int)D,
+                           (int)T, (int)H, (int)hd, dtype);
     EW_POSTCHECK("mg_tk_merge_heads");
 }
 
 int mg_tk_split_heads(mg_ctx *ctx, const float *src, void *dst16, int64_t n, int64_t D, int64_t T, int64_t H,
                       int64_t hd, int dtype) {
     EW_PRECHECK("mg_tk_split_heads", src && dst16 && heads_ok(n, (int)D, (int)T, (int)H, (int)hd) && dtype_ok(dtype));
-    hipLaunchKernelGGL(k_split_heads, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), src, (uint16_t *)dst16, n,
-                       (int)D, (int)T, (int)H, (int)hd, dtype);
+    if (hd % 4 == 0 && aligned16(src, src, src) && aligned8(dst16))
+        hipLaunchKernelGGL(k_heads_v4, dim3(blocks_for(n / 4)), dim3(256), 0, ctx_stream(ctx), src, (uint16_t *)dst16, n / 4,
+                           (int)D, (int)T, (int)H, (int)hd, dtype, 1);
+    else
+        hipLaunchKernelGGL(k_split_heads, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), src, (uint16_t *)dst16, n,
+                           (int)D, (int)T, (int)H, (int)hd, dtype);
     EW_POSTCHECK("mg_tk_split_heads");
 }
 
@@ -538,13 +722,20 @@ int mg_tk_embed_bwd(mg_ctx *ctx, const float *dx, const uint32_t *ids, const uin
 int mg_tk_residual(mg_ctx *ctx, const float *acc, const float *bias, const float *res, float *out, int64_t n,
                    int64_t D) {
     EW_PRECHECK("mg_tk_residual", acc && bias && res && out && count_ok(n) && D > 0 && D <= 0x7fffffff);
-    hipLaunchKernelGGL(k_residual, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), acc, bias, res, out, n, (int)D);
+    if (n % 4 == 0 && D % 4 == 0 && aligned16(acc, bias, res) && aligned16(out, out, out))
+        hipLaunchKernelGGL(k_add_v4, dim3(blocks_for(n / 4)), dim3(256), 0, ctx_stream(ctx), res, acc, bias, out, n / 4, (int)D);
+    else
+        hipLaunchKernelGGL(k_residual, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), acc, bias, res, out, n, (int)D);
     EW_POSTCHECK("mg_tk_residual");
 }
 
 int mg_tk_add(mg_ctx *ctx, const float *a, const float *b, float *out, int64_t n) {
     EW_PRECHECK("mg_tk_add", a && b && out && count_ok(n));
-    hipLaunchKernelGGL(k_add, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), a, b, out, n);
+    if (n % 4 == 0 && aligned16(a, b, out))
+        hipLaunchKernelGGL(k_add_v4, dim3(blocks_for(n / 4)), dim3(256), 0, ctx_stream(ctx), a, b, (const float *)nullptr, out,
+                           n / 4, 4);
+    else
+        hipLaunchKernelGGL(k_add, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), a, b, out, n);
     EW_POSTCHECK("mg_tk_add");
 }
 
