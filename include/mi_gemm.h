@@ -264,6 +264,20 @@ int mg_ew_softmax_ce(mg_ctx *ctx, const float *logits, const uint32_t *labels, v
 int mg_ew_adamw(mg_ctx *ctx, float *w, const float *g, float *m, float *v, void *w16,
                 const float *hp, int64_t n, float wd, int dtype);
 /* zero (kernels.py:853-854) */
+/* The same update for a list of parameters in one launch (the reference launches adamw once per
+ * parameter, autograd.py:331-343: 148 launches in a GPT-2-small step, most of them a few
+ * microseconds of work).  table_dev: `ntensors` entries in device memory, ordered, first_block =
+ * the sum of ceil(n / 1024) over the entries before; total_blocks = that sum over all entries.
+ * vec != 0 promises that w, g, m, v are 16-byte and w16 8-byte aligned. */
+typedef struct {
+    float *w; const float *g; float *m; float *v; void *w16;
+    int64_t n;
+    int64_t first_block;
+    float wd;
+    int32_t vec;
+} mg_adamw_entry;
+int mg_ew_adamw_multi(mg_ctx *ctx, const mg_adamw_entry *table_dev, int ntensors, int64_t total_blocks, const float *hp,
+                      int dtype);
 int mg_ew_zero(mg_ctx *ctx, float *dst, int64_t n);
 /* Device-side copy of nbytes (multiple of 4, both pointers 4-byte aligned) that can be
  * recorded into a graph, unlike mg_copy.  The reference's recorded step reads what the CPU

@@ -227,7 +227,8 @@ def test_embeddings_residual_and_column_sums(dev, tk):
 def test_wide_softmax_cross_entropy(dev, tk):
     dtype, TK = tk
     rng = np.random.default_rng(4)
-    for rows, stride, ncls in ((6, 16, 10), (5, 1040, 1000), (3, 50304, 50257)):
+    for rows, stride, ncls in ((6, 16, 10), (5, 1040, 1000), (3, 50304, 50257), (3, 4100, 4099), (2, 20480, 20000),
+                               (2, 60000, 59999), (2, 3001, 3000)):
         logits = (rng.standard_normal((rows, stride)) * 2).astype(np.float32)
         logits[:, ncls:] = 1e4                                      # padding must be masked
         labels = rng.integers(0, ncls, rows).astype(np.uint32)

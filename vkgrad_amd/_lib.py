@@ -42,6 +42,11 @@ class GemmArgs(C.Structure):
     ]
 
 
+class AdamWEntry(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("g", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p), ("w16", C.c_void_p),
+                ("n", C.c_int64), ("first_block", C.c_int64), ("wd", C.c_float), ("vec", C.c_int32)]
+
+
 class Tile(C.Structure):
     _fields_ = [
         ("id", C.c_int32), ("bm", C.c_int32), ("bn", C.c_int32), ("bk", C.c_int32),
@@ -94,6 +99,7 @@ SIGNATURES = {
     "mg_ew_col_sum": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int64, C.c_int]),
     "mg_ew_softmax_ce": (C.c_int, [_P, _P, _P, _P, _P, _P, C.c_int64, C.c_int64, C.c_int64, C.c_int]),
     "mg_ew_adamw": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, C.c_int64, C.c_float, C.c_int]),
+    "mg_ew_adamw_multi": (C.c_int, [_P, _P, C.c_int, C.c_int64, _P, C.c_int]),
     "mg_ew_zero": (C.c_int, [_P, _P, C.c_int64]),
     "mg_ew_copy": (C.c_int, [_P, _P, _P, C.c_int64]),
     "mg_ew_cast16": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int]),

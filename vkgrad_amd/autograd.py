@@ -16,12 +16,14 @@ Extensions (all off by default keep the reference's exact kernel sequence):
     Linear.backward(accumulate=True)   dW += (beta=1 epilogue), db +=
 """
 
+import ctypes as C
 import os
 import zlib
 
 import numpy as np
 
-from .kernels import CONFIGS, Matmul, autotune_matmul, lookup_tuned, make_kernels
+from . import _lib as L
+from .kernels import CONFIGS, Elementwise, Matmul, autotune_matmul, lookup_tuned, make_kernels
 from .vk import VkError
 
 
@@ -330,6 +332,7 @@ class AdamW:
         self.hp = ctx.buf(8 * 4, "shared")
         self.hpv = self.hp.array(np.float32)
         self.hp_dev = ctx.buf(8 * 4, "device")
+        self._table_dev, self._blocks = None, 0
         self._set_hp(lr)
 
     def _set_hp(self, lr):
@@ -342,11 +345,34 @@ class AdamW:
         self.t += 1
         self._set_hp(self.lr if lr is None else lr)
 
+    def _table(self):
+        """Device table of (w, g, m, v, w16, n, first workgroup, weight decay) per parameter for
+        the one-launch update; a workgroup covers 1024 elements."""
+        if self._table_dev is None:
+            entries = (L.AdamWEntry * len(self.params))()
+            blocks = 0
+            for e, p in zip(entries, self.params):
+                e.w, e.g, e.m, e.v, e.w16 = p.w32.ptr, p.g32.ptr, p.m.ptr, p.v.ptr, p.w16.ptr
+                e.n, e.first_block, e.wd = p.n, blocks, 0.0 if p.no_decay else self.wd
+                e.vec = int(all(ptr % 16 == 0 for ptr in (e.w, e.g, e.m, e.v)) and e.w16 % 8 == 0)
+                blocks += -(-p.n // 1024)
+            self._table_dev = self.ctx.buf(C.sizeof(entries), "device")
+            self._table_dev.upload(np.frombuffer(entries, dtype=np.uint8))
+            self._blocks = blocks
+        return self._table_dev
+
     def record(self, graph):
-        K = self.ctx.K
-        K["copy"]([self.hp, self.hp_dev], 8 * 4, graph=graph)
-        for p in self.params:
-            K["adamw"]([p.w32, p.g32, p.m, p.v, p.w16, self.hp_dev], p.n, 0.0 if p.no_decay else self.wd, graph=graph)
+        """Stage the step's scalars into HBM, then update every parameter in one launch (the
+        reference launches the kernel once per parameter, autograd.py:331-343)."""
+        ctx = self.ctx
+        ctx.K["copy"]([self.hp, self.hp_dev], 8 * 4, graph=graph)
+        table, lib, dt = self._table(), ctx.dev._lib, L.DTYPES[ctx.dtype]
+        n, blocks = len(self.params), self._blocks
+
+        def launch(lib, mg, ptrs, _n):
+            return lib.mg_ew_adamw_multi(mg, ptrs[0], n, blocks, ptrs[1], dt)
+
+        Elementwise(ctx.dev, "adamw_multi", launch)([table, self.hp_dev], n, graph=graph)
 
     def step(self, lr=None):
         self.advance(lr)

@@ -128,6 +128,52 @@ __global__ void k_adamw(float *w, const float *g, float *m, float *v, uint16_t *
     if (w16) w16[i] = narrow16(wi, dtype);
 }
 
+// AdamW over a list of parameters in one launch.  The table holds one entry per parameter and the
+// number of its first workgroup; a workgroup finds its parameter by bisection and updates 1024
+// consecutive elements of it, four per thread (same arithmetic as k_adamw, element by element).
+__device__ __forceinline__ float adamw_one(float &w, float g, float &m, float &v, float lr, float b1, float b2,
+                                           float bc1, float bc2, float eps, float wd) {
+    m = b1 * m + (1.0f - b1) * g;
+    v = b2 * v + (1.0f - b2) * g * g;
+    w -= lr * ((m / bc1) / (sqrtf(v / bc2) + eps) + wd * w);
+    return w;
+}
+__global__ void __launch_bounds__(256) k_adamw_multi(const mg_adamw_entry *table, int ntensors, const float *hp, int dtype) {
+    int lo = 0, hi = ntensors - 1;
+    while (lo < hi) {                      // last entry whose first_block <= blockIdx.x
+        const int mid = (lo + hi + 1) >> 1;
+        if (table[mid].first_block <= (int64_t)blockIdx.x) lo = mid;
+        else hi = mid - 1;
+    }
+    const mg_adamw_entry e = table[lo];
+    const float lr = hp[0], b1 = hp[1], b2 = hp[2], bc1 = hp[3], bc2 = hp[4], eps = hp[5];
+    const int64_t i0 = (((int64_t)blockIdx.x - e.first_block) * 256 + threadIdx.x) * 4;
+    if (i0 >= e.n) return;
+    float *w = e.w + i0, *m = e.m + i0, *v = e.v + i0;
+    const float *g = e.g + i0;
+    uint16_t *w16 = e.w16 ? (uint16_t *)e.w16 + i0 : nullptr;
+    if (i0 + 3 < e.n && e.vec) {
+        float4 wv = *reinterpret_cast<float4 *>(w), mv = *reinterpret_cast<float4 *>(m), vv = *reinterpret_cast<float4 *>(v);
+        const float4 gv = *reinterpret_cast<const float4 *>(g);
+        adamw_one(wv.x, gv.x, mv.x, vv.x, lr, b1, b2, bc1, bc2, eps, e.wd);
+        adamw_one(wv.y, gv.y, mv.y, vv.y, lr, b1, b2, bc1, bc2, eps, e.wd);
+        adamw_one(wv.z, gv.z, mv.z, vv.z, lr, b1, b2, bc1, bc2, eps, e.wd);
+        adamw_one(wv.w, gv.w, mv.w, vv.w, lr, b1, b2, bc1, bc2, eps, e.wd);
+        *reinterpret_cast<float4 *>(w) = wv;
+        *reinterpret_cast<float4 *>(m) = mv;
+        *reinterpret_cast<float4 *>(v) = vv;
+        if (w16)
+            *reinterpret_cast<uint2 *>(w16) =
+                make_uint2((uint32_t)narrow16(wv.x, dtype) | ((uint32_t)narrow16(wv.y, dtype) << 16),
+                           (uint32_t)narrow16(wv.z, dtype) | ((uint32_t)narrow16(wv.w, dtype) << 16));
+    } else {
+        for (int k = 0; k < 4 && i0 + k < e.n; k++) {
+            const float wi = adamw_one(w[k], g[k], m[k], v[k], lr, b1, b2, bc1, bc2, eps, e.wd);
+            if (w16) w16[k] = narrow16(wi, dtype);
+        }
+    }
+}
+
 __global__ void k_zero(float *dst, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) dst[i] = 0.f;
@@ -235,6 +281,15 @@ int mg_ew_adamw(mg_ctx *ctx, float *w, const float *g, float *m, float *v, void 
     hipLaunchKernelGGL(k_adamw, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), w, g, m, v, (uint16_t *)w16, hp, n,
                        wd, dtype);
     EW_POSTCHECK("mg_ew_adamw");
+}
+
+int mg_ew_adamw_multi(mg_ctx *ctx, const mg_adamw_entry *table_dev, int ntensors, int64_t total_blocks, const float *hp,
+                      int dtype) {
+    EW_PRECHECK("mg_ew_adamw_multi", table_dev && ntensors > 0 && total_blocks > 0 && total_blocks <= 0x7fffffff && hp &&
+                                         dtype_ok(dtype));
+    hipLaunchKernelGGL(k_adamw_multi, dim3((unsigned)total_blocks), dim3(256), 0, ctx_stream(ctx), table_dev, ntensors, hp,
+                       dtype);
+    EW_POSTCHECK("mg_ew_adamw_multi");
 }
 
 int mg_ew_zero(mg_ctx *ctx, float *dst, int64_t n) {
