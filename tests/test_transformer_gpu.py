@@ -216,6 +216,19 @@ def test_embeddings_residual_and_column_sums(dev, tk):
             TK["col_sum_zero"]([bs2], 70)
             TK["col_sum_chunk16"]([bbig, bs2], 32 * 70, 70, 1500, 32)
             assert np.array_equal(bs2.download(np.float32, (70,)), RT.col_sum16(big, dtype))
+            # the one-launch form overwrites whatever sums held, call after call (the chunks'
+            # arrival counters are back at zero after each launch)
+            for _ in range(3):
+                bs2.upload(np.full(70, np.nan, np.float32))
+                TK["col_sum16"]([bbig, bs2], 70, 1500)
+                assert np.array_equal(bs2.download(np.float32, (70,)), RT.col_sum16(big, dtype))
+            TK["col_sum_chunk16"]([bbig, bs2], 32 * 70, 70, 1500, 32)
+            assert np.array_equal(bs2.download(np.float32, (70,)), 2 * RT.col_sum16(big, dtype))
+            b32 = up(dev, O.widen(big, dtype))
+            bs2.upload(np.full(70, np.nan, np.float32))
+            TK["col_sum"]([b32, bs2], 70, 1500)
+            assert np.array_equal(bs2.download(np.float32, (70,)), RT.col_sum16(big, dtype))
+            b32.destroy()
         finally:
             bbig.destroy()
             bs2.destroy()

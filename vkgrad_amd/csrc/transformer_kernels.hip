@@ -466,7 +466,10 @@ __global__ void k_add_bias(float *x, const float *bias, int64_t n, int64_t ncol)
 
 // Column sums of a 16-bit matrix, f32 accumulation (tkernels.py:258-270): same blocking as the
 // f32 column sum: 64 columns x 512 rows per block, 8 row lanes per column, chunks of rows meet
-// through float atomics (the host clears sums first unless accumulating).
+// through float atomics (the host clears sums first unless accumulating).  (Parking the chunks'
+// partial sums in a scratch and letting the block that arrives last add them in order - no
+// clear, no atomics, reproducible bits - was measured too: 7 us slower per call at 8192 rows,
+// 0.7 ms on a GPT-2-small step, so the atomics stay.)
 constexpr int CS16_ROWS = 512;
 __global__ void __launch_bounds__(512)
 k_col_sum16(const uint16_t *g, float *sums, int64_t ncol, int64_t nrow, int accumulate, int atomic, int dtype) {

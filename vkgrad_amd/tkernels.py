@@ -89,6 +89,9 @@ def make_transformer_kernels(dev, dtype="f16"):
         lib.mg_ew_col_sum(ctx, p[0], p[1], int(ncol), int(nrow), 1))
     add("col_sum_chunk16", lambda lib, ctx, p, n, ncol, nrow, nchunk:
         lib.mg_tk_col_sum16(ctx, p[0], p[1], int(ncol), int(nrow), 1, dt))
+    # one-launch forms (no clear needed): buffers: g16 (or g32), sums ; n = ncol ; args: nrow
+    add("col_sum16", lambda lib, ctx, p, n, nrow: lib.mg_tk_col_sum16(ctx, p[0], p[1], n, int(nrow), 0, dt))
+    add("col_sum", lambda lib, ctx, p, n, nrow: lib.mg_ew_col_sum(ctx, p[0], p[1], n, int(nrow), 0))
     # buffers: tok, pos, ids, x / tok, pos, ids, seg, x ; n = rows * D ; args: D, T
     add("embed", lambda lib, ctx, p, n, D, T: lib.mg_tk_embed(ctx, p[0], p[1], p[2], None, p[3], n, int(D), int(T)))
     add("embed_doc", lambda lib, ctx, p, n, D, T: lib.mg_tk_embed(ctx, p[0], p[1], p[2], p[3], p[4], n, int(D), int(T)))

@@ -54,10 +54,10 @@ class TCtx(Ctx):
         self.TK[name](buffers, rows * self.wave, *args, graph=graph)
 
     def col_sum(self, src, dst, ncol, nrow, graph=None, f16=True):
-        """dst[c] = sum over rows of src[r, c]; reads the 16-bit copy unless f16=False."""
-        self.TK["col_sum_zero"]([dst], ncol, graph=graph)
-        self.TK["col_sum_chunk16" if f16 else "col_sum_chunk"]([src, dst], NCHUNK * ncol, ncol, nrow, NCHUNK,
-                                                                graph=graph)
+        """dst[c] = sum over rows of src[r, c]; reads the 16-bit copy unless f16=False.  The
+        library clears dst itself when the rows span several chunks (the reference's
+        `col_sum_zero` + `col_sum_chunk16` pair, transformer.py:30-37, in one call)."""
+        self.TK["col_sum16" if f16 else "col_sum"]([src, dst], ncol, nrow, graph=graph)
 
     def destroy(self):
         for kern in self.TK.values():
