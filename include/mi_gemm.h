@@ -55,7 +55,8 @@ enum { MG_DEVICE = 0, MG_SHARED = 1, MG_CACHED = 2, MG_BAR = 3 };
 /* activations for the companion elementwise kernels and the fused GEMM epilogues; the
  * _GRAD forms exist for mg_gemm only (result times the activation's derivative at z) */
 enum { MG_TRI_NONE = 0, MG_TRI_C_LOWER = 1, MG_TRI_A_LOWER = 2, MG_TRI_A_UPPER = 3 };
-enum { MG_ACT_NONE = 0, MG_ACT_GELU = 1, MG_ACT_RELU = 2, MG_ACT_GELU_GRAD = 3, MG_ACT_RELU_GRAD = 4 };
+enum { MG_ACT_NONE = 0, MG_ACT_GELU = 1, MG_ACT_RELU = 2, MG_ACT_GELU_GRAD = 3, MG_ACT_RELU_GRAD = 4,
+       MG_ACT_SOFTMAX_GRAD = 5 };
 
 typedef struct {
     int32_t struct_size;   /* sizeof(mg_gemm_args), checked */
@@ -113,6 +114,20 @@ typedef struct {
      * The A forms need m == k and run unsplit; every batch has the same structure. */
     int32_t tri;           /* MG_TRI_* */
     int32_t reserved;      /* 0 */
+    /* Softmax-backward epilogue - replaces the separate pass of attn_softmax_bwd
+     * (tkernels.py:167-187; its call site transformer.py:171-176): with act =
+     * MG_ACT_SOFTMAX_GRAD the dP = dOut V^T GEMM of attention writes
+     *   y16[i][j] = narrow(scale * p16[i][j] * (result[i][j] - rowsub[i]))
+     * (and the same value to C in f32 when C is given), where p16 is the 16-bit softmax
+     * output P (m, n) and rowsub[i] = sum_j P[i][j] dP[i][j], which the caller obtains without
+     * dP as sum_d dOut[i][d] * Out[i][d] (mg_tk_attn_rowdot).  Masked entries need no test of
+     * their own: P is zero there.  beta == 0, no bias, layouts NN and NT; batches are allowed:
+     * y16 and p16 advance sc elements per batch (they have the shape of C), rowsub m floats. */
+    const void *p16;       /* NULL unless act == MG_ACT_SOFTMAX_GRAD */
+    int64_t ldp;           /* its row pitch in elements (>= n) */
+    const float *rowsub;   /* m floats per batch */
+    float scale;
+    int32_t reserved2;     /* 0 */
 } mg_gemm_args;
 
 /* The buffers of A and B end at their last element: row padding (ld beyond the stored
@@ -315,6 +330,10 @@ int mg_tk_attn_softmax(mg_ctx *ctx, const float *s, const uint32_t *seg, void *p
 /* attn_softmax_bwd (tkernels.py:167-187): ds16 = narrow(P * (dP - sum_j dP_j P_j) * scale) */
 int mg_tk_attn_softmax_bwd(mg_ctx *ctx, const float *dp, const void *p16, void *ds16, int64_t rows, int64_t T,
                            float scale, int dtype);
+/* out[r] = sum_d a16[r][d] * b32[r][d] over `rows` rows of D elements.  With a16 = dOut and
+ * b32 = Out (head-side) this is the row term sum_j P_j dP_j of attn_softmax_bwd
+ * (tkernels.py:167-187), formed without P or dP: the `rowsub` of MG_ACT_SOFTMAX_GRAD. */
+int mg_tk_attn_rowdot(mg_ctx *ctx, const void *a16, const float *b32, float *out, int64_t rows, int64_t D, int dtype);
 /* split_qkv (tkernels.py:195-213): (B*T, 3D) f32 + bias[3D] (or NULL) -> q16, k16, v16 head-side */
 int mg_tk_split_qkv(mg_ctx *ctx, const float *qkv, const float *bias, void *q16, void *k16, void *v16, int64_t n,
                     int64_t D, int64_t T, int64_t H, int64_t hd, int dtype);

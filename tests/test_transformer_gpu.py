@@ -108,6 +108,54 @@ def test_attention_softmax_forward_backward(dev, tk):
                 t.destroy()
 
 
+def test_softmax_backward_in_the_dp_gemm(dev, tk):
+    """act='softmax_grad': dS leaves the epilogue of dP = dOut V^T (batched over the heads),
+    with the row term sum_j P_j dP_j taken from attn_rowdot(dOut, Out).  Checked against the
+    separate-pass oracle (attn_softmax_bwd on the f32 dP), for every tile that carries the
+    epilogue, with and without the causal tile skipping, ragged sizes included."""
+    from vkgrad_amd.kernels import Matmul
+    dtype, TK = tk
+    W = dev.row_subgroup_size
+    rng = np.random.default_rng(11)
+    for nbh, T, hd in ((3, 200, 40), (2, 64, 64), (1, 1024, 64), (2, 330, 24)):
+        rows = nbh * T
+        scale = 1.0 / np.sqrt(hd)
+        s = (rng.standard_normal((rows, T)) * 2).astype(np.float32)
+        p16 = RT.attn_softmax(s, T, 1.0, dtype)
+        p = O.widen(p16, dtype).reshape(nbh, T, T)
+        v16 = O.round_to(rng.standard_normal((nbh, T, hd)).astype(np.float32), dtype)
+        do16 = O.round_to(rng.standard_normal((nbh, T, hd)).astype(np.float32), dtype)
+        v, do = O.widen(v16, dtype), O.widen(do16, dtype)
+        out32 = np.einsum("bij,bjd->bid", p, v).astype(np.float32)
+        dp = np.einsum("bid,bjd->bij", do, v).astype(np.float32)
+        want = RT.attn_softmax_bwd(dp.reshape(rows, T), p16, T, scale, dtype)
+        bp, bv, bdo, bout = up(dev, p16), up(dev, v16), up(dev, do16), up(dev, out32)
+        bsum, bds, bc = dev.buffer(rows * 4, "device"), dev.buffer(rows * T * 2, "device"), dev.buffer(rows * T * 4, "device")
+        try:
+            TK["attn_rowdot"]([bdo, bout, bsum], rows * W, hd)
+            dot = bsum.download(np.float32, (rows,))
+            ref_dot = (dp * p).sum(2, dtype=np.float64).reshape(rows)
+            assert np.abs(dot - ref_dot).max() <= 1e-5 * max(1.0, np.abs(ref_dot).max())
+            for tile in (None, 3, 4, 10, 11):
+                for tri in (None, "c_lower"):
+                    bds.upload(np.zeros(rows * T, np.uint16))
+                    mm = Matmul(dev, trans_b=True, batched=True, dtype=dtype, tile=tile)
+                    mm(bdo, bv, None, T, T, hd, nbatch=nbh, strides=(T * hd, T * hd, T * T), tri=tri,
+                       act="softmax_grad", y16=bds, p16=bp, rowsub=bsum, scale=scale)
+                    got = stored(bds, dtype, (rows, T))
+                    assert close16(got, want, dtype, slack=5e-5), (nbh, T, hd, tile, tri)
+            # the f32 copy of the same values, one head
+            mm = Matmul(dev, trans_b=True, dtype=dtype)
+            mm(bdo, bv, bc, T, T, hd, act="softmax_grad", y16=bds, p16=bp, rowsub=bsum, scale=scale)
+            c = bc.download(np.float32, (rows, T))[:T]
+            exact = (p[0] * (dp[0] - ref_dot[:T, None]) * scale).astype(np.float32)
+            assert np.abs(c - exact).max() <= 5e-5
+            assert np.array_equal(stored(bds, dtype, (rows, T))[:T], O.round_to(c, dtype))
+        finally:
+            for t in (bp, bv, bdo, bout, bsum, bds, bc):
+                t.destroy()
+
+
 def test_head_permutes(dev, tk):
     dtype, TK = tk
     rng = np.random.default_rng(2)

@@ -17,10 +17,10 @@ MG_FLAG_SIDE_STREAM = 4
 
 DTYPES = {"f16": MG_F16, "bf16": MG_BF16}
 KINDS = {"device": MG_DEVICE, "shared": MG_SHARED, "cached": MG_CACHED, "bar": MG_BAR}
-MG_ACT_GELU_GRAD, MG_ACT_RELU_GRAD = 3, 4
+MG_ACT_GELU_GRAD, MG_ACT_RELU_GRAD, MG_ACT_SOFTMAX_GRAD = 3, 4, 5
 TRI = {None: 0, "c_lower": 1, "a_lower": 2, "a_upper": 3}
 ACTS = {None: MG_ACT_NONE, "none": MG_ACT_NONE, "gelu": MG_ACT_GELU, "relu": MG_ACT_RELU,
-        "gelu_grad": MG_ACT_GELU_GRAD, "relu_grad": MG_ACT_RELU_GRAD}
+        "gelu_grad": MG_ACT_GELU_GRAD, "relu_grad": MG_ACT_RELU_GRAD, "softmax_grad": MG_ACT_SOFTMAX_GRAD}
 
 
 class GemmArgs(C.Structure):
@@ -39,6 +39,8 @@ class GemmArgs(C.Structure):
         ("z", C.c_void_p), ("ldz", C.c_int64), ("colsum", C.c_void_p),
         ("res", C.c_void_p), ("ldr", C.c_int64),
         ("tri", C.c_int32), ("reserved", C.c_int32),
+        ("p16", C.c_void_p), ("ldp", C.c_int64), ("rowsub", C.c_void_p),
+        ("scale", C.c_float), ("reserved2", C.c_int32),
     ]
 
 
@@ -110,6 +112,7 @@ SIGNATURES = {
     "mg_tk_layernorm_bwd": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, C.c_int]),
     "mg_tk_attn_softmax": (C.c_int, [_P, _P, _P, _P, _I, _I, _I, C.c_float, C.c_int]),
     "mg_tk_attn_softmax_bwd": (C.c_int, [_P, _P, _P, _P, _I, _I, C.c_float, C.c_int]),
+    "mg_tk_attn_rowdot": (C.c_int, [_P, _P, _P, _P, _I, _I, C.c_int]),
     "mg_tk_split_qkv": (C.c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, C.c_int]),
     "mg_tk_merge_qkv_grad": (C.c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, C.c_int]),
     "mg_tk_merge_heads": (C.c_int, [_P, _P, _P, _I, _I, _I, _I, _I, C.c_int]),

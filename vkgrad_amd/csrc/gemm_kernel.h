@@ -68,6 +68,13 @@ struct GemmParams {
     const float *R;       // beta = 1 reads this matrix instead of C (or NULL)
     int64_t ldr;
     int tri;              // MG_TRI_*: causal structure (non-persistent kernels only)
+    // MG_ACT_SOFTMAX_GRAD: Y = narrow(scale * P16 * (result - rowsub[row])); Y and P16 advance
+    // sy elements per batch, rowsub M floats
+    const uint16_t *P16;
+    int64_t ldp;
+    const float *rowsub;
+    float scale;
+    int64_t sy;
 };
 
 template <int DT>
@@ -348,6 +355,11 @@ __device__ __forceinline__ void tri_k_range(int tri, int m0, int &kbeg, int &ken
 // 16-bit narrowing (round to nearest even) and the activations of the fused output;
 // same formulas as the companion kernels (reference kernels.py:625-629, 709-718).
 template <int DT>
+__device__ __forceinline__ float widen16_of(uint16_t b) {
+    if constexpr (DT == D_F16) return (float)__builtin_bit_cast(_Float16, b);
+    else return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+template <int DT>
 __device__ __forceinline__ uint16_t narrow16_rne(float x) {
     if constexpr (DT == D_F16) {
         return __builtin_bit_cast(uint16_t, (_Float16)x);
@@ -395,10 +407,14 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, float *C, f32x16
     const int col_l = n0 + wave_n * WTN + (lane & 31);
     float *cl = C + (int64_t)row_l * p.ldc + col_l;
     const int64_t ldc = p.ldc;
-    uint16_t *yl = ACT ? p.Y + (int64_t)row_l * p.ldy + col_l : nullptr;
+    uint16_t *yl = ACT ? p.Y + (int64_t)blockIdx.z * p.sy + (int64_t)row_l * p.ldy + col_l : nullptr;
     const int64_t ldy = ACT ? p.ldy : 0;
-    const bool have_c = !ACT || C != nullptr;
-    const bool grad = ACT && p.act >= 3;
+    const bool have_c = !ACT || p.C != nullptr;   // (C carries the batch offset: test the argument)
+    const bool grad = ACT && (p.act == 3 || p.act == 4);
+    const bool sgrad = ACT && p.act == 5;   // MG_ACT_SOFTMAX_GRAD
+    const uint16_t *pl = sgrad ? p.P16 + (int64_t)blockIdx.z * p.sy + (int64_t)row_l * p.ldp + col_l : nullptr;
+    const int64_t ldp = sgrad ? p.ldp : 0;
+    const float *rsl = sgrad ? p.rowsub + (int64_t)blockIdx.z * p.M + row_l : nullptr;
     // what beta = 1 adds to: C itself, or the residual matrix
     const float *rl = p.R ? p.R + (int64_t)row_l * p.ldr + col_l : cl;
     const int64_t ldr = p.R ? p.ldr : ldc;
@@ -416,6 +432,16 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, float *C, f32x16
         for (int j = 0; j < TN; j++) cs[j] = 0.f;
 #pragma unroll
         for (int i = 0; i < TM; i++) {
+            float rsub[16];   // what MG_ACT_SOFTMAX_GRAD subtracts from this lane's 16 rows
+            if constexpr (ACT && MODE == 0) {
+                if (sgrad) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int ro = (r >> 2) * 8 + (r & 3);
+                        rsub[r] = (!EDGE || row_l + i * 32 + ro < p.M) ? rsl[i * 32 + ro] : 0.f;
+                    }
+                }
+            }
 #pragma unroll
             for (int j = 0; j < TN; j++) {
                 float *ct = cl + (int64_t)(i * 32) * ldc + j * 32;
@@ -441,6 +467,15 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, float *C, f32x16
                             old[r] = ok ? __builtin_nontemporal_load(zt + ro * ldz) : 0.f;
                         }
                     }
+                    if (sgrad) {
+                        const uint16_t *pt = pl + (int64_t)(i * 32) * ldp + j * 32;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const int ro = (r >> 2) * 8 + (r & 3);
+                            const bool ok = col_ok && (!EDGE || row_l + i * 32 + ro < p.M);
+                            old[r] = ok ? widen16_of<DT>(pt[ro * ldp]) : 0.f;
+                        }
+                    }
                 }
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
@@ -453,6 +488,7 @@ __device__ __forceinline__ void store_tile(const GemmParams &p, float *C, f32x16
                             v *= fused_dact(old[r], p.act);
                             cs[j] += ok ? v : 0.f;
                         }
+                        if (sgrad) v = p.scale * old[r] * (v - rsub[r]);
                     }
                     if (ok) {
                         if constexpr (MODE == 2) {

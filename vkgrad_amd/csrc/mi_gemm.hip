@@ -295,7 +295,7 @@ static void finish_plan(const mg_gemm_args &a, int tile, int split, Plan &pl) {
     int64_t kblocks = cdiv(a.k, d->bk);
     if (split > kblocks) split = (int)kblocks;
     if (split < 1) split = 1;
-    if (d->persistent == 2 || d->gemv || a.tri) split = 1;
+    if (d->persistent == 2 || d->gemv || a.tri || a.act == MG_ACT_SOFTMAX_GRAD) split = 1;
     int64_t kb_per = cdiv(kblocks, split);
     split = (int)cdiv(kblocks, kb_per);   // no empty slices
     while (!dma_eligible(a, *d, kb_per * d->bk, split) && d->fallback != tile) {
@@ -389,9 +389,21 @@ static int check_args(const mg_gemm_args *a) {
     if (!a->a || !a->b) return fail(MG_ERR_ARG, "mg_gemm: NULL operand pointer");
     if (!a->c && !(a->y16 && a->beta == 0))
         return fail(MG_ERR_ARG, "mg_gemm: C may only be NULL with y16 given and beta == 0");
-    if (a->act < MG_ACT_NONE || a->act > MG_ACT_RELU_GRAD) return fail(MG_ERR_ARG, "mg_gemm: unknown activation %d", a->act);
+    if (a->act < MG_ACT_NONE || a->act > MG_ACT_SOFTMAX_GRAD) return fail(MG_ERR_ARG, "mg_gemm: unknown activation %d", a->act);
     if (!a->y16 && a->act != MG_ACT_NONE) return fail(MG_ERR_ARG, "mg_gemm: an activation needs the y16 output");
-    if (a->act >= MG_ACT_GELU_GRAD) {
+    if (a->act == MG_ACT_SOFTMAX_GRAD) {
+        if (!a->p16 || !a->rowsub) return fail(MG_ERR_ARG, "mg_gemm: MG_ACT_SOFTMAX_GRAD needs p16 and rowsub");
+        if (((uintptr_t)a->p16 & 1) || ((uintptr_t)a->rowsub & 3))
+            return fail(MG_ERR_ARG, "mg_gemm: p16 must be 2-byte and rowsub 4-byte aligned");
+        if (a->ldp < a->n) return fail(MG_ERR_ARG, "mg_gemm: ldp %lld < N %lld", (long long)a->ldp, (long long)a->n);
+        if (a->beta != 0 || a->bias) return fail(MG_ERR_ARG, "mg_gemm: MG_ACT_SOFTMAX_GRAD needs beta == 0 and no bias");
+        if (a->z || a->colsum) return fail(MG_ERR_ARG, "mg_gemm: z and colsum belong to the GELU / ReLU _GRAD activations");
+        if (!(a->scale == a->scale)) return fail(MG_ERR_ARG, "mg_gemm: scale is NaN");
+        if (a->nbatch > 1 && (a->sc < (a->m - 1) * a->ldy + a->n || a->sc < (a->m - 1) * a->ldp + a->n))
+            return fail(MG_ERR_ARG, "mg_gemm: batch stride sc %lld overlaps the batches of y16 or p16", (long long)a->sc);
+    } else if (a->p16 || a->rowsub) {
+        return fail(MG_ERR_ARG, "mg_gemm: p16 and rowsub belong to MG_ACT_SOFTMAX_GRAD");
+    } else if (a->act >= MG_ACT_GELU_GRAD) {
         if (!a->z) return fail(MG_ERR_ARG, "mg_gemm: a _GRAD activation needs the pre-activation z");
         if ((uintptr_t)a->z & 3) return fail(MG_ERR_ARG, "mg_gemm: z must be 4-byte aligned");
         if (a->ldz < a->n) return fail(MG_ERR_ARG, "mg_gemm: ldz %lld < N %lld", (long long)a->ldz, (long long)a->n);
@@ -402,7 +414,8 @@ static int check_args(const mg_gemm_args *a) {
     }
     if (a->y16) {
         if (a->layout == MG_TN) return fail(MG_ERR_ARG, "mg_gemm: the fused y16 output exists for layouts NN and NT only");
-        if (a->nbatch != 1) return fail(MG_ERR_ARG, "mg_gemm: the fused y16 output needs nbatch == 1");
+        if (a->nbatch != 1 && a->act != MG_ACT_SOFTMAX_GRAD)
+            return fail(MG_ERR_ARG, "mg_gemm: the fused y16 output needs nbatch == 1 (except with MG_ACT_SOFTMAX_GRAD)");
         if ((uintptr_t)a->y16 & 1) return fail(MG_ERR_ARG, "mg_gemm: y16 must be 2-byte aligned");
         if (a->ldy < a->n) return fail(MG_ERR_ARG, "mg_gemm: ldy %lld < N %lld", (long long)a->ldy, (long long)a->n);
         if (a->flags & MG_FLAG_SPLITK_ATOMIC)
@@ -777,6 +790,11 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
     p.Z = a.z;
     p.ldz = a.ldz;
     p.colsum = a.colsum;
+    p.P16 = (const uint16_t *)a.p16;
+    p.ldp = a.ldp;
+    p.rowsub = a.rowsub;
+    p.scale = a.scale;
+    p.sy = (a.y16 && a.nbatch > 1) ? a.sc : 0;
     p.tri = a.tri;
     p.R = (a.res && a.res != a.c) ? a.res : nullptr;
     p.ldr = a.ldr;

@@ -306,6 +306,21 @@ k_attn_softmax_bwd_reg(const float *dp, const uint16_t *p16, uint16_t *ds16, int
     }
 }
 
+// out[r] = sum_d a16[r][d] * b32[r][d], one wavefront per row.  With a = dOut and b = Out (both
+// head-side, D = head width) this is sum_j P[r][j] dP[r][j] of the softmax backward
+// (tkernels.py:167-187) without P or dP: dP = dOut V^T and Out = P V.
+__global__ void __launch_bounds__(64 * ROWS_PER_WG)
+k_attn_rowdot(const uint16_t *a16, const float *b32, float *out, int64_t rows, int D, int dtype) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * ROWS_PER_WG + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int64_t base = row * D;
+    float dot = 0.f;
+    for (int d = lane; d < D; d += 64) dot += widen16(a16[base + d], dtype) * b32[base + d];
+    dot = wave_sum(dot);
+    if (lane == 0) out[row] = dot;
+}
+
 // dS = P * (dP - sum_j dP_j P_j) * scale over the unmasked keys (tkernels.py:167-187); masked keys
 // hold P = 0, so only j <= q is read.
 __global__ void __launch_bounds__(64 * ROWS_PER_WG)
@@ -655,6 +670,13 @@ int mg_tk_attn_softmax_bwd(mg_ctx *ctx, const float *dp, const void *p16, void *
     else if (vec) hipLaunchKernelGGL(k_attn_softmax_bwd_reg<4>, grid, block, 0, ctx_stream(ctx), dp, p, d, rows, (int)T, scale, dtype);
     else hipLaunchKernelGGL(k_attn_softmax_bwd, grid, block, 0, ctx_stream(ctx), dp, p, d, rows, (int)T, scale, dtype);
     EW_POSTCHECK("mg_tk_attn_softmax_bwd");
+}
+
+int mg_tk_attn_rowdot(mg_ctx *ctx, const void *a16, const float *b32, float *out, int64_t rows, int64_t D, int dtype) {
+    EW_PRECHECK("mg_tk_attn_rowdot", a16 && b32 && out && count_ok(rows) && D > 0 && D <= 0x7fffffff && dtype_ok(dtype));
+    hipLaunchKernelGGL(k_attn_rowdot, dim3(row_blocks(rows)), dim3(64 * ROWS_PER_WG), 0, ctx_stream(ctx),
+                       (const uint16_t *)a16, b32, out, rows, (int)D, dtype);
+    EW_POSTCHECK("mg_tk_attn_rowdot");
 }
 
 int mg_tk_split_qkv(mg_ctx *ctx, const float *qkv, const float *bias, void *q16, void *k16, void *v16, int64_t n,

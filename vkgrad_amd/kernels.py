@@ -100,7 +100,8 @@ class Matmul:
         return m > 0 and n > 0 and k > 0
 
     def _args(self, a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side=False,
-              act=None, y16=None, ldy=None, z=None, ldz=None, colsum=None, res=None, ldr=None, tri=None):
+              act=None, y16=None, ldy=None, z=None, ldz=None, colsum=None, res=None, ldr=None, tri=None,
+              p16=None, ldp=None, rowsub=None, scale=1.0):
         if self.batched:
             nb = int(nbatch)
             sa, sb, sc = (int(s) for s in strides)
@@ -139,9 +140,23 @@ class Matmul:
             ga.flags |= L.MG_FLAG_SIDE_STREAM
         if act not in L.ACTS:
             raise VkError(f"{self.name}: unknown activation {act!r}; use None, 'gelu', 'relu', "
-                          f"'gelu_grad' or 'relu_grad'")
+                          f"'gelu_grad', 'relu_grad' or 'softmax_grad'")
         ga.act = L.ACTS[act]
-        if ga.act >= L.MG_ACT_GELU_GRAD:
+        if ga.act == L.MG_ACT_SOFTMAX_GRAD:
+            if p16 is None or rowsub is None:
+                raise VkError(f"{self.name}: act='softmax_grad' needs p16= (the 16-bit softmax output) and rowsub=")
+            if z is not None or colsum is not None:
+                raise VkError(f"{self.name}: z= and colsum= belong to act='gelu_grad' or 'relu_grad'")
+            ga.p16, ga.rowsub, ga.scale = p16.ptr, rowsub.ptr, float(scale)
+            ga.ldp = int(ldp) if ldp is not None else n
+            if m > 0 and n > 0:
+                if p16.size < ((nb - 1) * sc + (m - 1) * ga.ldp + n) * 2:
+                    raise VkError(f"{self.name}: p16 buffer of {p16.size} bytes is too small for {nb} x {m}x{n}")
+                if rowsub.size < nb * m * 4:
+                    raise VkError(f"{self.name}: rowsub buffer of {rowsub.size} bytes is shorter than {nb * m} floats")
+        elif p16 is not None or rowsub is not None:
+            raise VkError(f"{self.name}: p16= and rowsub= belong to act='softmax_grad'")
+        elif ga.act >= L.MG_ACT_GELU_GRAD:
             if z is None:
                 raise VkError(f"{self.name}: act={act!r} needs z= (the pre-activation, f32)")
             ga.z = z.ptr
@@ -157,7 +172,7 @@ class Matmul:
         if y16 is not None:
             ga.y16 = y16.ptr
             ga.ldy = int(ldy) if ldy is not None else n
-            if m > 0 and n > 0 and y16.size < ((m - 1) * ga.ldy + n) * 2:
+            if m > 0 and n > 0 and y16.size < ((nb - 1) * sc + (m - 1) * ga.ldy + n) * 2:
                 raise VkError(f"{self.name}: y16 buffer of {y16.size} bytes is too small for {m}x{n} (pitch {ga.ldy})")
         elif ga.act:
             raise VkError(f"{self.name}: act= needs y16= (the activated 16-bit output)")
@@ -184,7 +199,8 @@ class Matmul:
 
     def __call__(self, a, b, c, m, n, k, repeat=1, graph=None, nbatch=1, strides=(0, 0, 0),
                  *, bias=None, accumulate=False, lda=None, ldb=None, ldc=None, side=False,
-                 act=None, y16=None, ldy=None, z=None, ldz=None, colsum=None, res=None, ldr=None, tri=None):
+                 act=None, y16=None, ldy=None, z=None, ldz=None, colsum=None, res=None, ldr=None, tri=None,
+                 p16=None, ldp=None, rowsub=None, scale=1.0):
         """side=True (recorded calls only) puts the GEMM on the device's side stream:
         it runs concurrently with the main stream between graph.fork() and graph.join().
         y16= (with act=None, 'gelu' or 'relu') makes the epilogue also write
@@ -196,6 +212,10 @@ class Matmul:
         accumulating) has the column sums of g added to it (col_sum, kernels.py:753-761).
         res= (an (m, n) f32 matrix) makes it C = res + result (+ bias): the `residual`
         pass of the reference's transformer (tkernels.py:362-371) in the epilogue.
+        act='softmax_grad' with p16= (the 16-bit softmax output P), rowsub= (one float per
+        row: sum_j P_j dP_j) and scale= folds attn_softmax_bwd (tkernels.py:167-187) into the
+        dP = dOut V^T GEMM: y16 = narrow(scale * P * (result - rowsub[row])); batches allowed
+        (y16 and p16 advance strides[2] elements per batch, rowsub m floats).
         tri= declares the causal structure of an attention GEMM so that work on masked
         entries is skipped: 'c_lower' (only C[i, j <= i] is needed; the rest of C is left
         as it was), 'a_lower' / 'a_upper' (op(A)[i, k] is zero for k > i / k < i)."""
@@ -203,7 +223,8 @@ class Matmul:
         if side and graph is None:
             raise VkError(f"{self.name}: side=True needs graph= (eager calls wait for their result); "
                           f"use enqueue(..., side=True) between dev.side_fork() and dev.side_join()")
-        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz, colsum, res, ldr, tri)
+        ga = self._args(a, b, c, m, n, k, nbatch, strides, bias, accumulate, lda, ldb, ldc, side, act, y16, ldy, z, ldz, colsum, res, ldr, tri,
+                        p16, ldp, rowsub, scale)
         if graph is not None:
             _check(lib.mg_gemm_check(C.byref(ga)), self.name)
             self._keep.append(ga)
@@ -211,7 +232,7 @@ class Matmul:
             def launch(ga=ga):
                 _check(lib.mg_gemm(ctx, C.byref(ga)), self.name)
 
-            graph.record(launch, [x for x in (a, b, c, y16, z, colsum, res) if x is not None], name=self.name,
+            graph.record(launch, [x for x in (a, b, c, y16, z, colsum, res, p16, rowsub) if x is not None], name=self.name,
                          bytes_hint=self.traffic_bytes(m, n, k, nbatch))
             nb_ = nbatch if self.batched else 1
             graph.mm_split.append((nb_ * 2 * (m * k + k * n), nb_ * m * n * 4))

@@ -17,7 +17,8 @@ flavours chosen by `TCtx(fuse=...)`:
               GELU / residual passes, GELU' as its own pass in backward;
   fuse=True   those passes ride in GEMM epilogues: QKV bias, proj and fc2
               bias + residual (`res=`), fc1 bias + GELU + 16-bit copy (`act=`,
-              `y16=`), GELU' inside fc2's dX GEMM (`act='gelu_grad'`, `z=`).
+              `y16=`), GELU' inside fc2's dX GEMM (`act='gelu_grad'`, `z=`), the
+              softmax backward inside attention's dP GEMM (`act='softmax_grad'`).
 
 Shapes are free (tiles mask their edges); only the vocabulary is padded, to a
 multiple of 64 so that rows of the logits stay 16-byte aligned.
@@ -151,7 +152,15 @@ class Attention:
         self.scores, self.p16 = _f32(ctx, nbh, T_, T_), _h16(ctx, nbh, T_, T_)
         self.ao32, self.ao16 = _f32(ctx, nbh, T_, hd), _h16(ctx, self.rows, D)
         self.dao16 = _h16(ctx, nbh, T_, hd)
-        self.dp32, self.ds16 = _f32(ctx, nbh, T_, T_), _h16(ctx, nbh, T_, T_)
+        if ctx.fuse:
+            # dS comes straight out of the dP GEMM (act='softmax_grad'): no f32 dP.  Tiles wholly
+            # above the diagonal are never written, and the dQ / dK GEMMs may read into them
+            # (their row blocks can be taller than the dP GEMM's tiles): they stay zero from here.
+            self.dp32 = None
+            self.ds16 = ctx.zeros(nbh * T_ * T_ // 2 + 1)
+            self.dsum = _f32(ctx, nbh, T_)
+        else:
+            self.dp32, self.ds16 = _f32(ctx, nbh, T_, T_), _h16(ctx, nbh, T_, T_)
         self.dq32, self.dk32, self.dv32 = (_f32(ctx, nbh, T_, hd) for _ in range(3))
         self.dqkv16 = _h16(ctx, self.rows, 3 * D)
         # per-head GEMMs as (M, N, K, trans_a, trans_b); a (T, hd) tensor advances `vec`
@@ -168,10 +177,11 @@ class Attention:
             "dK":     (T, self.hd, T, True, False, (sq, vec, vec), "a_upper"),    # dS^T Q
         }
 
-    def _heads(self, which, a, b, c, graph):
+    def _heads(self, which, a, b, c, graph, **epilogue):
         m, n, k, ta, tb, strides, tri = self._head_gemms[which]
         mm = self.ctx.matmul(m, n, k, trans_a=ta, trans_b=tb, batched=True, nbatch=self.nbh)
-        mm(a, b, c, m, n, k, graph=graph, nbatch=self.nbh, strides=strides, tri=tri if self.ctx.causal_gemms else None)
+        mm(a, b, c, m, n, k, graph=graph, nbatch=self.nbh, strides=strides,
+           tri=tri if self.ctx.causal_gemms else None, **epilogue)
 
     def _permute(self, name, buffers, graph):
         self.ctx.TK[name](buffers, self.rows * self.D, self.D, self.T, self.H, self.hd, graph=graph)
@@ -200,9 +210,16 @@ class Attention:
         dao32 = self.proj.backward(dy16, need_dx=True, graph=graph)
         self._permute("split_heads", [dao32, self.dao16], graph)
         self._heads("dV", self.p16, self.dao16, self.dv32, graph)
-        self._heads("dP", self.dao16, self.v16, self.dp32, graph)
-        ctx.rowwise("attn_softmax_bwd", [self.dp32, self.p16, self.ds16], self.nbh * self.T, self.T, self.scale,
-                    graph=graph)
+        if ctx.fuse:
+            # sum_j P_j dP_j = sum_d dOut_d Out_d (dP = dOut V^T, Out = P V), so the row term of the
+            # softmax backward is known before dP, and dS leaves the dP GEMM's epilogue directly
+            ctx.rowwise("attn_rowdot", [self.dao16, self.ao32, self.dsum], self.nbh * self.T, self.hd, graph=graph)
+            self._heads("dP", self.dao16, self.v16, None, graph, act="softmax_grad", y16=self.ds16,
+                        p16=self.p16, rowsub=self.dsum, scale=self.scale)
+        else:
+            self._heads("dP", self.dao16, self.v16, self.dp32, graph)
+            ctx.rowwise("attn_softmax_bwd", [self.dp32, self.p16, self.ds16], self.nbh * self.T, self.T, self.scale,
+                        graph=graph)
         self._heads("dQ", self.ds16, self.k16, self.dq32, graph)
         self._heads("dK", self.ds16, self.q16, self.dk32, graph)
         self._permute("merge_qkv_grad", [self.dq32, self.dk32, self.dv32, self.dqkv16], graph)
