@@ -334,6 +334,17 @@ int mg_tk_attn_softmax_bwd(mg_ctx *ctx, const float *dp, const void *p16, void *
  * b32 = Out (head-side) this is the row term sum_j P_j dP_j of attn_softmax_bwd
  * (tkernels.py:167-187), formed without P or dP: the `rowsub` of MG_ACT_SOFTMAX_GRAD. */
 int mg_tk_attn_rowdot(mg_ctx *ctx, const void *a16, const float *b32, float *out, int64_t rows, int64_t D, int dtype);
+/* dS of attention in one kernel: the dP = dOut V^T product over the heads (transformer.py:171-173)
+ * and attn_softmax_bwd (tkernels.py:167-187) after it, without the f32 dP in between:
+ *   ds16[b][i][j] = narrow(scale * p16[b][i][j] * (sum_d dout16[b][i][d] * v16[b][j][d] - rowsub[b][i]))
+ * for nbh heads of T x T, head width hd in {32, 64, 128} and T a multiple of 8 (mg_tk_attn_ds_supported; other
+ * sizes take mg_gemm with MG_ACT_SOFTMAX_GRAD).  dout16 and v16 are (nbh, T, hd), 16-byte aligned,
+ * as are p16 and ds16; rowsub
+ * from mg_tk_attn_rowdot.  causal != 0: blocks of 32 queries x 256 keys wholly beyond the diagonal
+ * are neither computed nor written - keep ds16 zero there. */
+int mg_tk_attn_ds_supported(int64_t hd, int64_t T);
+int mg_tk_attn_ds(mg_ctx *ctx, const void *dout16, const void *v16, const void *p16, const float *rowsub, void *ds16,
+                  int64_t nbh, int64_t T, int64_t hd, float scale, int causal, int dtype);
 /* split_qkv (tkernels.py:195-213): (B*T, 3D) f32 + bias[3D] (or NULL) -> q16, k16, v16 head-side */
 int mg_tk_split_qkv(mg_ctx *ctx, const float *qkv, const float *bias, void *q16, void *k16, void *v16, int64_t n,
                     int64_t D, int64_t T, int64_t H, int64_t hd, int dtype);

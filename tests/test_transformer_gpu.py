@@ -117,7 +117,7 @@ def test_softmax_backward_in_the_dp_gemm(dev, tk):
     dtype, TK = tk
     W = dev.row_subgroup_size
     rng = np.random.default_rng(11)
-    for nbh, T, hd in ((3, 200, 40), (2, 64, 64), (1, 1024, 64), (2, 330, 24)):
+    for nbh, T, hd in ((3, 200, 40), (2, 64, 64), (1, 1024, 64), (2, 330, 24), (2, 80, 32), (1, 200, 128), (3, 129, 64), (3, 136, 64), (2, 520, 64), (2, 64, 20)):
         rows = nbh * T
         scale = 1.0 / np.sqrt(hd)
         s = (rng.standard_normal((rows, T)) * 2).astype(np.float32)
@@ -144,6 +144,15 @@ def test_softmax_backward_in_the_dp_gemm(dev, tk):
                        act="softmax_grad", y16=bds, p16=bp, rowsub=bsum, scale=scale)
                     got = stored(bds, dtype, (rows, T))
                     assert close16(got, want, dtype, slack=5e-5), (nbh, T, hd, tile, tri)
+            # the one-kernel form for common head widths (same formula, operands straight from memory)
+            if dev._lib.mg_tk_attn_ds_supported(hd, T):
+                for causal in (False, True):
+                    bds.upload(np.zeros(rows * T, np.uint16))
+                    TK["attn_ds"]([bdo, bv, bp, bsum, bds], nbh, T, hd, scale, causal)
+                    assert close16(stored(bds, dtype, (rows, T)), want, dtype, slack=5e-5), (nbh, T, hd, causal)
+            else:
+                with pytest.raises(Exception):
+                    TK["attn_ds"]([bdo, bv, bp, bsum, bds], nbh, T, hd, scale, False)
             # the f32 copy of the same values, one head
             mm = Matmul(dev, trans_b=True, dtype=dtype)
             mm(bdo, bv, bc, T, T, hd, act="softmax_grad", y16=bds, p16=bp, rowsub=bsum, scale=scale)

@@ -1,0 +1,165 @@
+// Attention's dS in one kernel: the dP = dOut V^T product of every head (reference call site
+// transformer.py:171-173) and the softmax backward that follows it (attn_softmax_bwd,
+// tkernels.py:167-187), without the f32 dP matrix in between:
+//
+//   dS[b][i][j] = narrow(scale * P[b][i][j] * (sum_d dOut[b][i][d] V[b][j][d] - rowsub[b][i]))
+//
+// rowsub[i] = sum_j P[i][j] dP[i][j], which the caller forms as sum_d dOut[i][d] Out[i][d]
+// (mg_tk_attn_rowdot).  The contraction is only as long as a head is wide (64 for GPT-2), so a
+// tiled GEMM has one K-block per tile and spends its time waiting: for the operands, and in
+// an epilogue version of this formula once more for P.  Here nothing passes through LDS and
+// nothing waits twice: the MFMA operands are 16-byte loads straight from dOut and V (a lane
+// of v_mfma_f32_32x32x16 holds 8 consecutive k of one row, which is how both tensors lie in
+// memory), and P and rowsub are requested in the same burst, before the first MFMA.
+//
+// What bounds such a kernel on this chip is the number of vector memory instructions, not their
+// bytes: a 4-byte and a 16-byte access per lane cost a wavefront about the same.  So a
+// wavefront owns 32 queries x 256 keys, eight accumulator blocks that share the dOut fragments,
+// and since the key an accumulator column stands for is decided by the row of V its lane
+// loaded, block t takes the keys 8n + t (n = lane % 32): a lane then holds eight neighbouring
+// keys of each of its rows, and P arrives and dS leaves as one 16-byte access per lane and row
+// (T must be a multiple of 8 for their alignment).  rowsub is one load per wavefront, handed
+// round by lane reads.  Four wavefronts (128 queries) share a workgroup.
+//
+// With `causal` set, a wavefront whose keys all lie beyond its queries neither computes nor
+// writes (P is zero there, and so is dS: the caller keeps the buffer zeroed); inside computed
+// blocks the masked entries come out as zero because P is.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mi_gemm.h"
+
+#include "ew_common.h"
+
+namespace mg {
+
+typedef _Float16 ak_half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 ak_bf8 __attribute__((ext_vector_type(8)));
+typedef float ak_f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t ak_u32x4 __attribute__((ext_vector_type(4)));
+
+template <int DT>
+__device__ __forceinline__ ak_f32x16 ak_mfma(ak_u32x4 a, ak_u32x4 b, ak_f32x16 c) {
+    if constexpr (DT == MG_F16)
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(ak_half8, a), __builtin_bit_cast(ak_half8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(ak_bf8, a), __builtin_bit_cast(ak_bf8, b), c, 0, 0, 0);
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t ak_narrow(float x) {
+    if constexpr (DT == MG_F16) return __builtin_bit_cast(uint16_t, (_Float16)x);
+    else return __builtin_bit_cast(uint16_t, (__bf16)x);   // round to nearest even, one instruction on gfx950
+}
+template <int DT>
+__device__ __forceinline__ float ak_widen(uint32_t b) {
+    if constexpr (DT == MG_F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
+    else return __builtin_bit_cast(float, b << 16);
+}
+
+constexpr int DS_BM = 128, DS_BN = 256;   // workgroup tile: 4 wavefronts of 32 queries x 256 keys
+
+template <int DT, int HD>
+__global__ void __launch_bounds__(256, 2)
+k_attn_ds(const uint16_t *dout, const uint16_t *v, const uint16_t *p16, const float *rowsub, uint16_t *ds16, int T,
+          float scale, int causal) {
+    constexpr int KK = HD / 16, NB = DS_BN / 32;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t b = blockIdx.z;
+    const int i0 = blockIdx.y * DS_BM + wave * 32;   // this wavefront's first query
+    const int j0 = blockIdx.x * DS_BN;               // and first key
+    if (i0 >= T) return;
+    if (causal && j0 > i0 + 31) return;              // every key beyond every query
+    const uint16_t *db = dout + b * (int64_t)T * HD;
+    const uint16_t *vb = v + b * (int64_t)T * HD;
+
+    // MFMA operands: lane l holds row l % 32, k = 8 * (l / 32) .. + 7 of each 16-wide k step
+    const int fr = lane & 31, fk = (lane >> 5) * 8;
+    const uint16_t *ap = db + (int64_t)min(i0 + fr, T - 1) * HD + fk;
+    ak_u32x4 af[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) af[kk] = *reinterpret_cast<const ak_u32x4 *>(ap + kk * 16);
+    // Accumulator register r belongs to row i0 + ro + 4 * (l / 32), ro = 8 * (r / 4) + r % 4; this
+    // lane's keys are jc .. jc + 7, one per block.  T is a multiple of 8: all eight exist or none.
+    const int rl = i0 + (lane >> 5) * 4;
+    const int jc = j0 + 8 * fr;
+    const bool col_ok = jc < T;
+    const int64_t cell = b * (int64_t)T * T + (col_ok ? jc : 0);
+    const bool whole = i0 + 32 <= T;                 // no row of this wavefront beyond the matrix
+    const float rs_lane = rowsub[b * (int64_t)T + min(i0 + fr, T - 1)] * scale;
+    ak_u32x4 pp[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int ro = (r >> 2) * 8 + (r & 3);
+        const int row = whole ? rl + ro : min(rl + ro, T - 1);
+        pp[r] = *reinterpret_cast<const ak_u32x4 *>(p16 + cell + (int64_t)row * T);
+    }
+    ak_f32x16 acc[NB];
+#pragma unroll
+    for (int t = 0; t < NB; t++) {
+        const uint16_t *bp = vb + (int64_t)min(j0 + 8 * fr + t, T - 1) * HD + fk;
+        ak_u32x4 bf[KK];
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) bf[kk] = *reinterpret_cast<const ak_u32x4 *>(bp + kk * 16);
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) acc[t] = ak_mfma<DT>(af[kk], bf[kk], acc[t]);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int ro = (r >> 2) * 8 + (r & 3);
+        // rowsub of this lane's row: lanes 0-31 hold the 32 rows of the wavefront
+        const float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, rs_lane), ro));
+        const float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, rs_lane), ro + 4));
+        const float rs = lane < 32 ? lo : hi;
+        ak_u32x4 o;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float p0 = ak_widen<DT>(pp[r][w] & 0xffffu), p1 = ak_widen<DT>(pp[r][w] >> 16);
+            o[w] = ak_narrow<DT>(p0 * (acc[2 * w][r] * scale - rs)) | (ak_narrow<DT>(p1 * (acc[2 * w + 1][r] * scale - rs)) << 16);
+        }
+        if (col_ok && (whole || rl + ro < T))
+            *reinterpret_cast<ak_u32x4 *>(ds16 + cell + (int64_t)(rl + ro) * T) = o;
+    }
+}
+
+template <int DT, int HD>
+static void launch_attn_ds(hipStream_t s, const void *dout, const void *v, const void *p16, const float *rowsub, void *ds16,
+                           int64_t nbh, int T, float scale, int causal) {
+    const dim3 grid((unsigned)((T + DS_BN - 1) / DS_BN), (unsigned)((T + DS_BM - 1) / DS_BM), (unsigned)nbh);
+    hipLaunchKernelGGL((k_attn_ds<DT, HD>), grid, dim3(256), 0, s, (const uint16_t *)dout, (const uint16_t *)v,
+                       (const uint16_t *)p16, rowsub, (uint16_t *)ds16, T, scale, causal);
+}
+
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" {
+
+int mg_tk_attn_ds_supported(int64_t hd, int64_t T) { return (hd == 32 || hd == 64 || hd == 128) && T > 0 && T % 8 == 0; }
+
+int mg_tk_attn_ds(mg_ctx *ctx, const void *dout16, const void *v16, const void *p16, const float *rowsub, void *ds16,
+                  int64_t nbh, int64_t T, int64_t hd, float scale, int causal, int dtype) {
+    EW_PRECHECK("mg_tk_attn_ds", dout16 && v16 && p16 && rowsub && ds16 && nbh > 0 && nbh <= 65535 && T > 0 &&
+                                     T <= 0x7fffffff / 2 && mg_tk_attn_ds_supported(hd, T) && dtype_ok(dtype) &&
+                                     (T + DS_BM - 1) / DS_BM <= 65535 && scale == scale &&
+                                     (((uintptr_t)dout16 | (uintptr_t)v16) & 15) == 0 &&
+                                     (((uintptr_t)p16 | (uintptr_t)ds16) & 15) == 0 && ((uintptr_t)rowsub & 3) == 0);
+    hipStream_t s = ctx_stream(ctx);
+    const int t = (int)T, c = causal ? 1 : 0;
+    if (dtype == MG_F16) {
+        if (hd == 32) launch_attn_ds<MG_F16, 32>(s, dout16, v16, p16, rowsub, ds16, nbh, t, scale, c);
+        else if (hd == 64) launch_attn_ds<MG_F16, 64>(s, dout16, v16, p16, rowsub, ds16, nbh, t, scale, c);
+        else launch_attn_ds<MG_F16, 128>(s, dout16, v16, p16, rowsub, ds16, nbh, t, scale, c);
+    } else {
+        if (hd == 32) launch_attn_ds<MG_BF16, 32>(s, dout16, v16, p16, rowsub, ds16, nbh, t, scale, c);
+        else if (hd == 64) launch_attn_ds<MG_BF16, 64>(s, dout16, v16, p16, rowsub, ds16, nbh, t, scale, c);
+        else launch_attn_ds<MG_BF16, 128>(s, dout16, v16, p16, rowsub, ds16, nbh, t, scale, c);
+    }
+    EW_POSTCHECK("mg_tk_attn_ds");
+}
+
+}  // extern "C"

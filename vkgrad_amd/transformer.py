@@ -214,8 +214,13 @@ class Attention:
             # sum_j P_j dP_j = sum_d dOut_d Out_d (dP = dOut V^T, Out = P V), so the row term of the
             # softmax backward is known before dP, and dS leaves the dP GEMM's epilogue directly
             ctx.rowwise("attn_rowdot", [self.dao16, self.ao32, self.dsum], self.nbh * self.T, self.hd, graph=graph)
-            self._heads("dP", self.dao16, self.v16, None, graph, act="softmax_grad", y16=self.ds16,
-                        p16=self.p16, rowsub=self.dsum, scale=self.scale)
+            if ctx.dev._lib.mg_tk_attn_ds_supported(self.hd, self.T):
+                # common head widths: product, P and the row term meet in one kernel without LDS
+                ctx.TK["attn_ds"]([self.dao16, self.v16, self.p16, self.dsum, self.ds16], self.nbh, self.T, self.hd,
+                                  self.scale, ctx.causal_gemms, graph=graph)
+            else:
+                self._heads("dP", self.dao16, self.v16, None, graph, act="softmax_grad", y16=self.ds16,
+                            p16=self.p16, rowsub=self.dsum, scale=self.scale)
         else:
             self._heads("dP", self.dao16, self.v16, self.dp32, graph)
             ctx.rowwise("attn_softmax_bwd", [self.dp32, self.p16, self.ds16], self.nbh * self.T, self.T, self.scale,
