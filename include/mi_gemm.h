@@ -334,6 +334,17 @@ int mg_tk_attn_softmax_bwd(mg_ctx *ctx, const float *dp, const void *p16, void *
  * b32 = Out (head-side) this is the row term sum_j P_j dP_j of attn_softmax_bwd
  * (tkernels.py:167-187), formed without P or dP: the `rowsub` of MG_ACT_SOFTMAX_GRAD. */
 int mg_tk_attn_rowdot(mg_ctx *ctx, const void *a16, const float *b32, float *out, int64_t rows, int64_t D, int dtype);
+/* P of attention in one kernel: the scores = Q K^T product over the heads (transformer.py:153-155)
+ * and attn_softmax / attn_softmax_doc (tkernels.py:105-165) after it, without the f32 scores in
+ * between: p16[b][i][j] = softmax over the seen keys j of scale * sum_d q16[b][i][d] * k16[b][j][d],
+ * 0 for the others.  Query i of head b sees keys first .. i, first = 0 (seg NULL) or
+ * seg[(b / H) * T + i].  nbh heads (a multiple of H) of T x T, head width hd in {32, 64, 128}, T a
+ * multiple of 8 and at most 1024 (mg_tk_attn_p_supported; other sizes take the GEMM and
+ * mg_tk_attn_softmax).  All three tensors 16-byte aligned.  causal != 0: blocks of 32 queries x
+ * 256 keys wholly beyond the diagonal are not written - keep p16 zero there. */
+int mg_tk_attn_p_supported(int64_t hd, int64_t T);
+int mg_tk_attn_p(mg_ctx *ctx, const void *q16, const void *k16, const uint32_t *seg, void *p16, int64_t nbh, int64_t T,
+                 int64_t H, int64_t hd, float scale, int causal, int dtype);
 /* dS of attention in one kernel: the dP = dOut V^T product over the heads (transformer.py:171-173)
  * and attn_softmax_bwd (tkernels.py:167-187) after it, without the f32 dP in between:
  *   ds16[b][i][j] = narrow(scale * p16[b][i][j] * (sum_d dout16[b][i][d] * v16[b][j][d] - rowsub[b][i]))

@@ -165,6 +165,41 @@ def test_softmax_backward_in_the_dp_gemm(dev, tk):
                 t.destroy()
 
 
+def test_scores_and_softmax_in_one_kernel(dev, tk):
+    """attn_p: P straight from Q and K (no f32 scores), against the oracle's softmax of the
+    numpy scores; plain causal and packed samples (seg), with and without the causal skipping."""
+    dtype, TK = tk
+    rng = np.random.default_rng(12)
+    for B, H, T, hd in ((1, 2, 64, 64), (2, 3, 200, 32), (1, 1, 1024, 64), (1, 2, 520, 128), (2, 1, 136, 64)):
+        nbh, rows = B * H, B * H * T
+        scale = 1.0 / np.sqrt(hd)
+        assert dev._lib.mg_tk_attn_p_supported(hd, T)
+        q16 = O.round_to((rng.standard_normal((nbh, T, hd)) * 1.5).astype(np.float32), dtype)
+        k16 = O.round_to((rng.standard_normal((nbh, T, hd)) * 1.5).astype(np.float32), dtype)
+        sc = np.einsum("bid,bjd->bij", O.widen(q16, dtype), O.widen(k16, dtype)).astype(np.float32).reshape(rows, T)
+        seg = np.zeros(B * T, np.uint32)
+        for b in range(B):
+            cut = 1 + (7 * b + T // 3) % (T - 1)
+            seg[b * T + cut:(b + 1) * T] = cut
+        bq, bk, bseg = up(dev, q16), up(dev, k16), up(dev, seg)
+        bp = dev.buffer(rows * T * 2, "device")
+        try:
+            for use_seg in (False, True):
+                want = RT.attn_softmax(sc, T, scale, dtype, seg=seg if use_seg else None, H=H)
+                for causal in (False, True):
+                    bp.upload(np.zeros(rows * T, np.uint16))
+                    TK["attn_p"]([bq, bk, bseg if use_seg else None, bp], nbh, T, H, hd, scale, causal)
+                    got = stored(bp, dtype, (rows, T))
+                    assert close16(got, want, dtype, slack=2e-5), (B, H, T, hd, use_seg, causal)
+                    tri = np.arange(T)[None, :] <= (np.arange(rows) % T)[:, None]
+                    assert not O.widen(got, dtype)[~tri].any()
+        finally:
+            for t in (bq, bk, bseg, bp):
+                t.destroy()
+    assert not dev._lib.mg_tk_attn_p_supported(64, 2048) and not dev._lib.mg_tk_attn_p_supported(40, 64)
+    assert not dev._lib.mg_tk_attn_p_supported(64, 100)
+
+
 def test_head_permutes(dev, tk):
     dtype, TK = tk
     rng = np.random.default_rng(2)

@@ -125,6 +125,121 @@ k_attn_ds(const uint16_t *dout, const uint16_t *v, const uint16_t *p16, const fl
     }
 }
 
+// P of attention in one kernel: the scores = Q K^T product of every head (reference call site
+// transformer.py:153-155) and the masked softmax over them (attn_softmax / attn_softmax_doc,
+// tkernels.py:105-165), without the f32 score matrix in between.  Same wavefront shape and key
+// interleaving as k_attn_ds above; the four wavefronts of a workgroup split the keys of the same
+// 32 queries between them (256 each, so T <= 1024), every wavefront reduces its part of a row
+// to a maximum and a sum of exponentials relative to it, the parts meet once in LDS, and each
+// wavefront rescales and writes its own 256 keys.  Row r (query q = r % T of its head) sees keys
+// first .. q, first = 0 or seg[batch * T + q]; masked keys get 0.  With `causal` set, a
+// wavefront whose keys all lie beyond its queries writes nothing: the caller keeps P zero there.
+template <int DT, int HD>
+__global__ void __launch_bounds__(256, 2)
+k_attn_p(const uint16_t *q16, const uint16_t *k16, const uint32_t *seg, uint16_t *p16, int T, int H, float scale,
+         int causal) {
+    constexpr int KK = HD / 16, NB = 8;
+    __shared__ float part_m[4][32], part_l[4][32];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t b = blockIdx.y;
+    const int i0 = blockIdx.x * 32;      // the workgroup's first query
+    const int j0 = wave * 256;           // this wavefront's first key
+    const int fr = lane & 31, fk = (lane >> 5) * 8, half = lane >> 5;
+    // keys that no query of this block may see: none of them, or (causal) all beyond the last query
+    const bool idle = j0 >= T || (causal && j0 > i0 + 31);
+    const int rl = i0 + half * 4;        // accumulator register r: row rl + ro, ro = 8 * (r / 4) + r % 4
+    const int jc = j0 + 8 * fr;          // this lane's keys: jc + t, one per block t
+    ak_f32x16 acc[NB];
+    float mloc[16], lloc[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        mloc[r] = -1e30f;
+        lloc[r] = 0.f;
+    }
+    if (!idle) {
+        const uint16_t *qb = q16 + b * (int64_t)T * HD + (int64_t)min(i0 + fr, T - 1) * HD + fk;
+        const uint16_t *kb = k16 + b * (int64_t)T * HD;
+        ak_u32x4 af[KK];
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) af[kk] = *reinterpret_cast<const ak_u32x4 *>(qb + kk * 16);
+#pragma unroll
+        for (int t = 0; t < NB; t++) {
+            const uint16_t *bp = kb + (int64_t)min(jc + t, T - 1) * HD + fk;
+            ak_u32x4 bf[KK];
+#pragma unroll
+            for (int kk = 0; kk < KK; kk++) bf[kk] = *reinterpret_cast<const ak_u32x4 *>(bp + kk * 16);
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < KK; kk++) acc[t] = ak_mfma<DT>(af[kk], bf[kk], acc[t]);
+        }
+        // per row: this lane's 8 keys, then the 32 lanes of the half-wave (they hold the same rows)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int ro = (r >> 2) * 8 + (r & 3);
+            const int q = rl + ro;
+            const int first = seg ? (int)seg[(b / H) * T + min(q, T - 1)] : 0;
+            float m = -1e30f;
+#pragma unroll
+            for (int t = 0; t < NB; t++) {
+                const int j = jc + t;
+                const bool seen = j >= first && j <= q && j < T;
+                acc[t][r] = seen ? acc[t][r] * scale : -1e30f;
+                m = fmaxf(m, acc[t][r]);
+            }
+#pragma unroll
+            for (int x = 16; x >= 1; x >>= 1) m = fmaxf(m, __shfl_xor(m, x, 64));
+            float l = 0.f;
+#pragma unroll
+            for (int t = 0; t < NB; t++) {
+                const float e = acc[t][r] > -1e29f ? __expf(acc[t][r] - m) : 0.f;
+                acc[t][r] = e;
+                l += e;
+            }
+#pragma unroll
+            for (int x = 16; x >= 1; x >>= 1) l += __shfl_xor(l, x, 64);
+            mloc[r] = m;
+            lloc[r] = l;
+        }
+    }
+    if (fr == 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int ro = (r >> 2) * 8 + (r & 3);
+            part_m[wave][ro + half * 4] = mloc[r];
+            part_l[wave][ro + half * 4] = lloc[r];
+        }
+    }
+    __syncthreads();
+    if (idle) return;
+    const bool col_ok = jc < T;          // T is a multiple of 8: all eight keys exist or none
+    uint16_t *pb = p16 + b * (int64_t)T * T + (col_ok ? jc : 0);
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int ro = (r >> 2) * 8 + (r & 3);
+        const int rw = ro + half * 4;
+        const float m0 = part_m[0][rw], m1 = part_m[1][rw], m2 = part_m[2][rw], m3 = part_m[3][rw];
+        const float mx = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
+        const float sum = part_l[0][rw] * __expf(m0 - mx) + part_l[1][rw] * __expf(m1 - mx) +
+                          part_l[2][rw] * __expf(m2 - mx) + part_l[3][rw] * __expf(m3 - mx);
+        const float f = __expf(mloc[r] - mx) / sum;   // (a row no key of which is seen does not occur: key q always is)
+        ak_u32x4 o;
+#pragma unroll
+        for (int w = 0; w < 4; w++)
+            o[w] = ak_narrow<DT>(acc[2 * w][r] * f) | (ak_narrow<DT>(acc[2 * w + 1][r] * f) << 16);
+        if (col_ok && rl + ro < T) *reinterpret_cast<ak_u32x4 *>(pb + (int64_t)(rl + ro) * T) = o;
+    }
+}
+
+template <int DT, int HD>
+static void launch_attn_p(hipStream_t s, const void *q, const void *k, const uint32_t *seg, void *p16, int64_t nbh, int T,
+                          int H, float scale, int causal) {
+    const dim3 grid((unsigned)((T + 31) / 32), (unsigned)nbh);
+    hipLaunchKernelGGL((k_attn_p<DT, HD>), grid, dim3(256), 0, s, (const uint16_t *)q, (const uint16_t *)k, seg,
+                       (uint16_t *)p16, T, H, scale, causal);
+}
+
 template <int DT, int HD>
 static void launch_attn_ds(hipStream_t s, const void *dout, const void *v, const void *p16, const float *rowsub, void *ds16,
                            int64_t nbh, int T, float scale, int causal) {
@@ -140,6 +255,28 @@ using namespace mg;
 extern "C" {
 
 int mg_tk_attn_ds_supported(int64_t hd, int64_t T) { return (hd == 32 || hd == 64 || hd == 128) && T > 0 && T % 8 == 0; }
+
+int mg_tk_attn_p_supported(int64_t hd, int64_t T) { return mg_tk_attn_ds_supported(hd, T) && T <= 1024; }
+
+int mg_tk_attn_p(mg_ctx *ctx, const void *q16, const void *k16, const uint32_t *seg, void *p16, int64_t nbh, int64_t T,
+                 int64_t H, int64_t hd, float scale, int causal, int dtype) {
+    EW_PRECHECK("mg_tk_attn_p", q16 && k16 && p16 && nbh > 0 && nbh <= 65535 && mg_tk_attn_p_supported(hd, T) &&
+                                    H > 0 && nbh % H == 0 && dtype_ok(dtype) && scale == scale &&
+                                    (((uintptr_t)q16 | (uintptr_t)k16 | (uintptr_t)p16) & 15) == 0 &&
+                                    ((uintptr_t)seg & 3) == 0);
+    hipStream_t s = ctx_stream(ctx);
+    const int t = (int)T, c = causal ? 1 : 0, h = (int)H;
+    if (dtype == MG_F16) {
+        if (hd == 32) launch_attn_p<MG_F16, 32>(s, q16, k16, seg, p16, nbh, t, h, scale, c);
+        else if (hd == 64) launch_attn_p<MG_F16, 64>(s, q16, k16, seg, p16, nbh, t, h, scale, c);
+        else launch_attn_p<MG_F16, 128>(s, q16, k16, seg, p16, nbh, t, h, scale, c);
+    } else {
+        if (hd == 32) launch_attn_p<MG_BF16, 32>(s, q16, k16, seg, p16, nbh, t, h, scale, c);
+        else if (hd == 64) launch_attn_p<MG_BF16, 64>(s, q16, k16, seg, p16, nbh, t, h, scale, c);
+        else launch_attn_p<MG_BF16, 128>(s, q16, k16, seg, p16, nbh, t, h, scale, c);
+    }
+    EW_POSTCHECK("mg_tk_attn_p");
+}
 
 int mg_tk_attn_ds(mg_ctx *ctx, const void *dout16, const void *v16, const void *p16, const float *rowsub, void *ds16,
                   int64_t nbh, int64_t T, int64_t hd, float scale, int causal, int dtype) {

@@ -75,6 +75,9 @@ def make_transformer_kernels(dev, dtype="f16"):
     # buffers: a16, b32, out ; n = rows * W ; args: D  (out[r] = sum_d a16[r][d] * b32[r][d])
     add("attn_rowdot", lambda lib, ctx, p, n, D:
         lib.mg_tk_attn_rowdot(ctx, p[0], p[1], p[2], rows_of(n), int(D), dt))
+    # buffers: q16, k16, seg (or None), p16 ; n = heads ; args: T, H, hd, scale, causal
+    add("attn_p", lambda lib, ctx, p, n, T, H, hd, scale, causal:
+        lib.mg_tk_attn_p(ctx, p[0], p[1], p[2], p[3], int(n), int(T), int(H), int(hd), float(scale), int(bool(causal)), dt))
     # buffers: dout16, v16, p16, rowsub, ds16 ; n = heads ; args: T, hd, scale, causal
     add("attn_ds", lambda lib, ctx, p, n, T, hd, scale, causal:
         lib.mg_tk_attn_ds(ctx, p[0], p[1], p[2], p[3], p[4], int(n), int(T), int(hd), float(scale), int(bool(causal)), dt))

@@ -149,7 +149,16 @@ class Attention:
         self.proj = Dense(ctx, self.rows, D, D, name + ".proj", scale=np.sqrt(2.0 / D) * 0.5)
         nbh, T_, hd = self.nbh, T, self.hd
         self.q16, self.k16, self.v16 = (_h16(ctx, nbh, T_, hd) for _ in range(3))
-        self.scores, self.p16 = _f32(ctx, nbh, T_, T_), _h16(ctx, nbh, T_, T_)
+        lib = ctx.dev._lib
+        self._one_kernel_p = bool(ctx.fuse and lib.mg_tk_attn_p_supported(self.hd, T))
+        self._one_kernel_ds = bool(ctx.fuse and lib.mg_tk_attn_ds_supported(self.hd, T))
+        if self._one_kernel_p:
+            # P comes out of one kernel (scores + softmax): no f32 scores.  Wavefronts whose keys all
+            # lie beyond their queries write nothing, so P is cleared once, here.
+            self.scores = None
+            self.p16 = ctx.zeros(nbh * T_ * T_ // 2 + 1)
+        else:
+            self.scores, self.p16 = _f32(ctx, nbh, T_, T_), _h16(ctx, nbh, T_, T_)
         self.ao32, self.ao16 = _f32(ctx, nbh, T_, hd), _h16(ctx, self.rows, D)
         self.dao16 = _h16(ctx, nbh, T_, hd)
         if ctx.fuse:
@@ -193,12 +202,16 @@ class Attention:
         fused = ctx.fuse
         qkv = self.qkv.forward(x16, graph=graph, bias=fused)
         self._permute("split_qkv", [qkv, None if fused else self.qkv.b.w32, self.q16, self.k16, self.v16], graph)
-        self._heads("scores", self.q16, self.k16, self.scores, graph)
-        if seg is None:
-            ctx.rowwise("attn_softmax", [self.scores, self.p16], self.nbh * self.T, self.T, self.scale, graph=graph)
+        if self._one_kernel_p:
+            ctx.TK["attn_p"]([self.q16, self.k16, seg, self.p16], self.nbh, self.T, self.H, self.hd, self.scale,
+                             ctx.causal_gemms, graph=graph)
         else:
-            ctx.rowwise("attn_softmax_doc", [self.scores, seg, self.p16], self.nbh * self.T, self.T, self.H,
-                        self.scale, graph=graph)
+            self._heads("scores", self.q16, self.k16, self.scores, graph)
+            if seg is None:
+                ctx.rowwise("attn_softmax", [self.scores, self.p16], self.nbh * self.T, self.T, self.scale, graph=graph)
+            else:
+                ctx.rowwise("attn_softmax_doc", [self.scores, seg, self.p16], self.nbh * self.T, self.T, self.H,
+                            self.scale, graph=graph)
         self._heads("mix", self.p16, self.v16, self.ao32, graph)
         self._permute("merge_heads", [self.ao32, self.ao16], graph)
         if fused and res is not None:
@@ -214,7 +227,7 @@ class Attention:
             # sum_j P_j dP_j = sum_d dOut_d Out_d (dP = dOut V^T, Out = P V), so the row term of the
             # softmax backward is known before dP, and dS leaves the dP GEMM's epilogue directly
             ctx.rowwise("attn_rowdot", [self.dao16, self.ao32, self.dsum], self.nbh * self.T, self.hd, graph=graph)
-            if ctx.dev._lib.mg_tk_attn_ds_supported(self.hd, self.T):
+            if self._one_kernel_ds:
                 # common head widths: product, P and the row term meet in one kernel without LDS
                 ctx.TK["attn_ds"]([self.dao16, self.v16, self.p16, self.dsum, self.ds16], self.nbh, self.T, self.hd,
                                   self.scale, ctx.causal_gemms, graph=graph)
