@@ -339,8 +339,8 @@ int mg_tk_attn_rowdot(mg_ctx *ctx, const void *a16, const float *b32, float *out
  * between: p16[b][i][j] = softmax over the seen keys j of scale * sum_d q16[b][i][d] * k16[b][j][d],
  * 0 for the others.  Query i of head b sees keys first .. i, first = 0 (seg NULL) or
  * seg[(b / H) * T + i].  nbh heads (a multiple of H) of T x T, head width hd in {32, 64, 128}, T a
- * multiple of 8 and at most 1024 (mg_tk_attn_p_supported; other sizes take the GEMM and
- * mg_tk_attn_softmax).  All three tensors 16-byte aligned.  causal != 0: blocks of 32 queries x
+ * multiple of 8, and at most 1024 for hd = 128 (mg_tk_attn_p_supported; other sizes take the GEMM
+ * and mg_tk_attn_softmax).  All three tensors 16-byte aligned.  causal != 0: blocks of 32 queries x
  * 256 keys wholly beyond the diagonal are not written - keep p16 zero there. */
 int mg_tk_attn_p_supported(int64_t hd, int64_t T);
 int mg_tk_attn_p(mg_ctx *ctx, const void *q16, const void *k16, const uint32_t *seg, void *p16, int64_t nbh, int64_t T,

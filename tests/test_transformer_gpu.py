@@ -170,7 +170,8 @@ def test_scores_and_softmax_in_one_kernel(dev, tk):
     numpy scores; plain causal and packed samples (seg), with and without the causal skipping."""
     dtype, TK = tk
     rng = np.random.default_rng(12)
-    for B, H, T, hd in ((1, 2, 64, 64), (2, 3, 200, 32), (1, 1, 1024, 64), (1, 2, 520, 128), (2, 1, 136, 64)):
+    for B, H, T, hd in ((1, 2, 64, 64), (2, 3, 200, 32), (1, 1, 1024, 64), (1, 2, 520, 128), (2, 1, 136, 64),
+                        (1, 1, 1288, 64), (1, 2, 8, 32)):
         nbh, rows = B * H, B * H * T
         scale = 1.0 / np.sqrt(hd)
         assert dev._lib.mg_tk_attn_p_supported(hd, T)
@@ -196,7 +197,7 @@ def test_scores_and_softmax_in_one_kernel(dev, tk):
         finally:
             for t in (bq, bk, bseg, bp):
                 t.destroy()
-    assert not dev._lib.mg_tk_attn_p_supported(64, 2048) and not dev._lib.mg_tk_attn_p_supported(40, 64)
+    assert not dev._lib.mg_tk_attn_p_supported(128, 2048) and not dev._lib.mg_tk_attn_p_supported(40, 64)
     assert not dev._lib.mg_tk_attn_p_supported(64, 100)
 
 

@@ -7,10 +7,10 @@
 // rowsub[i] = sum_j P[i][j] dP[i][j], which the caller forms as sum_d dOut[i][d] Out[i][d]
 // (mg_tk_attn_rowdot).  The contraction is only as long as a head is wide (64 for GPT-2), so a
 // tiled GEMM has one K-block per tile and spends its time waiting: for the operands, and in
-// an epilogue version of this formula once more for P.  Here nothing passes through LDS and
-// nothing waits twice: the MFMA operands are 16-byte loads straight from dOut and V (a lane
-// of v_mfma_f32_32x32x16 holds 8 consecutive k of one row, which is how both tensors lie in
-// memory), and P and rowsub are requested in the same burst, before the first MFMA.
+// an epilogue version of this formula once more for P.  Here nothing waits twice: the dOut
+// fragments are 16-byte loads straight from memory (a lane of v_mfma_f32_32x32x16 holds 8
+// consecutive k of one row, which is how the tensor lies in memory), the V rows of the
+// workgroup's keys pass through LDS once, and P and rowsub are requested before the first MFMA.
 //
 // What bounds such a kernel on this chip is the number of vector memory instructions, not their
 // bytes: a 4-byte and a 16-byte access per lane cost a wavefront about the same.  So a
@@ -69,10 +69,28 @@ k_attn_ds(const uint16_t *dout, const uint16_t *v, const uint16_t *p16, const fl
     const int64_t b = blockIdx.z;
     const int i0 = blockIdx.y * DS_BM + wave * 32;   // this wavefront's first query
     const int j0 = blockIdx.x * DS_BN;               // and first key
-    if (i0 >= T) return;
-    if (causal && j0 > i0 + 31) return;              // every key beyond every query
+    if (causal && j0 > blockIdx.y * DS_BM + DS_BM - 1) return;   // the whole workgroup lies beyond the diagonal
     const uint16_t *db = dout + b * (int64_t)T * HD;
     const uint16_t *vb = v + b * (int64_t)T * HD;
+    // The 256 rows of V go to LDS once per workgroup, in whole 128-byte-or-longer runs (the
+    // strided 16-byte operand loads of four wavefronts were what this kernel spent its time
+    // on).  Key j0 + 8 n + t is placed at row t * 32 + n, so a block's 32 rows are neighbours;
+    // 16 bytes of padding per row spread a fragment read's 16 lanes over all banks.
+    // (Heads 128 wide would need more than the 64 KiB a static array may hold: they keep the
+    // direct loads.)
+    constexpr bool STAGE = HD <= 64;
+    constexpr int CPR = HD / 8, PITCH = HD * 2 + 16;   // 16-byte chunks per row, bytes per LDS row
+    __shared__ __attribute__((aligned(16))) char vt[STAGE ? DS_BN * PITCH : 16];
+    if constexpr (STAGE) {
+        for (int c = threadIdx.x; c < DS_BN * CPR; c += 256) {
+            const int key = c / CPR, part = c % CPR;
+            const ak_u32x4 x = *reinterpret_cast<const ak_u32x4 *>(vb + (int64_t)min(j0 + key, T - 1) * HD + part * 8);
+            *reinterpret_cast<ak_u32x4 *>(vt + ((key & 7) * 32 + (key >> 3)) * PITCH + part * 16) = x;
+        }
+        __syncthreads();
+    }
+    if (i0 >= T) return;
+    if (causal && j0 > i0 + 31) return;              // every key beyond every query of this wavefront
 
     // MFMA operands: lane l holds row l % 32, k = 8 * (l / 32) .. + 7 of each 16-wide k step
     const int fr = lane & 31, fk = (lane >> 5) * 8;
@@ -98,10 +116,16 @@ k_attn_ds(const uint16_t *dout, const uint16_t *v, const uint16_t *p16, const fl
     ak_f32x16 acc[NB];
 #pragma unroll
     for (int t = 0; t < NB; t++) {
-        const uint16_t *bp = vb + (int64_t)min(j0 + 8 * fr + t, T - 1) * HD + fk;
         ak_u32x4 bf[KK];
+        if constexpr (STAGE) {
+            const char *bp = vt + (t * 32 + fr) * PITCH + fk * 2;
 #pragma unroll
-        for (int kk = 0; kk < KK; kk++) bf[kk] = *reinterpret_cast<const ak_u32x4 *>(bp + kk * 16);
+            for (int kk = 0; kk < KK; kk++) bf[kk] = *reinterpret_cast<const ak_u32x4 *>(bp + kk * 32);
+        } else {
+            const uint16_t *bp = vb + (int64_t)min(j0 + 8 * fr + t, T - 1) * HD + fk;
+#pragma unroll
+            for (int kk = 0; kk < KK; kk++) bf[kk] = *reinterpret_cast<const ak_u32x4 *>(bp + kk * 16);
+        }
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
 #pragma unroll
@@ -232,9 +256,153 @@ k_attn_p(const uint16_t *q16, const uint16_t *k16, const uint32_t *seg, uint16_t
     }
 }
 
+// The same for heads up to 64 wide and any T (a multiple of 8): a workgroup is four blocks of 32
+// queries that walk the key tiles of 256 together, so the K rows of a tile pass through LDS once
+// for 128 queries (in the kernel above every 32 queries fetch all of K with strided 16-byte
+// loads, which is where its time goes).  A row's keys no longer sit in one workgroup's registers
+// at once, so the tiles are walked twice: the first walk keeps, per lane and row, a running
+// maximum and a sum of exponentials relative to it over the lane's own keys (merged across the
+// half-wave once, at the end), the second recomputes the scores and writes P.  The products are
+// cheap next to the memory traffic they save: no f32 scores, K read twice from L2.
+template <int DT, int HD>
+__global__ void __launch_bounds__(256, 2)
+k_attn_p_tiled(const uint16_t *q16, const uint16_t *k16, const uint32_t *seg, uint16_t *p16, int T, int H, float scale,
+               int causal) {
+    constexpr int KK = HD / 16, NB = 8, BN = 256, BM = 128;
+    constexpr int CPR = HD / 8, PITCH = HD * 2 + 16;
+    __shared__ __attribute__((aligned(16))) char kt[BN * PITCH];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t b = blockIdx.y;
+    const int iw = blockIdx.x * BM;      // the workgroup's first query
+    const int i0 = iw + wave * 32;       // this wavefront's
+    const int fr = lane & 31, fk = (lane >> 5) * 8, half = lane >> 5;
+    const int rl = i0 + half * 4;
+    const uint16_t *kb = k16 + b * (int64_t)T * HD;
+    int ntiles = (T + BN - 1) / BN;
+    if (causal) ntiles = min(ntiles, (min(iw + BM, T) - 1) / BN + 1);   // tiles that hold a key <= the last query
+
+    ak_u32x4 af[KK];
+    {
+        const uint16_t *qb = q16 + b * (int64_t)T * HD + (int64_t)min(i0 + fr, T - 1) * HD + fk;
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) af[kk] = *reinterpret_cast<const ak_u32x4 *>(qb + kk * 16);
+    }
+    // first seen key of row i0 + fr, held by lanes fr and fr + 32 and handed round by lane reads
+    const int first_lane = seg ? (int)seg[(b / H) * T + min(i0 + fr, T - 1)] : 0;
+    float mrow[16], lrow[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        mrow[r] = -1e30f;
+        lrow[r] = 0.f;
+    }
+    ak_f32x16 acc[NB];
+    // scores of one tile for this wavefront: acc[t][r] = scale * q . k, or -1e30 where not seen
+    auto tile_scores = [&](int j0) {
+        const int jc = j0 + 8 * fr;
+#pragma unroll
+        for (int t = 0; t < NB; t++) {
+            const char *bp = kt + (t * 32 + fr) * PITCH + fk * 2;
+            ak_u32x4 bf[KK];
+#pragma unroll
+            for (int kk = 0; kk < KK; kk++) bf[kk] = *reinterpret_cast<const ak_u32x4 *>(bp + kk * 32);
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < KK; kk++) acc[t] = ak_mfma<DT>(af[kk], bf[kk], acc[t]);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int ro = (r >> 2) * 8 + (r & 3);
+            const int q = rl + ro;
+            const int flo = __builtin_amdgcn_readlane(first_lane, ro), fhi = __builtin_amdgcn_readlane(first_lane, ro + 4);
+            const int first = half ? fhi : flo;
+#pragma unroll
+            for (int t = 0; t < NB; t++) {
+                const int j = jc + t;
+                acc[t][r] = (j >= first && j <= q && j < T) ? acc[t][r] * scale : -1e30f;
+            }
+        }
+    };
+    auto stage = [&](int j0) {
+        for (int c = threadIdx.x; c < BN * CPR; c += 256) {
+            const int key = c / CPR, part = c % CPR;
+            const ak_u32x4 x = *reinterpret_cast<const ak_u32x4 *>(kb + (int64_t)min(j0 + key, T - 1) * HD + part * 8);
+            *reinterpret_cast<ak_u32x4 *>(kt + ((key & 7) * 32 + (key >> 3)) * PITCH + part * 16) = x;
+        }
+    };
+    for (int pass = 0; pass < 2; pass++) {
+        for (int jt = 0; jt < ntiles; jt++) {
+            const int j0 = jt * BN;
+            __syncthreads();             // everybody is done with the tile before
+            stage(j0);
+            __syncthreads();
+            if (i0 >= T || (causal && j0 > i0 + 31)) continue;   // no key of this tile is seen by this wavefront
+            tile_scores(j0);
+            if (pass == 0) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    float m = mrow[r];
+#pragma unroll
+                    for (int t = 0; t < NB; t++) m = fmaxf(m, acc[t][r]);
+                    float l = lrow[r] * __expf(mrow[r] - m);
+#pragma unroll
+                    for (int t = 0; t < NB; t++) l += acc[t][r] > -1e29f ? __expf(acc[t][r] - m) : 0.f;
+                    mrow[r] = m;
+                    lrow[r] = l;
+                }
+            } else {
+                const int jc = j0 + 8 * fr;
+                const bool col_ok = jc < T;      // T is a multiple of 8: all eight keys exist or none
+                uint16_t *pb = p16 + b * (int64_t)T * T + (col_ok ? jc : 0);
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int ro = (r >> 2) * 8 + (r & 3);
+                    ak_u32x4 o;
+#pragma unroll
+                    for (int w = 0; w < 4; w++) {
+                        const float e0 = acc[2 * w][r] > -1e29f ? __expf(acc[2 * w][r] - mrow[r]) * lrow[r] : 0.f;
+                        const float e1 = acc[2 * w + 1][r] > -1e29f ? __expf(acc[2 * w + 1][r] - mrow[r]) * lrow[r] : 0.f;
+                        o[w] = ak_narrow<DT>(e0) | (ak_narrow<DT>(e1) << 16);
+                    }
+                    if (col_ok && rl + ro < T) *reinterpret_cast<ak_u32x4 *>(pb + (int64_t)(rl + ro) * T) = o;
+                }
+            }
+        }
+        if (pass == 0) {
+            // merge the lanes' (maximum, sum) pairs over the 32 lanes that hold the same rows;
+            // afterwards mrow is the row's maximum and lrow the reciprocal of its sum
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                float m = mrow[r], l = lrow[r];
+#pragma unroll
+                for (int x = 16; x >= 1; x >>= 1) {
+                    const float mo = __shfl_xor(m, x, 64), lo = __shfl_xor(l, x, 64);
+                    const float mn = fmaxf(m, mo);
+                    l = l * __expf(m - mn) + lo * __expf(mo - mn);
+                    m = mn;
+                }
+                mrow[r] = m;
+                lrow[r] = l > 0.f ? 1.0f / l : 0.f;
+            }
+        }
+    }
+}
+
 template <int DT, int HD>
 static void launch_attn_p(hipStream_t s, const void *q, const void *k, const uint32_t *seg, void *p16, int64_t nbh, int T,
                           int H, float scale, int causal) {
+    // up to 1024 keys a row fits the registers of one workgroup and the one-walk kernel is faster
+    // (163 against 127 us at 96 heads x 1024 x 1024 x 64: the second walk's exponentials and
+    // masks cost more than the strided K loads it saves); beyond that only the tiled one exists
+    if constexpr (HD <= 64) {
+        if (T > 1024) {
+            const dim3 grid((unsigned)((T + 127) / 128), (unsigned)nbh);
+            hipLaunchKernelGGL((k_attn_p_tiled<DT, HD>), grid, dim3(256), 0, s, (const uint16_t *)q, (const uint16_t *)k,
+                               seg, (uint16_t *)p16, T, H, scale, causal);
+            return;
+        }
+    }
     const dim3 grid((unsigned)((T + 31) / 32), (unsigned)nbh);
     hipLaunchKernelGGL((k_attn_p<DT, HD>), grid, dim3(256), 0, s, (const uint16_t *)q, (const uint16_t *)k, seg,
                        (uint16_t *)p16, T, H, scale, causal);
@@ -256,11 +424,12 @@ extern "C" {
 
 int mg_tk_attn_ds_supported(int64_t hd, int64_t T) { return (hd == 32 || hd == 64 || hd == 128) && T > 0 && T % 8 == 0; }
 
-int mg_tk_attn_p_supported(int64_t hd, int64_t T) { return mg_tk_attn_ds_supported(hd, T) && T <= 1024; }
+int mg_tk_attn_p_supported(int64_t hd, int64_t T) { return mg_tk_attn_ds_supported(hd, T) && (hd <= 64 || T <= 1024); }
 
 int mg_tk_attn_p(mg_ctx *ctx, const void *q16, const void *k16, const uint32_t *seg, void *p16, int64_t nbh, int64_t T,
                  int64_t H, int64_t hd, float scale, int causal, int dtype) {
     EW_PRECHECK("mg_tk_attn_p", q16 && k16 && p16 && nbh > 0 && nbh <= 65535 && mg_tk_attn_p_supported(hd, T) &&
+                                    T <= 0x7fffffff / 2 &&
                                     H > 0 && nbh % H == 0 && dtype_ok(dtype) && scale == scale &&
                                     (((uintptr_t)q16 | (uintptr_t)k16 | (uintptr_t)p16) & 15) == 0 &&
                                     ((uintptr_t)seg & 3) == 0);
