@@ -198,26 +198,30 @@ k_attn_p(const uint16_t *q16, const uint16_t *k16, const uint32_t *seg, uint16_t
 #pragma unroll
             for (int kk = 0; kk < KK; kk++) acc[t] = ak_mfma<DT>(af[kk], bf[kk], acc[t]);
         }
-        // per row: this lane's 8 keys, then the 32 lanes of the half-wave (they hold the same rows)
+        // Per row: this lane's 8 keys, then the 32 lanes of the half-wave (they hold the same rows).
+        // Everything from here on is in the base-2 domain (scores times scale * log2 e), so an
+        // exponential is one v_exp_f32: this kernel is bound by its instructions per score, not
+        // by memory.  A key that is not seen holds -1e30 and its exponential is exactly 0 - unless
+        // no key of the row is seen by this wavefront, in which case they are all 1 and the sum is
+        // wrong, but then the row's factor below is 2^(-1e30 - max) = 0 and nothing of it is used.
+        // (Keys j >= T need no test: j <= q < T for every row that is stored.)
+        const float c2 = scale * 1.4426950408889634f;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const int ro = (r >> 2) * 8 + (r & 3);
-            const int q = rl + ro;
+            const int q = rl + (r >> 2) * 8 + (r & 3);
             const int first = seg ? (int)seg[(b / H) * T + min(q, T - 1)] : 0;
-            float m = -1e30f;
+            float m = -1e30f, l = 0.f;
 #pragma unroll
             for (int t = 0; t < NB; t++) {
                 const int j = jc + t;
-                const bool seen = j >= first && j <= q && j < T;
-                acc[t][r] = seen ? acc[t][r] * scale : -1e30f;
+                acc[t][r] = (j >= first && j <= q) ? acc[t][r] * c2 : -1e30f;
                 m = fmaxf(m, acc[t][r]);
             }
 #pragma unroll
             for (int x = 16; x >= 1; x >>= 1) m = fmaxf(m, __shfl_xor(m, x, 64));
-            float l = 0.f;
 #pragma unroll
             for (int t = 0; t < NB; t++) {
-                const float e = acc[t][r] > -1e29f ? __expf(acc[t][r] - m) : 0.f;
+                const float e = __builtin_amdgcn_exp2f(acc[t][r] - m);
                 acc[t][r] = e;
                 l += e;
             }
@@ -245,9 +249,9 @@ k_attn_p(const uint16_t *q16, const uint16_t *k16, const uint32_t *seg, uint16_t
         const int rw = ro + half * 4;
         const float m0 = part_m[0][rw], m1 = part_m[1][rw], m2 = part_m[2][rw], m3 = part_m[3][rw];
         const float mx = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
-        const float sum = part_l[0][rw] * __expf(m0 - mx) + part_l[1][rw] * __expf(m1 - mx) +
-                          part_l[2][rw] * __expf(m2 - mx) + part_l[3][rw] * __expf(m3 - mx);
-        const float f = __expf(mloc[r] - mx) / sum;   // (a row no key of which is seen does not occur: key q always is)
+        const float sum = part_l[0][rw] * __builtin_amdgcn_exp2f(m0 - mx) + part_l[1][rw] * __builtin_amdgcn_exp2f(m1 - mx) +
+                          part_l[2][rw] * __builtin_amdgcn_exp2f(m2 - mx) + part_l[3][rw] * __builtin_amdgcn_exp2f(m3 - mx);
+        const float f = __builtin_amdgcn_exp2f(mloc[r] - mx) / sum;   // (a row no key of which is seen does not occur: key q always is)
         ak_u32x4 o;
 #pragma unroll
         for (int w = 0; w < 4; w++)
