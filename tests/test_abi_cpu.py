@@ -80,6 +80,24 @@ def test_validation_rejects(lib, kw, needle):
     assert needle in L.last_error(), L.last_error()
 
 
+def test_softmax_grad_epilogue_validation(lib):
+    """act = MG_ACT_SOFTMAX_GRAD: needs y16, p16 and rowsub, beta 0, no bias; batches allowed
+    (the other fused outputs are not), their stride must keep the batches of y16 and p16 apart."""
+    sg = dict(act=L.MG_ACT_SOFTMAX_GRAD, y16=0x5000, ldy=96, p16=0x6000, ldp=96, rowsub=0x7000, scale=0.125)
+    assert lib.mg_gemm_check(C.byref(good_args(**sg))) == L.MG_OK
+    assert lib.mg_gemm_check(C.byref(good_args(c=None, **sg))) == L.MG_OK          # C is optional
+    assert lib.mg_gemm_check(C.byref(good_args(nbatch=3, sa=128 * 64, sb=64 * 96, sc=128 * 96, **sg))) == L.MG_OK
+    for bad, needle in ((dict(p16=None), "p16"), (dict(rowsub=None), "rowsub"), (dict(ldp=95), "ldp"),
+                        (dict(beta=1), "beta"), (dict(bias=0x4000), "bias"), (dict(z=0x8000, ldz=96), "z and colsum"),
+                        (dict(scale=float("nan")), "NaN"), (dict(y16=None), "y16"), (dict(layout=L.MG_TN, lda=128), "NN and NT"),
+                        (dict(nbatch=3, sa=128 * 64, sb=64 * 96, sc=128 * 96 - 8, ldc=90, n=90, ldb=90, ldy=96, ldp=96), "overlaps")):
+        assert lib.mg_gemm_check(C.byref(good_args(**{**sg, **bad}))) == L.MG_ERR_ARG, bad
+        assert needle in L.last_error(), (bad, L.last_error())
+    # p16 / rowsub without the activation, and batches with another fused output
+    assert lib.mg_gemm_check(C.byref(good_args(p16=0x6000, ldp=96))) == L.MG_ERR_ARG
+    assert lib.mg_gemm_check(C.byref(good_args(nbatch=2, sa=128 * 64, sb=64 * 96, sc=128 * 96, y16=0x5000, ldy=96))) == L.MG_ERR_ARG
+
+
 def test_layout_dependent_leading_dimensions(lib):
     # TN: A is (K, M), so lda >= M; NT: B is (N, K), so ldb >= K
     assert lib.mg_gemm_check(C.byref(good_args(layout=L.MG_TN, lda=128))) == L.MG_OK
