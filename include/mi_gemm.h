@@ -293,6 +293,10 @@ typedef struct {
 } mg_adamw_entry;
 int mg_ew_adamw_multi(mg_ctx *ctx, const mg_adamw_entry *table_dev, int ntensors, int64_t total_blocks, const float *hp,
                       int dtype);
+/* g[0 .. n) = 0 for every entry of such a table (only g, n and first_block are read), in one launch:
+ * the clears in front of the bias and LayerNorm gradient sums of a step (col_sum_zero,
+ * tkernels.py:238-246, once per sum in the reference), gathered at the start of its backward pass. */
+int mg_ew_zero_multi(mg_ctx *ctx, const mg_adamw_entry *table_dev, int ntensors, int64_t total_blocks);
 int mg_ew_zero(mg_ctx *ctx, float *dst, int64_t n);
 /* Device-side copy of nbytes (multiple of 4, both pointers 4-byte aligned) that can be
  * recorded into a graph, unlike mg_copy.  The reference's recorded step reads what the CPU

@@ -102,6 +102,7 @@ SIGNATURES = {
     "mg_ew_softmax_ce": (C.c_int, [_P, _P, _P, _P, _P, _P, C.c_int64, C.c_int64, C.c_int64, C.c_int]),
     "mg_ew_adamw": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, C.c_int64, C.c_float, C.c_int]),
     "mg_ew_adamw_multi": (C.c_int, [_P, _P, C.c_int, C.c_int64, _P, C.c_int]),
+    "mg_ew_zero_multi": (C.c_int, [_P, _P, C.c_int, C.c_int64]),
     "mg_ew_zero": (C.c_int, [_P, _P, C.c_int64]),
     "mg_ew_copy": (C.c_int, [_P, _P, _P, C.c_int64]),
     "mg_ew_cast16": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int]),

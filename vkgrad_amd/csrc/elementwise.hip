@@ -174,6 +174,20 @@ __global__ void __launch_bounds__(256) k_adamw_multi(const mg_adamw_entry *table
     }
 }
 
+// Clears the gradient of every entry of an AdamW-style table in one launch (same block numbering).
+__global__ void __launch_bounds__(256) k_zero_multi(const mg_adamw_entry *table, int ntensors) {
+    int lo = 0, hi = ntensors - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (table[mid].first_block <= (int64_t)blockIdx.x) lo = mid;
+        else hi = mid - 1;
+    }
+    const mg_adamw_entry e = table[lo];
+    float *g = const_cast<float *>(e.g);
+    const int64_t i0 = (((int64_t)blockIdx.x - e.first_block) * 256 + threadIdx.x) * 4;
+    for (int k = 0; k < 4 && i0 + k < e.n; k++) g[i0 + k] = 0.f;
+}
+
 __global__ void k_zero(float *dst, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) dst[i] = 0.f;
@@ -290,6 +304,12 @@ int mg_ew_adamw_multi(mg_ctx *ctx, const mg_adamw_entry *table_dev, int ntensors
     hipLaunchKernelGGL(k_adamw_multi, dim3((unsigned)total_blocks), dim3(256), 0, ctx_stream(ctx), table_dev, ntensors, hp,
                        dtype);
     EW_POSTCHECK("mg_ew_adamw_multi");
+}
+
+int mg_ew_zero_multi(mg_ctx *ctx, const mg_adamw_entry *table_dev, int ntensors, int64_t total_blocks) {
+    EW_PRECHECK("mg_ew_zero_multi", table_dev && ntensors > 0 && total_blocks > 0 && total_blocks <= 0x7fffffff);
+    hipLaunchKernelGGL(k_zero_multi, dim3((unsigned)total_blocks), dim3(256), 0, ctx_stream(ctx), table_dev, ntensors);
+    EW_POSTCHECK("mg_ew_zero_multi");
 }
 
 int mg_ew_zero(mg_ctx *ctx, float *dst, int64_t n) {

@@ -24,9 +24,13 @@ Shapes are free (tiles mask their edges); only the vocabulary is padded, to a
 multiple of 64 so that rows of the logits stay 16-byte aligned.
 """
 
+import ctypes as C
+
 import numpy as np
 
+from . import _lib as _L
 from .autograd import Ctx, Param, _seed
+from .kernels import Elementwise
 from .tkernels import make_transformer_kernels
 
 NCHUNK = 32   # part of the reference's column-sum call shape; the library picks its own chunks
@@ -49,6 +53,7 @@ class TCtx(Ctx):
         self.causal_gemms = bool(causal_gemms)   # attention GEMMs skip what the causal mask zeroes
         self.TK = make_transformer_kernels(dev, dtype)
         self.wave = dev.row_subgroup_size
+        self._cleared = set()   # gradient buffers that clear_grads zeroes at the start of a backward pass
 
     def rowwise(self, name, buffers, rows, *args, graph=None):
         """A row kernel over `rows` rows (dispatch size rows * wavefront width)."""
@@ -57,8 +62,32 @@ class TCtx(Ctx):
     def col_sum(self, src, dst, ncol, nrow, graph=None, f16=True):
         """dst[c] = sum over rows of src[r, c]; reads the 16-bit copy unless f16=False.  The
         library clears dst itself when the rows span several chunks (the reference's
-        `col_sum_zero` + `col_sum_chunk16` pair, transformer.py:30-37, in one call)."""
-        self.TK["col_sum16" if f16 else "col_sum"]([src, dst], ncol, nrow, graph=graph)
+        `col_sum_zero` + `col_sum_chunk16` pair, transformer.py:30-37, in one call) - unless
+        `clear_grads` has cleared it at the start of this backward pass already."""
+        if dst.ptr in self._cleared:
+            self.TK["col_sum_chunk16" if f16 else "col_sum_chunk"]([src, dst], NCHUNK * ncol, ncol, nrow, NCHUNK,
+                                                                    graph=graph)
+        else:
+            self.TK["col_sum16" if f16 else "col_sum"]([src, dst], ncol, nrow, graph=graph)
+
+    def clear_grads(self, params, graph=None):
+        """One launch that zeroes the gradients of `params` (the step's bias and LayerNorm
+        parameters); `col_sum` into them then only adds.  The reference clears in front of every
+        sum (transformer.py:30-37): a hundred 4 us launches in a GPT-2-small step."""
+        params = list(params)
+        if not params:
+            return
+        entries = (_L.AdamWEntry * len(params))()
+        blocks = 0
+        for e, p in zip(entries, params):
+            e.g, e.n, e.first_block = p.g32.ptr, p.n, blocks
+            blocks += -(-p.n // 1024)
+        table = self.buf(C.sizeof(entries), "device")
+        table.upload(np.frombuffer(entries, dtype=np.uint8))
+        n = len(params)
+        Elementwise(self.dev, "zero_multi", lambda lib, mg, ptrs, _n: lib.mg_ew_zero_multi(mg, ptrs[0], n, blocks))(
+            [table], n, graph=graph)
+        self._cleared.update(p.g32.ptr for p in params)
 
     def destroy(self):
         for kern in self.TK.values():
@@ -413,9 +442,14 @@ class GPT:
             TK["softmax_ce_w"]([logits, targets_buf, weights, self.dlog16, self.loss], *shape, graph=stage(L))
         if not backward:
             return
+        if self.ctx.fuse:
+            # every bias and LayerNorm gradient is a column sum: clear them all in one launch here
+            # instead of one small launch in front of each sum
+            self.ctx.clear_grads([p for p in self.params() if len(p.shape) == 1], graph=stage(L + 1))
         d = self.lnf.backward(self._head_backward(stage(L + 1)), graph=stage(L + 1))
         for k, blk in enumerate(reversed(self.blocks)):
             d = blk.backward(d, graph=stage(L + 2 + k))
+        self.ctx._cleared.clear()   # later recordings clear for themselves again
         last = stage(2 * L + 2)
         TK["col_sum_zero"]([self.pos.g32], self.pos.n, graph=last)
         self._embedding("embed_bwd", [d], ids_buf, seg, [self.tok.g32, self.pos.g32], last)
