@@ -151,13 +151,20 @@ k_attn_ds(const uint16_t *dout, const uint16_t *v, const uint16_t *p16, const fl
 
 // P of attention in one kernel: the scores = Q K^T product of every head (reference call site
 // transformer.py:153-155) and the masked softmax over them (attn_softmax / attn_softmax_doc,
-// tkernels.py:105-165), without the f32 score matrix in between.  Same wavefront shape and key
-// interleaving as k_attn_ds above; the four wavefronts of a workgroup split the keys of the same
-// 32 queries between them (256 each, so T <= 1024), every wavefront reduces its part of a row
-// to a maximum and a sum of exponentials relative to it, the parts meet once in LDS, and each
-// wavefront rescales and writes its own 256 keys.  Row r (query q = r % T of its head) sees keys
-// first .. q, first = 0 or seg[batch * T + q]; masked keys get 0.  With `causal` set, a
-// wavefront whose keys all lie beyond its queries writes nothing: the caller keeps P zero there.
+// tkernels.py:105-165), without the f32 score matrix in between.  The product is formed
+// transposed, K Q^T: the 32 queries of a workgroup lie along the accumulator columns (one query
+// per lane), the keys along the rows, so everything a softmax row needs - its maximum, its sum -
+// is a reduction over a lane's own registers plus one exchange between the two half-waves.  (With
+// the queries along the rows each of the 16 rows a lane holds had to be reduced over 32 lanes:
+// 160 lane exchanges per wavefront, which an ablation showed to cost more than the loads.)
+// The four wavefronts of a workgroup split the keys between them (256 each, so T <= 1024), meet
+// once in LDS with their (maximum, sum) pairs, and each rescales and writes its own keys.  Which
+// key an accumulator row stands for is decided by the row of K its lane loaded: row 8g + 4h + e
+// of a block takes key 16h + 4g + e, so register r of half-wave h is key 16h + r and a lane
+// writes 16 neighbouring keys of its query as two 16-byte stores per block.
+// Query q (= row % T of its head) sees keys first .. q, first = 0 or seg[batch * T + q]; masked
+// keys get 0.  With `causal` set, a wavefront whose keys all lie beyond its queries writes
+// nothing: the caller keeps P zero there.
 template <int DT, int HD>
 __global__ void __launch_bounds__(256, 2)
 k_attn_p(const uint16_t *q16, const uint16_t *k16, const uint32_t *seg, uint16_t *p16, int T, int H, float scale,
@@ -169,95 +176,81 @@ k_attn_p(const uint16_t *q16, const uint16_t *k16, const uint32_t *seg, uint16_t
     const int64_t b = blockIdx.y;
     const int i0 = blockIdx.x * 32;      // the workgroup's first query
     const int j0 = wave * 256;           // this wavefront's first key
-    const int fr = lane & 31, fk = (lane >> 5) * 8, half = lane >> 5;
+    const int n = lane & 31, half = lane >> 5, fk = half * 8;
+    const int q = i0 + n;                // this lane's query
     // keys that no query of this block may see: none of them, or (causal) all beyond the last query
     const bool idle = j0 >= T || (causal && j0 > i0 + 31);
-    const int rl = i0 + half * 4;        // accumulator register r: row rl + ro, ro = 8 * (r / 4) + r % 4
-    const int jc = j0 + 8 * fr;          // this lane's keys: jc + t, one per block t
     ak_f32x16 acc[NB];
-    float mloc[16], lloc[16];
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-        mloc[r] = -1e30f;
-        lloc[r] = 0.f;
-    }
+    float m = -1e30f, l = 0.f;
     if (!idle) {
-        const uint16_t *qb = q16 + b * (int64_t)T * HD + (int64_t)min(i0 + fr, T - 1) * HD + fk;
+        const uint16_t *qb = q16 + b * (int64_t)T * HD + (int64_t)min(q, T - 1) * HD + fk;
         const uint16_t *kb = k16 + b * (int64_t)T * HD;
-        ak_u32x4 af[KK];
+        ak_u32x4 bf[KK];                 // B operand: the queries
 #pragma unroll
-        for (int kk = 0; kk < KK; kk++) af[kk] = *reinterpret_cast<const ak_u32x4 *>(qb + kk * 16);
+        for (int kk = 0; kk < KK; kk++) bf[kk] = *reinterpret_cast<const ak_u32x4 *>(qb + kk * 16);
+        const int first = seg ? (int)seg[(b / H) * T + min(q, T - 1)] : 0;
+        // A operand row n = 8g + 4h' + e of block t is key j0 + 32 t + 16 h' + 4 g + e
+        const int arow = 16 * ((n >> 2) & 1) + 4 * (n >> 3) + (n & 3);
 #pragma unroll
         for (int t = 0; t < NB; t++) {
-            const uint16_t *bp = kb + (int64_t)min(jc + t, T - 1) * HD + fk;
-            ak_u32x4 bf[KK];
+            const uint16_t *ap = kb + (int64_t)min(j0 + 32 * t + arow, T - 1) * HD + fk;
+            ak_u32x4 af[KK];
 #pragma unroll
-            for (int kk = 0; kk < KK; kk++) bf[kk] = *reinterpret_cast<const ak_u32x4 *>(bp + kk * 16);
+            for (int kk = 0; kk < KK; kk++) af[kk] = *reinterpret_cast<const ak_u32x4 *>(ap + kk * 16);
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
 #pragma unroll
             for (int kk = 0; kk < KK; kk++) acc[t] = ak_mfma<DT>(af[kk], bf[kk], acc[t]);
         }
-        // Per row: this lane's 8 keys, then the 32 lanes of the half-wave (they hold the same rows).
-        // Everything from here on is in the base-2 domain (scores times scale * log2 e), so an
-        // exponential is one v_exp_f32: this kernel is bound by its instructions per score, not
-        // by memory.  A key that is not seen holds -1e30 and its exponential is exactly 0 - unless
-        // no key of the row is seen by this wavefront, in which case they are all 1 and the sum is
-        // wrong, but then the row's factor below is 2^(-1e30 - max) = 0 and nothing of it is used.
-        // (Keys j >= T need no test: j <= q < T for every row that is stored.)
+        // Base-2 domain (scores times scale * log2 e): an exponential is one v_exp_f32.  A key that
+        // is not seen holds -1e30 and its exponential is exactly 0 - unless no key of this
+        // wavefront is seen by the query, in which case they are all 1 and the sum is wrong, but
+        // then the factor below is 2^(-1e30 - max) = 0 and nothing of it is used.  (Keys >= T need
+        // no test: key <= q < T for every query that is stored.)
         const float c2 = scale * 1.4426950408889634f;
+        const int k0 = j0 + 16 * half;   // register r of block t: key k0 + 32 t + r
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int q = rl + (r >> 2) * 8 + (r & 3);
-            const int first = seg ? (int)seg[(b / H) * T + min(q, T - 1)] : 0;
-            float m = -1e30f, l = 0.f;
+        for (int t = 0; t < NB; t++)
 #pragma unroll
-            for (int t = 0; t < NB; t++) {
-                const int j = jc + t;
-                acc[t][r] = (j >= first && j <= q) ? acc[t][r] * c2 : -1e30f;
+            for (int r = 0; r < 16; r++) {
+                const int key = k0 + 32 * t + r;
+                acc[t][r] = (key >= first && key <= q) ? acc[t][r] * c2 : -1e30f;
                 m = fmaxf(m, acc[t][r]);
             }
+        m = fmaxf(m, __shfl_xor(m, 32, 64));
 #pragma unroll
-            for (int x = 16; x >= 1; x >>= 1) m = fmaxf(m, __shfl_xor(m, x, 64));
+        for (int t = 0; t < NB; t++)
 #pragma unroll
-            for (int t = 0; t < NB; t++) {
+            for (int r = 0; r < 16; r++) {
                 const float e = __builtin_amdgcn_exp2f(acc[t][r] - m);
                 acc[t][r] = e;
                 l += e;
             }
-#pragma unroll
-            for (int x = 16; x >= 1; x >>= 1) l += __shfl_xor(l, x, 64);
-            mloc[r] = m;
-            lloc[r] = l;
-        }
+        l += __shfl_xor(l, 32, 64);
     }
-    if (fr == 0) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int ro = (r >> 2) * 8 + (r & 3);
-            part_m[wave][ro + half * 4] = mloc[r];
-            part_l[wave][ro + half * 4] = lloc[r];
-        }
+    if (half == 0) {
+        part_m[wave][n] = m;
+        part_l[wave][n] = l;
     }
     __syncthreads();
-    if (idle) return;
-    const bool col_ok = jc < T;          // T is a multiple of 8: all eight keys exist or none
-    uint16_t *pb = p16 + b * (int64_t)T * T + (col_ok ? jc : 0);
+    if (idle || q >= T) return;
+    const float m0 = part_m[0][n], m1 = part_m[1][n], m2 = part_m[2][n], m3 = part_m[3][n];
+    const float mx = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
+    const float sum = part_l[0][n] * __builtin_amdgcn_exp2f(m0 - mx) + part_l[1][n] * __builtin_amdgcn_exp2f(m1 - mx) +
+                      part_l[2][n] * __builtin_amdgcn_exp2f(m2 - mx) + part_l[3][n] * __builtin_amdgcn_exp2f(m3 - mx);
+    const float f = __builtin_amdgcn_exp2f(m - mx) / sum;   // (a query that sees no key does not occur: key q always is)
+    uint16_t *pq = p16 + b * (int64_t)T * T + (int64_t)q * T + j0 + 16 * half;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const int ro = (r >> 2) * 8 + (r & 3);
-        const int rw = ro + half * 4;
-        const float m0 = part_m[0][rw], m1 = part_m[1][rw], m2 = part_m[2][rw], m3 = part_m[3][rw];
-        const float mx = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
-        const float sum = part_l[0][rw] * __builtin_amdgcn_exp2f(m0 - mx) + part_l[1][rw] * __builtin_amdgcn_exp2f(m1 - mx) +
-                          part_l[2][rw] * __builtin_amdgcn_exp2f(m2 - mx) + part_l[3][rw] * __builtin_amdgcn_exp2f(m3 - mx);
-        const float f = __builtin_amdgcn_exp2f(mloc[r] - mx) / sum;   // (a row no key of which is seen does not occur: key q always is)
-        ak_u32x4 o;
+    for (int t = 0; t < NB; t++)
 #pragma unroll
-        for (int w = 0; w < 4; w++)
-            o[w] = ak_narrow<DT>(acc[2 * w][r] * f) | (ak_narrow<DT>(acc[2 * w + 1][r] * f) << 16);
-        if (col_ok && rl + ro < T) *reinterpret_cast<ak_u32x4 *>(pb + (int64_t)(rl + ro) * T) = o;
-    }
+        for (int u = 0; u < 2; u++) {
+            ak_u32x4 o;
+#pragma unroll
+            for (int w = 0; w < 4; w++)
+                o[w] = ak_narrow<DT>(acc[t][8 * u + 2 * w] * f) | (ak_narrow<DT>(acc[t][8 * u + 2 * w + 1] * f) << 16);
+            // T is a multiple of 8: the eight keys of a store exist or none does
+            if (j0 + 16 * half + 32 * t + 8 * u < T) *reinterpret_cast<ak_u32x4 *>(pq + 32 * t + 8 * u) = o;
+        }
 }
 
 // The same for heads up to 64 wide and any T (a multiple of 8): a workgroup is four blocks of 32
