@@ -111,7 +111,8 @@ typedef struct {
      *                   its last row;
      *   MG_TRI_A_UPPER  op(A)[i][k] == 0 for k < i (P^T dOut, dS^T Q with A stored (k, m)): the K
      *                   loop starts at the block's first row.
-     * The A forms need m == k and run unsplit; every batch has the same structure. */
+     * The A forms need m == k; they split K only on request (split_k > 1: a slice wholly outside a row
+ * block's range is empty), MG_TRI_C_LOWER never; every batch has the same structure. */
     int32_t tri;           /* MG_TRI_* */
     int32_t reserved;      /* 0 */
     /* Softmax-backward epilogue - replaces the separate pass of attn_softmax_bwd

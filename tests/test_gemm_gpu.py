@@ -480,12 +480,13 @@ def test_triangular_structure_of_causal_attention(dev, dtype):
     from vkgrad_amd.vk import VkError
     rng = np.random.default_rng(5)
 
-    def run(layout, m, n, k, tile, tri, nb, a, b):
+    def run(layout, m, n, k, tile, tri, nb, a, b, split_k=0, atomic=False):
         ta, tb = LAYOUTS[layout]
         ba, bb, bc = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), dev.buffer(nb * m * n * 4, "device")
         ba.upload(a); bb.upload(b)
         bc.upload(np.full((nb, m, n), np.nan, np.float32))
-        mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype=dtype, tile=tile, batched=nb > 1)
+        mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype=dtype, tile=tile, batched=nb > 1, split_k=split_k,
+                    atomic_split=atomic)
         try:
             mm(ba, bb, bc, m, n, k, nbatch=nb, strides=(a[0].size, b[0].size, m * n), tri=tri)
             return bc.download(np.float32, (nb, m, n))
@@ -527,6 +528,14 @@ def test_triangular_structure_of_causal_attention(dev, dtype):
         at_tri[:, ~np.tril(np.ones((k, m), bool))] = 0          # stored A lower triangular = op(A) upper
         got = run("TN", m, n, k, tile, "a_upper", nb, at_tri, bt)
         assert np.array_equal(got, product("TN", at_tri, bt)), (m, n, k, tile, "a_upper")
+        # with a K split (on request only): slices wholly outside a row block's K range are empty;
+        # they meet in the workspace, or add into C with atomics (integer data: exact either way)
+        if tile in (None, 14, 4, 11):
+            for split, atomic in ((4, False), (3, True), (4, True)):
+                got = run("NN", m, n, k, tile, "a_lower", nb, a_tri, b, split, atomic)
+                assert np.array_equal(got, product("NN", a_tri, b)), (m, n, k, tile, "a_lower", split, atomic)
+                got = run("TN", m, n, k, tile, "a_upper", nb, at_tri, bt, split, atomic)
+                assert np.array_equal(got, product("TN", at_tri, bt)), (m, n, k, tile, "a_upper", split, atomic)
     buf = dev.buffer(64 * 64 * 4, "device")
     mm = Matmul(dev, dtype=dtype)
     mm2 = Matmul(dev, dtype=dtype, split_k=2)

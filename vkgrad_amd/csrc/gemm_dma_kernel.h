@@ -217,6 +217,7 @@ gemm_dma_kernel(const GemmParams p) {
     int kbeg = blockIdx.y * p.k_per_split;
     int kend = min(p.K, kbeg + p.k_per_split);
     tri_k_range<BM, BK>(p.tri, m0, kbeg, kend);
+    if (kend == kbeg && p.split_k > 1 && p.ws == nullptr) return;   // an empty slice has nothing to add to C
     const int krem = (kend - kbeg) % BK;          // K remainder, multiplied first
     const int kdma = kbeg + krem;                 // the ring covers [kdma, kend)
     const int nkb = (kend - kdma) / BK;

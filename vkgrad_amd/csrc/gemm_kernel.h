@@ -344,12 +344,14 @@ __device__ __forceinline__ void interleave_group() {
     interleave_step<0, NMFMA, NDSR, NDSW, NVMEM>();
 }
 
-// K range of a row block when op(A) is triangular (one slice, M == K): rows m0 .. m0 + BM - 1
-// meet non-zero entries of op(A) only for k <= m0 + BM - 1 (lower) or k >= m0 (upper).
+// K range of a row block when op(A) is triangular (M == K): rows m0 .. m0 + BM - 1 meet non-zero
+// entries of op(A) only for k <= m0 + BM - 1 (lower) or k >= m0 (upper).  With a K split a
+// slice may lie wholly outside that range: it comes back empty (kend == kbeg).
 template <int BM, int BK>
 __device__ __forceinline__ void tri_k_range(int tri, int m0, int &kbeg, int &kend) {
     if (tri == 2) kend = min(kend, m0 + BM);
     if (tri == 3) kbeg = max(kbeg, (m0 / BK) * BK);
+    if (kend < kbeg) kend = kbeg;
 }
 
 // 16-bit narrowing (round to nearest even) and the activations of the fused output;
@@ -561,6 +563,7 @@ gemm_kernel(const GemmParams p) {
     int kbeg = blockIdx.y * p.k_per_split;
     int kend = min(p.K, kbeg + p.k_per_split);
     tri_k_range<BM, BK>(p.tri, m0, kbeg, kend);
+    if (kend == kbeg && p.split_k > 1 && p.ws == nullptr) return;   // an empty slice has nothing to add to C
     const int nkb = (kend - kbeg + BK - 1) / BK;
     // K-blocks that the unconditional loader may fetch: the whole block inside
     // K, and the tile inside M and N.

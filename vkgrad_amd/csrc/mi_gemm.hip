@@ -295,7 +295,11 @@ static void finish_plan(const mg_gemm_args &a, int tile, int split, Plan &pl) {
     int64_t kblocks = cdiv(a.k, d->bk);
     if (split > kblocks) split = (int)kblocks;
     if (split < 1) split = 1;
-    if (d->persistent == 2 || d->gemv || a.tri || a.act == MG_ACT_SOFTMAX_GRAD) split = 1;
+    // a triangular op(A) splits only on request (the K ranges of the row blocks differ: the picker's
+    // cost model does not price that), the lower-triangular C never
+    if (d->persistent == 2 || d->gemv || a.tri == MG_TRI_C_LOWER || (a.tri && a.split_k <= 1) ||
+        a.act == MG_ACT_SOFTMAX_GRAD)
+        split = 1;
     int64_t kb_per = cdiv(kblocks, split);
     split = (int)cdiv(kblocks, kb_per);   // no empty slices
     while (!dma_eligible(a, *d, kb_per * d->bk, split) && d->fallback != tile) {
@@ -425,7 +429,8 @@ static int check_args(const mg_gemm_args *a) {
     if (a->tri >= MG_TRI_A_LOWER && a->m != a->k)
         return fail(MG_ERR_ARG, "mg_gemm: a triangular op(A) needs M == K, got %lld and %lld", (long long)a->m,
                     (long long)a->k);
-    if (a->tri && a->split_k > 1) return fail(MG_ERR_ARG, "mg_gemm: tri runs unsplit; split_k is %d", a->split_k);
+    if (a->tri == MG_TRI_C_LOWER && a->split_k > 1)
+        return fail(MG_ERR_ARG, "mg_gemm: MG_TRI_C_LOWER runs unsplit; split_k is %d", a->split_k);
     if (a->res) {
         if (a->beta != 1) return fail(MG_ERR_ARG, "mg_gemm: res is what beta == 1 adds to; beta is %d", a->beta);
         if ((uintptr_t)a->res & 3) return fail(MG_ERR_ARG, "mg_gemm: res must be 4-byte aligned");
