@@ -253,14 +253,14 @@ k_attn_p(const uint16_t *q16, const uint16_t *k16, const uint32_t *seg, uint16_t
         }
 }
 
-// The same for heads up to 64 wide and any T (a multiple of 8): a workgroup is four blocks of 32
-// queries that walk the key tiles of 256 together, so the K rows of a tile pass through LDS once
-// for 128 queries (in the kernel above every 32 queries fetch all of K with strided 16-byte
-// loads, which is where its time goes).  A row's keys no longer sit in one workgroup's registers
-// at once, so the tiles are walked twice: the first walk keeps, per lane and row, a running
+// The same for heads up to 64 wide and any T (a multiple of 8), for rows longer than the 1024 keys
+// the kernel above can hold: a workgroup is four blocks of 32 queries (queries along the
+// accumulator rows here, as in k_attn_ds) that walk the key tiles of 256 together, the K rows of
+// a tile passing through LDS once for the 128 queries.  A row's keys never sit in the registers
+// all at once, so the tiles are walked twice: the first walk keeps, per lane and row, a running
 // maximum and a sum of exponentials relative to it over the lane's own keys (merged across the
-// half-wave once, at the end), the second recomputes the scores and writes P.  The products are
-// cheap next to the memory traffic they save: no f32 scores, K read twice from L2.
+// half-wave once, at the end), the second recomputes the scores and writes P.  Still no f32
+// scores; K is read twice from L2.
 template <int DT, int HD>
 __global__ void __launch_bounds__(256, 2)
 k_attn_p_tiled(const uint16_t *q16, const uint16_t *k16, const uint32_t *seg, uint16_t *p16, int T, int H, float scale,
