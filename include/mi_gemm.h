@@ -387,6 +387,9 @@ int mg_tk_residual(mg_ctx *ctx, const float *acc, const float *bias, const float
                    int64_t D);
 /* add (tkernels.py:373-377) and add_bias (in place, tkernels.py:379-382) */
 int mg_tk_add(mg_ctx *ctx, const float *a, const float *b, float *out, int64_t n);
+/* out = a + b together with out16 = narrow(out): `add` followed by `to16` of the sum
+ * (transformer.py:242-252, tkernels.py:372-389) in one pass. */
+int mg_tk_add16(mg_ctx *ctx, const float *a, const float *b, float *out, void *out16, int64_t n, int dtype);
 int mg_tk_add_bias(mg_ctx *ctx, float *x, const float *bias, int64_t n, int64_t ncol);
 /* col_sum_zero + col_sum_chunk16 (tkernels.py:238-270; transformer.py:30-37): column sums of a
  * 16-bit (nrow, ncol) matrix, f32 accumulation; accumulate != 0 adds to sums. */

@@ -274,6 +274,9 @@ def test_embeddings_residual_and_column_sums(dev, tk):
                 np.allclose(bo.download(np.float32, (rows, D)), RT.residual(acc, bias, res), atol=1e-6)
             TK["add"]([ba, br, bo], rows * D)
             assert np.array_equal(bo.download(np.float32, (rows, D)), acc + res)
+            TK["add16"]([ba, br, bo, b16], rows * D)        # the sum and its 16-bit copy in one pass
+            assert np.array_equal(bo.download(np.float32, (rows, D)), acc + res)
+            assert np.array_equal(stored(b16, dtype, (rows, D)).view(np.uint16), O.round_to(acc + res, dtype).view(np.uint16))
             TK["add_bias"]([bo, bb], rows * D, D)
             assert np.array_equal(bo.download(np.float32, (rows, D)), (acc + res) + bias[None, :])
             TK["to16"]([ba, b16], rows * D)
@@ -298,6 +301,9 @@ def test_embeddings_residual_and_column_sums(dev, tk):
             assert np.array_equal(bo.download(np.float32, (r2, d2)), (res2 + acc2) + bias2[None, :])
             TK["add"]([ba, br, bo], r2 * d2)
             assert np.array_equal(bo.download(np.float32, (r2, d2)), acc2 + res2)
+            TK["add16"]([ba, br, bo, b16], r2 * d2)
+            assert np.array_equal(bo.download(np.float32, (r2, d2)), acc2 + res2)
+            assert np.array_equal(stored(b16, dtype, (r2, d2)).view(np.uint16), O.round_to(acc2 + res2, dtype).view(np.uint16))
             TK["to16"]([ba, b16], r2 * d2)
             assert np.array_equal(stored(b16, dtype, (r2, d2)).view(np.uint16), O.round_to(acc2, dtype).view(np.uint16))
         finally:

@@ -126,6 +126,7 @@ SIGNATURES = {
     "mg_tk_embed_bwd": (C.c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I]),
     "mg_tk_residual": (C.c_int, [_P, _P, _P, _P, _P, _I, _I]),
     "mg_tk_add": (C.c_int, [_P, _P, _P, _P, _I]),
+    "mg_tk_add16": (C.c_int, [_P, _P, _P, _P, _P, _I, C.c_int]),
     "mg_tk_add_bias": (C.c_int, [_P, _P, _P, _I, _I]),
     "mg_tk_col_sum16": (C.c_int, [_P, _P, _P, _I, _I, C.c_int, C.c_int]),
     "mg_tk_softmax_ce": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, C.c_int]),

@@ -495,6 +495,25 @@ __global__ void k_residual(const float *acc, const float *bias, const float *res
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) out[i] = res[i] + acc[i] + bias[i % D];
 }
+// out = a + b and its 16-bit copy in one pass: the `add` of a residual's two gradient paths
+// followed by the `to16` of the sum for the next GEMMs (transformer.py:242-252).
+__global__ void k_add16_v4(const float *a, const float *b, float *out, uint16_t *out16, int64_t n4, int dtype) {
+    const int64_t i4 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i4 >= n4) return;
+    float4 x = reinterpret_cast<const float4 *>(a)[i4];
+    const float4 y = reinterpret_cast<const float4 *>(b)[i4];
+    x.x += y.x; x.y += y.y; x.z += y.z; x.w += y.w;
+    reinterpret_cast<float4 *>(out)[i4] = x;
+    reinterpret_cast<uint2 *>(out16)[i4] = narrow16x4(x.x, x.y, x.z, x.w, dtype);
+}
+__global__ void k_add16(const float *a, const float *b, float *out, uint16_t *out16, int64_t n, int dtype) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const float x = a[i] + b[i];
+        out[i] = x;
+        out16[i] = narrow16(x, dtype);
+    }
+}
 __global__ void k_add(const float *a, const float *b, float *out, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) out[i] = a[i] + b[i];
@@ -799,6 +818,16 @@ int mg_tk_add(mg_ctx *ctx, const float *a, const float *b, float *out, int64_t n
     else
         hipLaunchKernelGGL(k_add, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), a, b, out, n);
     EW_POSTCHECK("mg_tk_add");
+}
+
+int mg_tk_add16(mg_ctx *ctx, const float *a, const float *b, float *out, void *out16, int64_t n, int dtype) {
+    EW_PRECHECK("mg_tk_add16", a && b && out && out16 && count_ok(n) && dtype_ok(dtype));
+    if (n % 4 == 0 && aligned16(a, b, out) && aligned8(out16))
+        hipLaunchKernelGGL(k_add16_v4, dim3(blocks_for(n / 4)), dim3(256), 0, ctx_stream(ctx), a, b, out, (uint16_t *)out16,
+                           n / 4, dtype);
+    else
+        hipLaunchKernelGGL(k_add16, dim3(blocks_for(n)), dim3(256), 0, ctx_stream(ctx), a, b, out, (uint16_t *)out16, n, dtype);
+    EW_POSTCHECK("mg_tk_add16");
 }
 
 int mg_tk_add_bias(mg_ctx *ctx, float *x, const float *bias, int64_t n, int64_t ncol) {

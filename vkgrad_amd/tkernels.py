@@ -112,6 +112,8 @@ def make_transformer_kernels(dev, dtype="f16"):
     # buffers: acc, bias, res, out ; args: D
     add("residual", lambda lib, ctx, p, n, D: lib.mg_tk_residual(ctx, p[0], p[1], p[2], p[3], n, int(D)))
     add("add", lambda lib, ctx, p, n: lib.mg_tk_add(ctx, p[0], p[1], p[2], n))
+    # buffers: a, b, out, out16 ; out = a + b and its 16-bit copy
+    add("add16", lambda lib, ctx, p, n: lib.mg_tk_add16(ctx, p[0], p[1], p[2], p[3], n, dt))
     add("add_bias", lambda lib, ctx, p, n, ncol: lib.mg_tk_add_bias(ctx, p[0], p[1], n, int(ncol)))
     add("to16", lambda lib, ctx, p, n: lib.mg_ew_cast16(ctx, p[0], p[1], n, dt))
     # softmax + cross-entropy over wide rows (the LM head; kernels.py:766-823) — same buffers and

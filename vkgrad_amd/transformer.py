@@ -288,6 +288,7 @@ class Block:
         self.z1, self.h16, self.dh16 = _f32(ctx, R, 4 * D), _h16(ctx, R, 4 * D), _h16(ctx, R, 4 * D)
         self.dres1, self.dx = _f32(ctx, R, D), _f32(ctx, R, D)
         self.attn16, self.mlp16 = _h16(ctx, R, D), _h16(ctx, R, D)
+        self.dx16 = _h16(ctx, R, D) if ctx.fuse else None
         self.x32 = None
 
     # -- forward -----------------------------------------------------------
@@ -319,22 +320,31 @@ class Block:
         return self.res2
 
     # -- backward ----------------------------------------------------------
-    def backward(self, d32, graph=None):
-        """d32 = dLoss/d res2.  A residual passes its gradient to both of its inputs, so each
-        sublayer's input gradient is the incoming one plus what comes back through the branch."""
+    def backward(self, d32, graph=None, d16=None):
+        """d32 = dLoss/d res2 (d16: its 16-bit copy, if the caller has one).  A residual passes
+        its gradient to both of its inputs, so each sublayer's input gradient is the incoming one
+        plus what comes back through the branch.  In a fused context the sums leave their `add`
+        together with the 16-bit copy the next GEMMs read (`self.dx16` for the block below)."""
         ctx, TK, n = self.ctx, self.ctx.TK, self.rows * self.D
-        TK["to16"]([d32, self.mlp16], n, graph=graph)
+        if d16 is None:
+            d16 = self.mlp16
+            TK["to16"]([d32, d16], n, graph=graph)
         if ctx.fuse:
-            self.fc2.backward(self.mlp16, graph=graph, act_grad="gelu_grad", z=self.z1, dz16=self.dh16)
+            self.fc2.backward(d16, graph=graph, act_grad="gelu_grad", z=self.z1, dz16=self.dh16)
         else:
-            dh32 = self.fc2.backward(self.mlp16, graph=graph)
+            dh32 = self.fc2.backward(d16, graph=graph)
             ctx.K["bias_gelu_bwd16"]([dh32, self.z1, self.dh16], self.rows * 4 * self.D, graph=graph)
         through_mlp = self.ln2.backward(self.fc1.backward(self.dh16, graph=graph), graph=graph)
-        TK["add"]([d32, through_mlp, self.dres1], n, graph=graph)
-
-        TK["to16"]([self.dres1, self.attn16], n, graph=graph)
+        if ctx.fuse:
+            TK["add16"]([d32, through_mlp, self.dres1, self.attn16], n, graph=graph)
+        else:
+            TK["add"]([d32, through_mlp, self.dres1], n, graph=graph)
+            TK["to16"]([self.dres1, self.attn16], n, graph=graph)
         through_attn = self.ln1.backward(self.attn.backward(self.attn16, graph=graph), graph=graph)
-        TK["add"]([self.dres1, through_attn, self.dx], n, graph=graph)
+        if ctx.fuse:
+            TK["add16"]([self.dres1, through_attn, self.dx, self.dx16], n, graph=graph)
+        else:
+            TK["add"]([self.dres1, through_attn, self.dx], n, graph=graph)
         return self.dx
 
     def params(self):
@@ -447,8 +457,10 @@ class GPT:
             # instead of one small launch in front of each sum
             self.ctx.clear_grads([p for p in self.params() if len(p.shape) == 1], graph=stage(L + 1))
         d = self.lnf.backward(self._head_backward(stage(L + 1)), graph=stage(L + 1))
+        d16 = None
         for k, blk in enumerate(reversed(self.blocks)):
-            d = blk.backward(d, graph=stage(L + 2 + k))
+            d = blk.backward(d, graph=stage(L + 2 + k), d16=d16)
+            d16 = blk.dx16
         self.ctx._cleared.clear()   # later recordings clear for themselves again
         last = stage(2 * L + 2)
         TK["col_sum_zero"]([self.pos.g32], self.pos.n, graph=last)
