@@ -49,6 +49,30 @@ def gemm_list():
 
 LAYOUT_FLAGS = {"NN": (False, False), "NT": (False, True), "TN": (True, False)}
 
+
+def head_pitch(dense_head=False):
+    """Row pitch of logits / dlogits: the next multiple of 64 elements, as any allocator of a
+    (rows x vocab) tensor would give it (the reference pads the vocabulary itself,
+    transformer.py:258), or exactly VOCAB with dense_head (rows then start at odd addresses)."""
+    return VOCAB if dense_head else (VOCAB + 63) // 64 * 64
+
+
+def pitches_for(name, vpitch):
+    """Non-default row pitches of one GEMM of gemm_list(): the LM head's logits (C of the
+    forward product) and dlogits (A of dX and dW) have pitch vpitch."""
+    if not name.startswith("head") or vpitch == VOCAB:
+        return {}
+    return {"ldc": vpitch} if name.endswith(".fwd") else {"lda": vpitch}
+
+
+def plan_for(dev, name, layout, m, n, k, vpitch):
+    """(Matmul, pitches) exactly as the timed step builds them: the tuned table's plan for
+    the shape (tile, K split, band, split mode), the library's picker where it has none."""
+    from vkgrad_amd.kernels import tuned_matmul
+    ta, tb = LAYOUT_FLAGS[layout]
+    kw = pitches_for(name, vpitch)
+    return tuned_matmul(dev, m, n, k, ta, tb, DTYPE, **kw)[0], kw
+
 # HBM-side bytes per launch (L2 fetches + L2 write-backs) of each GEMM of the step,
 # measured on MI355X with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over
 # `bench.py --pmc-pass`, each counter scaled by what it reads for the cast kernel of
@@ -123,12 +147,48 @@ def cpu_baseline(min_seconds=10.0):
                       f"of bf16-rounded operands, {secs:.1f} s of matmul time"}
 
 
+def other_workloads(dev):
+    """Compact figures for the workloads the headline does not cover (the reference's
+    bench/matmul_sweep.py:60-107 writes one record with every size): the largest square
+    of configs[1] in the three layouts, one optimiser step of the d_model-1024 decoder of
+    configs[3] (every distinct GEMM timed, weighted by its count), and the two skinniest
+    memory-bound cases of configs[4].  Median of 3 batches of >= 10 ms each per GEMM."""
+    from vkgrad_amd import sweep
+    r = sweep.Runner(dev=dev, warm=False)
+    out = {}
+    sq = {}
+    for c in sweep.cases_for("square"):
+        if c["m"] == 8192:
+            row = r.time_case(c, samples=3, min_seconds=0.01)
+            sq[c["layout"]] = {"tflops": row["tflops"], "frac_mfma": row["frac_mfma"], "us": row["us"], "tile": row["tile"]}
+    out["square_8192_f16"] = sq
+    rows = [r.time_case(c, samples=3, min_seconds=0.01) for c in sweep.cases_for("decoder")]
+    us = sum(x["us"] * x["count"] for x in rows)
+    fl = sum(2.0 * x["m"] * x["n"] * x["k"] * x["count"] for x in rows)
+    out["decoder_1024_optimiser_step_bf16"] = {
+        "gemms": sum(x["count"] for x in rows), "tflop": round(fl / 1e12, 2), "gemm_ms": round(us / 1e3, 2),
+        "tflops": round(fl / us / 1e6, 1), "frac_mfma": round(fl / us / 1e6 / PEAK_TFLOPS, 4),
+        "dw": "beta = 1 over 4 micro-batches (the first overwrites)"}
+    sk = {}
+    for c in sweep.cases_for("skinny"):
+        if c["n"] == VOCAB and c["m"] in (1, 7):
+            row = r.time_case(c, samples=3, min_seconds=0.01)
+            sk[f"{c['m']}x{c['n']}x{c['k']}"] = {"us": row["us"], "gbps": row["gbps"], "frac_hbm": row["frac_hbm"],
+                                                 "tile": row["tile"]}
+    out["skinny_nt_bias_f16"] = sk
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="skip the dense-head step and the other workloads (square, decoder, skinny)")
+    ap.add_argument("--warm-seconds", type=float, default=2.0,
+                    help="sustained GEMM load before anything is timed (kernels.py:353-381)")
     ap.add_argument("--eager", action="store_true", help="enqueue GEMMs one by one instead of replaying a graph")
     ap.add_argument("--overlap-dw", action="store_true",
                     help="forward pass, then the backward pass with the dW GEMMs of the layers on the library's "
@@ -146,7 +206,7 @@ def main():
         sys.exit("bench.py: this build measures one GPU only (the path has no multi-GPU part); run with --gpus 1")
 
     from vkgrad_amd.vk import Device
-    from vkgrad_amd.kernels import Matmul, lookup_tuned
+    from vkgrad_amd.kernels import warmup
 
     dev = Device()
     rng = np.random.default_rng(1)
@@ -168,50 +228,45 @@ def main():
             bufs[name] = dict(x=x, w=w, dy=dy, y=dev.buffer(ROWS * fout * 4, "device"),
                               dx=dev.buffer(ROWS * fin * 4, "device"), dw=dev.buffer(fout * fin * 4, "device"))
         sets.append(bufs)
-    # logits / dlogits: N = 50257 columns are computed and counted; their row pitch is padded
-    # to a multiple of 64 elements unless --dense-head, as any allocator of a (rows x vocab)
-    # tensor would (the reference pads the vocabulary itself, transformer.py:258)
-    vpitch = VOCAB if args.dense_head else (VOCAB + 63) // 64 * 64
+    # logits / dlogits: N = 50257 columns are computed and counted; see head_pitch()
+    vpitch = head_pitch(args.dense_head)
+    vmax = head_pitch(False)
     head = dict(x=dev.buffer(ROWS * D * 2, "device"), w=dev.buffer(VOCAB * D * 2, "device"),
-                dy=dev.buffer(ROWS * vpitch * 2, "device"), y=dev.buffer(ROWS * vpitch * 4, "device"),
+                dy=dev.buffer(ROWS * vmax * 2, "device"), y=dev.buffer(ROWS * vmax * 4, "device"),
                 dx=dev.buffer(ROWS * D * 4, "device"), dw=dev.buffer(VOCAB * D * 4, "device"))
     fill_bf16(dev, head["x"], ROWS * D, rng, 1.0)
     fill_bf16(dev, head["w"], VOCAB * D, rng, 0.02)
-    fill_bf16(dev, head["dy"], ROWS * vpitch, rng, 1.0)
+    fill_bf16(dev, head["dy"], ROWS * vmax, rng, 1.0)
 
     mms = {}
 
-    def mm_for(layout, m, n, k, **pitch):
-        key = (layout, m, n, k)
+    def mm_for(name, layout, m, n, k, vp):
+        kw = pitches_for(name, vp)
+        key = (layout, m, n, k, tuple(sorted(kw.items())))
         if key not in mms:
-            ta, tb = LAYOUT_FLAGS[layout]
-            e = lookup_tuned(dev.name, m, n, k, ta, tb, DTYPE, **pitch)
-            if e is not None:
-                mms[key] = Matmul(dev, trans_a=ta, trans_b=tb, dtype=DTYPE, tile=e["tile_id"],
-                                  split_k=e.get("split_k", 0), group_m=e.get("group_m", 0),
-                                  atomic_split=e.get("atomic_split", False))
-            else:
-                mms[key] = Matmul(dev, trans_a=ta, trans_b=tb, dtype=DTYPE)
-        return mms[key]
+            mms[key] = plan_for(dev, name, layout, m, n, k, vp)[0]
+        return mms[key], kw
 
-    def linear_calls(b, fin, fout, rows=ROWS, ypitch=None):
-        """The three GEMMs of one linear: (mm, a, b, c, m, n, k, pitches).  ypitch is the
-        row pitch of the (rows x fout) tensors y and dy when it is not fout."""
-        yp = {} if ypitch is None else {"ldc": ypitch}
-        dp = {} if ypitch is None else {"lda": ypitch}
-        return [
-            (mm_for("NT", rows, fout, fin, **yp), b["x"], b["w"], b["y"], rows, fout, fin, yp),
-            (mm_for("NN", rows, fin, fout, **dp), b["dy"], b["w"], b["dx"], rows, fin, fout, dp),
-            (mm_for("TN", fout, fin, rows, **dp), b["dy"], b["x"], b["dw"], fout, fin, rows, dp),
-        ]
+    role_bufs = {"fwd": ("x", "w", "y"), "dX": ("dy", "w", "dx"), "dW": ("dy", "x", "dw")}
 
-    calls = []
-    for layer in range(LAYERS):
-        b = sets[layer % NSET]
-        for name, fin, fout in LINEARS:
-            calls += linear_calls(b[name], fin, fout)
-    head_calls = linear_calls(head, D, VOCAB, ypitch=vpitch)
-    calls += head_calls
+    def step_calls(vp):
+        """Every GEMM of one step in order: (mm, a, b, c, m, n, k, pitches)."""
+        shapes = {nm: (lay, m, n, k) for nm, lay, m, n, k, _ in gemm_list()}
+        calls = []
+        for layer in range(LAYERS):
+            b = sets[layer % NSET]
+            for name, _, _ in LINEARS:
+                for role in ("fwd", "dX", "dW"):
+                    lay, m, n, k = shapes[f"{name}.{role}"]
+                    mm, kw = mm_for(f"{name}.{role}", lay, m, n, k, vp)
+                    calls.append((mm,) + tuple(b[name][x] for x in role_bufs[role]) + (m, n, k, kw))
+        for role in ("fwd", "dX", "dW"):
+            lay, m, n, k = shapes[f"head.{role}"]
+            mm, kw = mm_for(f"head.{role}", lay, m, n, k, vp)
+            calls.append((mm,) + tuple(head[x] for x in role_bufs[role]) + (m, n, k, kw))
+        return calls
+
+    calls = step_calls(vpitch)
     step_flops = sum(2.0 * c[4] * c[5] * c[6] for c in calls)
 
     if args.pmc_pass:
@@ -241,23 +296,18 @@ def main():
         dev.destroy()
         return
 
-    # Order of one step.  Default: forward, dX, dW of each linear in turn, every GEMM
-    # behind the previous one.
-    # --overlap-dw: the forward pass (layer 0 .. 11, LM head), then the backward pass from
-    # the head down; dW of a linear depends on nothing that follows it
-    # (autograd.py:218-227), so the dW GEMMs of a layer go to the library's second stream
-    # once that layer's dX chain is done and overlap the next layer's dX chain; the
-    # streams join at the end of the step.
-    # schedule entries: ("gemm", call, on_side_stream) | ("fork",) | ("join",)
-    per_linear = [calls[i:i + 3] for i in range(0, len(calls), 3)]     # (fwd, dX, dW) per linear, head last
-    if not args.overlap_dw:
-        schedule = [("gemm", c, False) for c in calls]
-    else:
+    def schedule_of(calls):
+        """Order of one step.  Default: forward, dX, dW of each linear in turn, every GEMM
+        behind the previous one.  --overlap-dw: the forward pass (layer 0 .. 11, LM head), then
+        the backward pass from the head down; dW of a linear depends on nothing that follows it
+        (autograd.py:218-227), so the dW GEMMs of a layer go to the library's second stream once
+        that layer's dX chain is done and overlap the next layer's dX chain; the streams join at
+        the end of the step.  Entries: ("gemm", call, on_side_stream) | ("fork",) | ("join",)"""
+        if not args.overlap_dw:
+            return [("gemm", c, False) for c in calls]
+        per_linear = [calls[i:i + 3] for i in range(0, len(calls), 3)]     # (fwd, dX, dW) per linear, head last
         schedule = [("gemm", fwd, False) for fwd, _, _ in per_linear]
-        # backward: groups of linears from the top down (the LM head, then layer 11 .. 0);
-        # the dW GEMMs of a group go to the side stream when the group's dX chain is done
-        # (all their operands are complete then) and run beside the next group's dX chain
-        # (the LM head's two products stay on the main stream: each fills the chip with
+        # (the LM head's two backward products stay on the main stream: each fills the chip with
         # resident workgroups and two such kernels only take CUs from each other)
         schedule += [("gemm", per_linear[-1][1], False), ("gemm", per_linear[-1][2], False)]
         groups = [per_linear[l * len(LINEARS):(l + 1) * len(LINEARS)][::-1] for l in reversed(range(LAYERS))]
@@ -266,20 +316,11 @@ def main():
             schedule.append(("fork",))
             schedule += [("gemm", dw, True) for _, _, dw in g]
         schedule.append(("join",))
+        return schedule
 
-    if args.eager:
-        def run_step():
-            for item in schedule:
-                if item[0] == "fork":
-                    dev.side_fork()
-                elif item[0] == "join":
-                    dev.side_join()
-                else:
-                    mm, a, b, c, m, n, k, kw = item[1]
-                    mm.enqueue(a, b, c, m, n, k, side=item[2], **kw)
-    else:
-        graph = dev.graph("gpt2_small_gemms")
-        for item in schedule:
+    def record(calls, name):
+        graph = dev.graph(name)
+        for item in schedule_of(calls):
             if item[0] == "fork":
                 graph.fork()
             elif item[0] == "join":
@@ -287,19 +328,45 @@ def main():
             else:
                 mm, a, b, c, m, n, k, kw = item[1]
                 mm(a, b, c, m, n, k, graph=graph, side=item[2], **kw)
-        graph.finish()
+        return graph.finish()
 
-        def run_step():
+    def run_eager(calls):
+        for item in schedule_of(calls):
+            if item[0] == "fork":
+                dev.side_fork()
+            elif item[0] == "join":
+                dev.side_join()
+            else:
+                mm, a, b, c, m, n, k, kw = item[1]
+                mm.enqueue(a, b, c, m, n, k, side=item[2], **kw)
+
+    def time_steps(calls, name, steps, nwarm):
+        """nwarm untimed steps, then `steps` timed ones: host wall clock around all of them
+        (synchronised on both sides) and, for a graph, device time of each replay."""
+        if args.eager:
+            for _ in range(nwarm):
+                run_eager(calls)
+            dev.sync()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                run_eager(calls)
+            dev.sync()
+            return time.perf_counter() - t0, None
+        graph = record(calls, name)
+        for _ in range(nwarm):
             graph.enqueue()
+        dev.sync()
+        t0 = time.perf_counter()
+        each = graph.time(steps)
+        dev.sync()
+        wall = time.perf_counter() - t0
+        graph.destroy()
+        return wall, each
 
-    for _ in range(args.warmup):
-        run_step()
-    dev.sync()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run_step()
-    dev.sync()
-    dt = time.perf_counter() - t0
+    # Sustained load first: the chip's clock under matrix load settles over milliseconds, and the
+    # first kernels after an idle period run at a different clock than a training loop sees.
+    warm_s = warmup(dev, args.warm_seconds, force=True) if args.warm_seconds > 0 else 0.0
+    dt, each = time_steps(calls, "gpt2_small_gemms", args.steps, args.warmup)
     ms_per_step = dt / args.steps * 1e3
     tflops = step_flops / (dt / args.steps) / 1e12
 
@@ -309,15 +376,11 @@ def main():
     # it does inside the step.
     per_shape = []
     for name, layout, m, n, k, count in gemm_list():
-        mm = mm_for(layout, m, n, k)
+        mm, kw = mm_for(name, layout, m, n, k, vpitch)
         is_head = name.startswith("head")
-        role = name.split(".")[1]
-        pick = {"fwd": ("x", "w", "y"), "dX": ("dy", "w", "dx"), "dW": ("dy", "x", "dw")}[role]
-        groups = [head] if is_head else [s[name.split(".")[0]] for s in sets]
-        rot = [tuple(g[x] for x in pick) for g in groups]
-        kw = {}
-        if is_head and vpitch != VOCAB:
-            kw = {"ldc": vpitch} if role == "fwd" else {"lda": vpitch}
+        lin, role = name.split(".")
+        groups = [head] if is_head else [s[lin] for s in sets]
+        rot = [tuple(g[x] for x in role_bufs[role]) for g in groups]
         t1 = mm.time_rotating(rot, m, n, k, repeat=len(rot), **kw) / len(rot)
         rep = max(1, int(0.02 / max(t1, 1e-6)) // len(rot)) * len(rot)
         sec = min(mm.time_rotating(rot, m, n, k, repeat=rep, **kw) / rep for _ in range(3))
@@ -354,12 +417,25 @@ def main():
                             "forward pass, then backward pass with the layers' dW GEMMs on a second stream "
                             "beside the next layer's dX chain (joined at the end)"},
         "frac_of_mfma_peak": round(tflops / PEAK_TFLOPS, 4),
+        "sustained_warmup_s": round(warm_s, 2),
         "sum_of_event_timed_gemms_ms": round(events_ms, 4),
         "roofline": roofline,
         "device": {"name": dev.name, "compute_units": dev.compute_units, "clock_khz": dev.clock_khz,
                    "derived_peak_tflops": round(dev.compute_units * 4 * 1024 * dev.clock_khz * 1e3 / 1e12, 1)},
         "per_shape": per_shape,
     }
+    if each is not None:
+        ev = sorted(x * 1e3 for x in each)
+        out["ms_per_step_events"] = {"median": round(ev[len(ev) // 2], 4), "min": round(ev[0], 4), "max": round(ev[-1], 4),
+                                     "what": "device time of each timed replay, HIP events on the library's stream"}
+    if not args.no_extra:
+        if not args.dense_head and not args.eager:
+            # the same step with logits / dlogits rows exactly 50257 elements apart
+            dcalls = step_calls(VOCAB)
+            ddt, deach = time_steps(dcalls, "gpt2_small_gemms_dense_head", args.steps, args.warmup)
+            out["dense_head"] = {"logits_row_pitch": VOCAB, "value": round(step_flops / (ddt / args.steps) / 1e12, 2),
+                                 "unit": "TFLOP/s", "ms_per_step": round(ddt / args.steps * 1e3, 4)}
+        out["other_workloads"] = other_workloads(dev)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     else:

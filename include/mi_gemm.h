@@ -256,6 +256,10 @@ int mg_graph_launch(mg_ctx *ctx, mg_graph *g, double *seconds);
 /* Graph.submit without the fence wait (vk.py:1295 `wait=False` is the eager analogue):
  * replay on the context's stream and return; mg_sync waits for it. */
 int mg_graph_enqueue(mg_ctx *ctx, mg_graph *g);
+/* Replays the graph `repeat` (1..4096) times back to back with a HIP event between
+ * replays and waits; seconds_each[i] = device time of replay i.  The reference times a
+ * recorded step by host wall clock around submit (vk.py:877-889, bench/ab.py:36-51). */
+int mg_graph_time(mg_ctx *ctx, mg_graph *g, int repeat, double *seconds_each);
 int mg_graph_destroy(mg_ctx *ctx, mg_graph *g);
 
 /* ---- companion elementwise kernels: kernels.make_kernels (kernels.py:699-862) ----

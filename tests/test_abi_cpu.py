@@ -339,3 +339,52 @@ def test_sweep_workloads_match_the_stated_configurations():
     one = next(c for c in sk if (c["m"], c["n"]) == (1, 50257))
     assert algorithmic_bytes(one) == 2 * (768 + 768 * 50257) + 4 * 50257 + 4 * 50257
     assert len(cases_for("charlm")) == 15
+
+
+def test_documented_ctypes_stub_matches_the_binding():
+    """INTEGRATION.md shows a maintainer the ctypes struct to bind mg_gemm_args with; the library
+    rejects any other struct_size, so the documented definition must stay the real one."""
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    start = text.index("class GemmArgs(C.Structure):")
+    end = text.index("\n\n", start)
+    ns = {"C": C}
+    exec(text[start:end], ns)   # the class statement only
+    doc = ns["GemmArgs"]
+    assert C.sizeof(doc) == C.sizeof(L.GemmArgs)
+    assert [f[0] for f in doc._fields_] == [f[0] for f in L.GemmArgs._fields_]
+    for name, ctype in L.GemmArgs._fields_:
+        assert getattr(doc, name).offset == getattr(L.GemmArgs, name).offset, name
+        assert getattr(doc, name).size == getattr(L.GemmArgs, name).size, name
+    # and the call the document shows passes validation
+    m, n, k = 96, 64, 128
+    args = doc(struct_size=C.sizeof(doc), layout=2, dtype=1, beta=1, m=m, n=n, k=k, a=0x1000, lda=m, b=0x2000, ldb=n,
+               c=0x3000, ldc=n, nbatch=1, tile=-1)
+    lib = L.load()
+    assert lib.mg_gemm_check(C.cast(C.byref(args), C.POINTER(L.GemmArgs))) == L.MG_OK, L.last_error()
+
+
+def test_graph_refuses_replay_after_a_buffer_was_destroyed():
+    """A finished graph has device addresses baked in; replaying it on freed memory must
+    be refused on the host (no device needed: the check precedes the library call)."""
+    from vkgrad_amd.vk import Graph, VkError
+
+    class FakeBuf:
+        def __init__(self):
+            self.ptr, self.size = 0x1000, 64
+
+    class FakeDev:
+        _graphs = set()
+    g = Graph(FakeDev(), "g")
+    b = FakeBuf()
+    g.record(lambda: None, [b], name="k")
+    g._finished, g._handle = True, object()
+    b.ptr = None
+    with pytest.raises(VkError, match="destroyed"):
+        g.submit()
+    with pytest.raises(VkError, match="destroyed"):
+        g.enqueue()
+    dead = FakeBuf()
+    dead.ptr = None
+    g2 = Graph(FakeDev(), "g2")
+    with pytest.raises(VkError, match="destroyed"):
+        g2.record(lambda: None, [dead], name="k")

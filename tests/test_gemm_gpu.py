@@ -552,6 +552,33 @@ def test_triangular_structure_of_causal_attention(dev, dtype):
         buf.destroy()
 
 
+@pytest.mark.parametrize("tile", [None, 4, 11, 14])
+def test_triangular_a_with_bias_and_atomic_k_split(dev, tile):
+    """op(A) upper triangular (TN, A stored lower triangular), a bias, and K slices that add
+    into C atomically: for the lower row blocks slice 0 - the one that carries the bias - has
+    an empty K range, and must still add the bias."""
+    from vkgrad_amd.kernels import Matmul
+    m, n, k = 512, 64, 512
+    a, b = O.make_operands(m, n, k, True, False, "bf16", seed=21, integer=True)
+    a[~np.tril(np.ones((k, m), bool))] = 0
+    bias = (np.arange(n, dtype=np.float32) % 9) - 4
+    ref = O.ref_gemm(a, b, True, False, "bf16", bias, None)
+    for split, atomic in ((4, True), (4, False), (3, True)):
+        ba, bb, bc, bz = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), \
+            dev.buffer(m * n * 4, "device"), dev.buffer(n * 4, "device")
+        ba.upload(a); bb.upload(b); bz.upload(bias)
+        bc.upload(np.full((m, n), np.nan, np.float32))
+        mm = Matmul(dev, trans_a=True, dtype="bf16", tile=tile, split_k=split, atomic_split=atomic)
+        try:
+            mm(ba, bb, bc, m, n, k, bias=bz, tri="a_upper")
+            got = bc.download(np.float32, (m, n))
+            assert np.array_equal(got, ref), (tile, split, atomic, int((got != ref).sum()))
+        finally:
+            mm.destroy()
+            for x in (ba, bb, bc, bz):
+                x.destroy()
+
+
 def test_timing_over_rotating_operand_sets(dev):
     """The rotating timer launches argument set i % nsets on launch i: after seven
     launches over three sets with different integer operands, every set's C holds

@@ -385,12 +385,20 @@ def _relerr(got, want):
     return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-8))
 
 
-def _check_model(dev, B, T, D, H, L, vocab, tie, fuse, dtype, packed=False, staged=False):
+def _check_model(dev, B, T, D, H, L, vocab, tie, fuse, dtype, packed=False, staged=False, one_kernel=None,
+                 replay_other_first=False):
+    """one_kernel: assert that Attention took (True) or did not take (False) its one-kernel
+    P and dS paths.  replay_other_first: the recorded graphs are first replayed on another
+    batch (other tokens, another packing), then on the batch that is checked - what the
+    first replay left in P, dS and the gradient buffers must not show."""
     from vkgrad_amd.transformer import GPT, TCtx
     rows = B * T
     ctx = TCtx(dev, dtype=dtype, fuse=fuse)
     try:
         model = GPT(ctx, B, T, D, H, L, vocab, tie=tie)
+        if one_kernel is not None:
+            for blk in model.blocks:
+                assert blk.attn._one_kernel_p == one_kernel and blk.attn._one_kernel_ds == one_kernel
         rng = np.random.default_rng(0)
         ids = rng.integers(0, vocab, rows).astype(np.uint32)
         tgt = rng.integers(0, vocab, rows).astype(np.uint32)
@@ -423,6 +431,26 @@ def _check_model(dev, B, T, D, H, L, vocab, tie, fuse, dtype, packed=False, stag
             assert sorted(graphs) == list(range(model.n_stages()))
         for s in sorted(graphs):
             graphs[s].finish()
+        if replay_other_first:
+            ro = np.random.default_rng(7)
+            idb.array(np.uint32, (rows,))[:] = ro.integers(0, vocab, rows)
+            tgb.array(np.uint32, (rows,))[:] = ro.integers(0, vocab, rows)
+            if packed:
+                other = np.zeros(rows, np.uint32)
+                for b in range(B):
+                    cut = int(ro.integers(T // 4, 3 * T // 4))
+                    other[b * T + cut:(b + 1) * T] = cut
+                segb.array(np.uint32, (rows,))[:] = other
+                wb.array(np.float32, (rows,))[:] = ro.uniform(0.5, 2.0, rows)
+            for s in sorted(graphs):
+                graphs[s].submit()
+            dev.sync()
+            idb.array(np.uint32, (rows,))[:] = ids
+            tgb.array(np.uint32, (rows,))[:] = tgt
+            if packed:
+                segb.array(np.uint32, (rows,))[:] = seg
+                wb.array(np.float32, (rows,))[:] = weights
+        for s in sorted(graphs):
             graphs[s].submit()
         dev.sync()
         model.loss.invalidate()
@@ -459,6 +487,33 @@ def test_gpt_bf16_ragged_dimensions(dev):
     """bf16 operands, and sizes that are multiples of nothing (T = 19, hd = 9 -> D = 27,
     vocabulary 21): no padding is needed anywhere but the logits' pitch."""
     _check_model(dev, 2, 19, 27, 3, 1, 21, True, True, "bf16")
+
+
+def test_gpt_one_kernel_attention_paths(dev):
+    """Head width 32: Attention takes mg_tk_attn_p and mg_tk_attn_ds (one kernel each for
+    P and dS, half-size P / dS buffers cleared once at construction, the row term from
+    attn_rowdot, and dQ / dK / dV GEMMs that read the never-written zero region above the
+    diagonal) - the path a GPT-2-small step runs."""
+    _check_model(dev, 2, 72, 64, 2, 2, 16, True, True, "f16", one_kernel=True)
+
+
+def test_gpt_one_kernel_attention_long_rows(dev):
+    """Head width 64, T = 264 > 256: wavefronts of attn_p with no key to see and key blocks
+    that attn_ds skips occur; bf16."""
+    _check_model(dev, 1, 264, 128, 2, 1, 32, True, True, "bf16", one_kernel=True)
+
+
+def test_gpt_one_kernel_attention_packed_replayed_twice(dev):
+    """Packed samples, loss weights and one graph per stage through the one-kernel paths;
+    every graph is first replayed on another batch with another packing, then on the one
+    that is checked: entries of P and dS that the first packing filled and the second masks
+    must come back as zeros, and no gradient may carry over."""
+    _check_model(dev, 2, 72, 64, 2, 2, 16, True, True, "f16", packed=True, staged=True, one_kernel=True,
+                 replay_other_first=True)
+
+
+def test_gpt_small_heads_do_not_take_the_one_kernel_paths(dev):
+    _check_model(dev, 2, 16, 32, 2, 1, 16, True, True, "f16", one_kernel=False)
 
 
 @pytest.mark.parametrize("fuse", [False, True])

@@ -217,7 +217,8 @@ gemm_dma_kernel(const GemmParams p) {
     int kbeg = blockIdx.y * p.k_per_split;
     int kend = min(p.K, kbeg + p.k_per_split);
     tri_k_range<BM, BK>(p.tri, m0, kbeg, kend);
-    if (kend == kbeg && p.split_k > 1 && p.ws == nullptr) return;   // an empty slice has nothing to add to C
+    // an empty slice has nothing to add to C, except the bias when it is the slice that carries it
+    if (kend == kbeg && p.split_k > 1 && p.ws == nullptr && !(p.bias != nullptr && blockIdx.y == 0)) return;
     const int krem = (kend - kbeg) % BK;          // K remainder, multiplied first
     const int kdma = kbeg + krem;                 // the ring covers [kdma, kend)
     const int nkb = (kend - kdma) / BK;

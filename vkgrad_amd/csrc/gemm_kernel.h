@@ -295,7 +295,7 @@ __device__ __forceinline__ bool splitk_gather(f32x16 (&acc)[TM][TN], float *ws, 
     const bool last = *flag != 0;
     __syncthreads();      // flag may be reused (persistent kernel) once everyone has read it
     if (!last) return false;
-    if (tid == 0) *counter = 0;   // ready for the next launch
+    if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -563,7 +563,8 @@ gemm_kernel(const GemmParams p) {
     int kbeg = blockIdx.y * p.k_per_split;
     int kend = min(p.K, kbeg + p.k_per_split);
     tri_k_range<BM, BK>(p.tri, m0, kbeg, kend);
-    if (kend == kbeg && p.split_k > 1 && p.ws == nullptr) return;   // an empty slice has nothing to add to C
+    // an empty slice has nothing to add to C, except the bias when it is the slice that carries it
+    if (kend == kbeg && p.split_k > 1 && p.ws == nullptr && !(p.bias != nullptr && blockIdx.y == 0)) return;
     const int nkb = (kend - kbeg + BK - 1) / BK;
     // K-blocks that the unconditional loader may fetch: the whole block inside
     // K, and the tile inside M and N.

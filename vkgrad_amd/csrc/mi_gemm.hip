@@ -740,17 +740,40 @@ int mg_pick(const mg_gemm_args *args, int compute_units, int *tile, int *split_k
     return MG_OK;
 }
 
-static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
-    const mg_gemm_args &a = *args;
-    const TileDesc &t = g_tiles[pl.tile];
-    // the stream this GEMM runs on, and that stream's half of the split-K workspace
+// Where a GEMM runs and what it may use there: a stream, that stream's share of the split-K
+// workspace (partial tiles and per-tile arrival counters), and the limits of the device.
+struct Lane {
+    hipStream_t stream;
+    float *ws;            // NULL: no workspace, K slices add into C with atomics
+    int64_t ws_bytes;
+    int *cnt;
+    int64_t max_tiles;    // arrival counters available
+    int cus;
+    int lds_limit;        // LDS bytes a workgroup may use
+};
+
+static int lane_of(mg_ctx *ctx, const mg_gemm_args &a, Lane &ln) {
     const bool on_side = (a.flags & MG_FLAG_SIDE_STREAM) != 0;
-    hipStream_t stream = on_side ? ctx->side : ctx->stream;
-    const int64_t lane_bytes = ctx->ws_bytes / 2;
-    float *lane_ws = ctx->ws ? ctx->ws + (on_side ? lane_bytes / (int64_t)sizeof(float) : 0) : nullptr;
-    int *lane_cnt = ctx->cnt ? ctx->cnt + (on_side ? MG_MAX_COUNTED_TILES : 0) : nullptr;
     if (on_side && !ctx->side_forked)
         return fail(MG_ERR_STATE, "mg_gemm: MG_FLAG_SIDE_STREAM needs mg_side_fork first");
+    // the stream this GEMM runs on, and that stream's half of the split-K workspace
+    ln.stream = on_side ? ctx->side : ctx->stream;
+    ln.ws_bytes = ctx->ws_bytes / 2;
+    ln.ws = ctx->ws ? ctx->ws + (on_side ? ln.ws_bytes / (int64_t)sizeof(float) : 0) : nullptr;
+    ln.cnt = ctx->cnt ? ctx->cnt + (on_side ? MG_MAX_COUNTED_TILES : 0) : nullptr;
+    ln.max_tiles = MG_MAX_COUNTED_TILES;
+    ln.cus = ctx->prop.multiProcessorCount;
+    ln.lds_limit = (int)ctx->prop.maxSharedMemoryPerMultiProcessor;
+    return MG_OK;
+}
+
+static int enqueue_gemm(const Lane &ln, const mg_gemm_args *args, const Plan &pl) {
+    const mg_gemm_args &a = *args;
+    const TileDesc &t = g_tiles[pl.tile];
+    hipStream_t stream = ln.stream;
+    const int64_t lane_bytes = ln.ws_bytes;
+    float *lane_ws = ln.ws;
+    int *lane_cnt = ln.cnt;
     GemmParams p;
     p.A = (const uint16_t *)a.a;
     p.B = (const uint16_t *)a.b;
@@ -787,7 +810,7 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
         if (e != hipSuccess) return hip_fail(e, "mg_gemm: kernel launch");
         return MG_OK;
     }
-    if (lds_bytes_for(t, a.layout) > (int)ctx->prop.maxSharedMemoryPerMultiProcessor)
+    if (lds_bytes_for(t, a.layout) > ln.lds_limit)
         return fail(MG_ERR_ARG, "mg_gemm: tile %d needs %d bytes of LDS", pl.tile, lds_bytes_for(t, a.layout));
     p.Y = (uint16_t *)a.y16;
     p.ldy = a.ldy;
@@ -812,7 +835,7 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
         // partial tiles go through the workspace when they fit
         const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n * a.nbatch;
         const int64_t need = tiles * pl.split_k * t.bm * t.bn * (int64_t)sizeof(float);
-        if (lane_ws && need <= lane_bytes && tiles <= MG_MAX_COUNTED_TILES && !(a.flags & MG_FLAG_SPLITK_ATOMIC)) {
+        if (lane_ws && need <= lane_bytes && tiles <= ln.max_tiles && !(a.flags & MG_FLAG_SPLITK_ATOMIC)) {
             p.ws = lane_ws;
             p.cnt = lane_cnt;
         }
@@ -822,8 +845,8 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
             mg_gemm_args whole = a;
             whole.split_k = 1;
             Plan unsplit;
-            pick_plan(whole, ctx->prop.multiProcessorCount, unsplit);
-            return enqueue_gemm(ctx, &whole, unsplit);
+            pick_plan(whole, ln.cus, unsplit);
+            return enqueue_gemm(ln, &whole, unsplit);
         }
     }
     if (pl.split_k > 1 && a.beta == 0 && p.ws == nullptr) {
@@ -850,7 +873,7 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
         // resident workgroups loop over (slice, tile) units; [1] = epilogue with bias
         general = a.bias != nullptr ? 1 : 0;
         const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n;
-        const int64_t slots = (int64_t)ctx->prop.multiProcessorCount * wgs_per_cu(t, a.layout);
+        const int64_t slots = (int64_t)ln.cus * wgs_per_cu(t, a.layout);
         // stream-K cuts tiles only when the batches together leave resident slots idle: every batch
         // (one grid.z slice) is partitioned by itself, over its share of the slots
         const int64_t slots_z = slots / a.nbatch > 0 ? slots / a.nbatch : 1;
@@ -861,7 +884,7 @@ static int enqueue_gemm(mg_ctx *ctx, const mg_gemm_args *args, const Plan &pl) {
             const int64_t need = (int64_t)sk.pieces * sk.rem_tiles * a.nbatch * t.bm * t.bn * (int64_t)sizeof(float);
             if (sk.pieces == 1) {
                 g = tiles < slots ? tiles : slots;   // nothing to cut
-            } else if (lane_ws && need <= lane_bytes && tiles * a.nbatch <= MG_MAX_COUNTED_TILES) {
+            } else if (lane_ws && need <= lane_bytes && tiles * a.nbatch <= ln.max_tiles) {
                 p.stream_k = 1;
                 p.sk_full_rounds = sk.full_rounds;
                 p.sk_rem_tiles = sk.rem_tiles;
@@ -886,9 +909,12 @@ int mg_gemm(mg_ctx *ctx, const mg_gemm_args *args) {
     if (!ctx) return fail(MG_ERR_ARG, "mg_gemm: ctx is NULL");
     int rc = check_args(args);
     if (rc != MG_OK) return rc;
+    Lane ln;
+    rc = lane_of(ctx, *args, ln);
+    if (rc != MG_OK) return rc;
     Plan pl;
-    pick_plan(*args, ctx->prop.multiProcessorCount, pl);
-    return enqueue_gemm(ctx, args, pl);
+    pick_plan(*args, ln.cus, pl);
+    return enqueue_gemm(ln, args, pl);
 }
 
 int mg_gemm_time(mg_ctx *ctx, const mg_gemm_args *args, int repeat, double *seconds) {
@@ -898,11 +924,14 @@ int mg_gemm_time(mg_ctx *ctx, const mg_gemm_args *args, int repeat, double *seco
     int rc = check_args(args);
     if (rc != MG_OK) return rc;
     if (args->flags & MG_FLAG_SIDE_STREAM) return fail(MG_ERR_ARG, "mg_gemm_time: timing runs on the main stream");
+    Lane ln;
+    rc = lane_of(ctx, *args, ln);
+    if (rc != MG_OK) return rc;
     Plan pl;
-    pick_plan(*args, ctx->prop.multiProcessorCount, pl);
+    pick_plan(*args, ln.cus, pl);
     HIP_TRY(hipEventRecord(ctx->ev0, ctx->stream));
     for (int i = 0; i < repeat; i++) {
-        rc = enqueue_gemm(ctx, args, pl);
+        rc = enqueue_gemm(ln, args, pl);
         if (rc != MG_OK) return rc;
     }
     HIP_TRY(hipEventRecord(ctx->ev1, ctx->stream));
@@ -927,9 +956,14 @@ int mg_gemm_time_rotating(mg_ctx *ctx, const mg_gemm_args *args, int nargs, int 
             return fail(MG_ERR_ARG, "mg_gemm_time_rotating: timing runs on the main stream");
         pick_plan(args[i], ctx->prop.multiProcessorCount, pl[i]);
     }
+    Lane ln;
+    {
+        int rc = lane_of(ctx, args[0], ln);
+        if (rc != MG_OK) return rc;
+    }
     HIP_TRY(hipEventRecord(ctx->ev0, ctx->stream));
     for (int i = 0; i < repeat; i++) {
-        int rc = enqueue_gemm(ctx, &args[i % nargs], pl[i % nargs]);
+        int rc = enqueue_gemm(ln, &args[i % nargs], pl[i % nargs]);
         if (rc != MG_OK) return rc;
     }
     HIP_TRY(hipEventRecord(ctx->ev1, ctx->stream));
@@ -1004,6 +1038,41 @@ int mg_graph_enqueue(mg_ctx *ctx, mg_graph *g) {
     if (ctx->capturing) return fail(MG_ERR_STATE, "mg_graph_enqueue: a graph is being recorded");
     HIP_TRY(hipGraphLaunch(g->exec, ctx->stream));
     return MG_OK;
+}
+
+int mg_graph_time(mg_ctx *ctx, mg_graph *g, int repeat, double *seconds_each) {
+    if (!ctx || !g || !seconds_each) return fail(MG_ERR_ARG, "mg_graph_time: NULL argument");
+    if (repeat < 1 || repeat > 4096) return fail(MG_ERR_ARG, "mg_graph_time: repeat must be 1..4096");
+    if (ctx->capturing) return fail(MG_ERR_STATE, "mg_graph_time: a graph is being recorded");
+    HIP_TRY(hipSetDevice(ctx->device));
+    hipEvent_t *ev = new (std::nothrow) hipEvent_t[repeat + 1]();
+    if (!ev) return fail(MG_ERR_NOMEM, "mg_graph_time: out of host memory");
+    int rc = MG_OK;
+    int made = 0;
+    for (; made <= repeat; made++) {
+        hipError_t e = hipEventCreate(&ev[made]);
+        if (e != hipSuccess) {
+            rc = hip_fail(e, "mg_graph_time: hipEventCreate");
+            break;
+        }
+    }
+    if (rc == MG_OK) {
+        hipError_t e = hipEventRecord(ev[0], ctx->stream);
+        for (int i = 0; i < repeat && e == hipSuccess; i++) {
+            e = hipGraphLaunch(g->exec, ctx->stream);
+            if (e == hipSuccess) e = hipEventRecord(ev[i + 1], ctx->stream);
+        }
+        if (e == hipSuccess) e = hipEventSynchronize(ev[repeat]);
+        for (int i = 0; i < repeat && e == hipSuccess; i++) {
+            float ms = 0.f;
+            e = hipEventElapsedTime(&ms, ev[i], ev[i + 1]);
+            seconds_each[i] = (double)ms * 1e-3;
+        }
+        if (e != hipSuccess) rc = hip_fail(e, "mg_graph_time");
+    }
+    for (int i = 0; i < made; i++) (void)hipEventDestroy(ev[i]);
+    delete[] ev;
+    return rc;
 }
 
 int mg_graph_destroy(mg_ctx *ctx, mg_graph *g) {

@@ -232,7 +232,7 @@ class Matmul:
             def launch(ga=ga):
                 _check(lib.mg_gemm(ctx, C.byref(ga)), self.name)
 
-            graph.record(launch, [x for x in (a, b, c, y16, z, colsum, res, p16, rowsub) if x is not None], name=self.name,
+            graph.record(launch, [x for x in (a, b, c, bias, y16, z, colsum, res, p16, rowsub) if x is not None], name=self.name,
                          bytes_hint=self.traffic_bytes(m, n, k, nbatch))
             nb_ = nbatch if self.batched else 1
             graph.mm_split.append((nb_ * 2 * (m * k + k * n), nb_ * m * n * 4))
@@ -348,6 +348,21 @@ def lookup_tuned(dev_name, m, n, k, trans_a, trans_b, dtype="f16", batched=False
         if e is not None:
             return e
     return None
+
+
+def tuned_matmul(dev, m, n, k, trans_a=False, trans_b=False, dtype="f16", batched=False, nbatch=1,
+                 accumulate=False, lda=None, ldb=None, ldc=None):
+    """(Matmul, how) for one shape as the benchmarks run it: the cached pick (tile,
+    K split, rasterisation band, split mode) when a cache holds the shape, else a
+    Matmul that leaves the choice to the library's picker.  how is 'tuned table' or
+    'picker'.  The parity tests build their GEMMs through this same function, so what
+    is timed is what is checked."""
+    e = lookup_tuned(dev.name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate, lda, ldb, ldc)
+    if e is None:
+        return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, dtype=dtype), "picker"
+    return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, dtype=dtype, tile=e["tile_id"],
+                  split_k=e.get("split_k", 0), group_m=e.get("group_m", 0),
+                  atomic_split=e.get("atomic_split", False)), "tuned table"
 
 
 _WARMED = set()

@@ -87,11 +87,11 @@ def algorithmic_bytes(c):
 
 
 class Runner:
-    def __init__(self, tune=False, warm=True):
+    def __init__(self, tune=False, warm=True, dev=None):
         from . import kernels
         from .vk import Device
         self.K = kernels
-        self.dev = Device()
+        self.dev = dev if dev is not None else Device()
         self.tune = tune
         self.fill = {}
         if warm:
@@ -105,18 +105,13 @@ class Runner:
     def matmul_for(self, c):
         K, dev = self.K, self.dev
         ta, tb = LAYOUT_FLAGS[c["layout"]]
-        how = "tuned table"
-        e = K.lookup_tuned(dev.name, c["m"], c["n"], c["k"], ta, tb, c["dtype"], accumulate=c["accumulate"],
-                           **c["pitch"])
-        if e is None and self.tune:
+        if self.tune and K.lookup_tuned(dev.name, c["m"], c["n"], c["k"], ta, tb, c["dtype"],
+                                        accumulate=c["accumulate"], **c["pitch"]) is None:
             mm, e = K.autotune_matmul(dev, c["m"], c["n"], c["k"], ta, tb, dtype=c["dtype"],
                                       accumulate=c["accumulate"], **c["pitch"])
-            mm.destroy()
-            how = "tuned now"
-        if e is None:
-            return K.Matmul(dev, trans_a=ta, trans_b=tb, dtype=c["dtype"]), "picker"
-        return K.Matmul(dev, trans_a=ta, trans_b=tb, dtype=c["dtype"], tile=e["tile_id"], split_k=e.get("split_k", 0),
-                        group_m=e.get("group_m", 0), atomic_split=e.get("atomic_split", False)), how
+            return mm, "tuned now"
+        return K.tuned_matmul(dev, c["m"], c["n"], c["k"], ta, tb, c["dtype"], accumulate=c["accumulate"],
+                              **c["pitch"])
 
     def allocate(self, c, nsets):
         dev = self.dev

@@ -99,6 +99,7 @@ class Graph:
         self._handle = None
         self.traffic = []
         self.mm_split = []
+        self._buffers = {}   # id -> every buffer a recorded launch names: its address is baked into the graph
 
     def record(self, launch, buffers=(), name="kernel", bytes_hint=None):
         """launch: zero-argument callable that enqueues work on the device
@@ -108,6 +109,10 @@ class Graph:
         if not callable(launch):
             raise VkError(f"{self.name}: record() needs a callable launch")
         self._thunks.append(launch)
+        for b in buffers:
+            if b.ptr is None:
+                raise VkError(f"{self.name}: {name} names a destroyed buffer")
+            self._buffers[id(b)] = b
         compulsory = sum(b.size for b in buffers)
         self.traffic.append((name, compulsory, compulsory if bytes_hint is None else bytes_hint))
         self.n_dispatch += 1
@@ -152,18 +157,35 @@ class Graph:
         self.dev._graphs.add(self)
         return self
 
-    def submit(self):
+    def _check_alive(self, what):
+        """A finished graph holds raw device addresses: replaying it after one of its
+        buffers was destroyed would run kernels on freed memory."""
         if not self._finished:
-            raise VkError(f"{self.name}: call finish() before submit()")
+            raise VkError(f"{self.name}: call finish() before {what}()")
+        if self._handle is None:
+            raise VkError(f"{self.name}: {what}() on a destroyed graph")
+        for b in self._buffers.values():
+            if b.ptr is None:
+                raise VkError(f"{self.name}: {what}() after a buffer of {b.size} bytes it uses was destroyed")
+
+    def submit(self):
+        self._check_alive("submit")
         dt = C.c_double()
         _check(self.dev._lib.mg_graph_launch(self.dev._ctx, self._handle, C.byref(dt)), f"{self.name}: submit")
         return dt.value
 
     def enqueue(self):
         """Replay without waiting; the stream keeps order with later work."""
-        if not self._finished:
-            raise VkError(f"{self.name}: call finish() before enqueue()")
+        self._check_alive("enqueue")
         _check(self.dev._lib.mg_graph_enqueue(self.dev._ctx, self._handle), f"{self.name}: enqueue")
+
+    def time(self, repeat=1):
+        """Replay `repeat` times back to back; device seconds of each replay (HIP events
+        on the context's stream)."""
+        self._check_alive("time")
+        out = (C.c_double * int(repeat))()
+        _check(self.dev._lib.mg_graph_time(self.dev._ctx, self._handle, int(repeat), out), f"{self.name}: time")
+        return list(out)
 
     def destroy(self):
         if self._handle is not None:
