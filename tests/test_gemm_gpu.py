@@ -177,7 +177,7 @@ def test_split_k_clear_respects_pitch_and_tails(dev, tile):
         assert r["exact"], f"tile {tile} n {n} ldc {ldc}: max diff {np.abs(got - ref).max()}"
 
 
-@pytest.mark.parametrize("tile", [0, 10, 15, 17])
+@pytest.mark.parametrize("tile", [0, 10, 15, 17, 21])
 def test_split_k_is_bit_reproducible(dev, tile):
     """The K slices meet in a workspace and are summed in slice order by whichever
     slice arrives last, so random data gives the same bits on every run."""
@@ -274,7 +274,7 @@ def test_fused_activation_output(dev, layout, dtype):
     np16 = np.float16 if dtype == "f16" else np.uint16
     cases = [(200, 136, 320, None, 0, "gelu"), (512, 384, 256, 11, 0, "relu"), (1000, 1016, 1024, 10, 0, "gelu"),
              (392, 648, 2048, 11, 4, None), (129, 96, 768, 4, 3, "relu"), (300, 200, 264, 15, 0, "gelu"),
-             (64, 50, 72, 20, 0, "relu")]
+             (64, 50, 72, 20, 0, "relu"), (520, 776, 1024, 21, 0, "gelu"), (512, 264, 2048, 21, 3, "relu")]
     for m, n, k, tile, split, act in cases:
         a, b = O.make_operands(m, n, k, ta, tb, dtype, seed=m + k, integer=True)
         bias = (np.arange(n) % 9 - 4).astype(np.float32) * 0.5
@@ -577,6 +577,92 @@ def test_triangular_a_with_bias_and_atomic_k_split(dev, tile):
             mm.destroy()
             for x in (ba, bb, bc, bz):
                 x.destroy()
+
+
+@pytest.mark.parametrize("layout", list(LAYOUTS))
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_ping_pong_tile(dev, layout, dtype):
+    """The ping-pong tile (two wavefront groups half a K-block apart, three operand tiles per
+    ring stage, loads addressed by a scalar base): integer data, so every case is exact.
+    Shapes where a half tile of A lies wholly or partly beyond M, ragged N and K (the K
+    remainder goes through registers), one to five K-blocks (prologue and tail branches of
+    the load schedule), padded pitches, bias, beta = 1, K splits both ways, batches, and
+    the causal forms."""
+    from vkgrad_amd.kernels import CONFIGS, Matmul
+    pp = next(t["id"] for t in CONFIGS if t["name"].startswith("mmq_"))
+    ta, tb = LAYOUTS[layout]
+    shapes = [(256, 256, 64), (256, 256, 128), (256, 256, 192), (512, 512, 320), (100, 256, 256), (130, 300, 264),
+              (257, 8, 72), (384, 520, 200), (1000, 264, 1032), (777, 1031, 136), (640, 768, 4096)]
+    for m, n, k in shapes:
+        if layout == "TN":
+            m = max(8, m)
+        r, got, ref = check_case(dev, m, n, k, ta, tb, dtype, seed=m + n + k, integer=True, tile=pp, bias=(k % 128 == 0),
+                                 accumulate=(m % 2 == 1))
+        assert r["exact"], f"{layout} {dtype} {m}x{n}x{k}: {int((got != ref).sum())} entries differ"
+    # padded pitches (the padding holds NaN) and K splits through the workspace and with atomics
+    r, got, ref = check_case(dev, 300, 520, 1024, ta, tb, dtype, seed=5, integer=True, tile=pp, split_k=4, bias=True,
+                             lda=(304 if ta else 1032), ldb=(1032 if tb else 528), ldc=536)
+    assert r["exact"]
+    mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype=dtype, tile=pp, split_k=3, atomic_split=True)
+    a, b = O.make_operands(264, 392, 1536, ta, tb, dtype, seed=6, integer=True)
+    ba, bb, bc = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), dev.buffer(264 * 392 * 4, "device")
+    try:
+        ba.upload(a); bb.upload(b)
+        bc.upload(np.full((264, 392), np.nan, np.float32))
+        mm(ba, bb, bc, 264, 392, 1536)
+        assert np.array_equal(bc.download(np.float32, (264, 392)), O.ref_gemm(a, b, ta, tb, dtype))
+        assert mm.plan(264, 392, 1536)[0] == pp
+    finally:
+        mm.destroy()
+        for x in (ba, bb, bc):
+            x.destroy()
+    # random data within the tolerances
+    r, _, _ = check_case(dev, 1024, 768, 1536, ta, tb, dtype, seed=12, bias=True, tile=pp)
+    _assert_close(r, f"ping-pong {layout} {dtype}")
+
+
+def test_ping_pong_tile_batched_and_causal(dev):
+    """Strided batches and the causal forms on the ping-pong tile (integer data, exact)."""
+    from vkgrad_amd.kernels import CONFIGS, Matmul
+    pp = next(t["id"] for t in CONFIGS if t["name"].startswith("mmq_"))
+
+    def run(layout, m, n, k, nb, a, b, tri=None):
+        ta, tb = LAYOUTS[layout]
+        ba, bb, bc = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), dev.buffer(nb * m * n * 4, "device")
+        ba.upload(a); bb.upload(b)
+        bc.upload(np.full((nb, m, n), np.nan, np.float32))
+        mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype="bf16", tile=pp, batched=True)
+        try:
+            mm(ba, bb, bc, m, n, k, nbatch=nb, strides=(a[0].size, b[0].size, m * n), tri=tri)
+            assert mm.plan(m, n, k, nbatch=nb)[0] == pp
+            return bc.download(np.float32, (nb, m, n))
+        finally:
+            mm.destroy()
+            for x in (ba, bb, bc):
+                x.destroy()
+
+    def operands(layout, m, n, k, nb, seed):
+        ta, tb = LAYOUTS[layout]
+        pairs = [O.make_operands(m, n, k, ta, tb, "bf16", seed=seed + i, integer=True) for i in range(nb)]
+        return np.stack([p[0] for p in pairs]), np.stack([p[1] for p in pairs])
+
+    def product(layout, a, b):
+        ta, tb = LAYOUTS[layout]
+        return np.stack([O.ref_gemm(a[i], b[i], ta, tb, "bf16") for i in range(a.shape[0])])
+
+    a, b = operands("NT", 520, 520, 128, 3, 1)
+    got = run("NT", 520, 520, 128, 3, a, b, tri="c_lower")
+    low = np.tril(np.ones((520, 520), bool))
+    assert np.array_equal(got[:, low], product("NT", a, b)[:, low])
+    assert np.isnan(got[:, :256, 256:512]).all(), "a tile wholly above the diagonal was written"
+    a, b = operands("NN", 768, 64, 768, 2, 2)
+    a[:, ~np.tril(np.ones((768, 768), bool))] = 0
+    assert np.array_equal(run("NN", 768, 64, 768, 2, a, b, tri="a_lower"), product("NN", a, b))
+    a, b = operands("TN", 768, 72, 768, 2, 3)
+    a[:, ~np.tril(np.ones((768, 768), bool))] = 0
+    assert np.array_equal(run("TN", 768, 72, 768, 2, a, b, tri="a_upper"), product("TN", a, b))
+    a, b = operands("NN", 300, 264, 200, 4, 4)
+    assert np.array_equal(run("NN", 300, 264, 200, 4, a, b), product("NN", a, b))
 
 
 def test_timing_over_rotating_operand_sets(dev):

@@ -3,8 +3,9 @@
 // for direct-to-LDS tiles, which fall back to a register-staged tile instead).
 // Persistent and stream-K tiles use [0] for the plain epilogue and [1] for the one with bias.
 // Entry [tile][2] is the variant whose epilogue also writes the activated 16-bit output
-// (forward layouts NN and NT, tiles 3, 4, 10 and 11; null elsewhere).
+// (forward layouts NN and NT, tiles 3, 4, 10, 11 and 21; null elsewhere).
 #include "gemm_dma_kernel.h"
+#include "gemm_pp_kernel.h"
 #include "gemm_kernel.h"
 #include "tiles.h"
 
@@ -19,6 +20,11 @@ constexpr launch_fn act_variant_d() {
     if constexpr ((ID == 10 || ID == 11) && L_NN != L_TN) return launch_gemm_dma<L_NN, D_BF16, BM, BN, BK, WGM, WGN, NS, true>;
     else return nullptr;
 }
+template <int BM, int BN, int BK, int WGM, int WGN>
+constexpr launch_fn act_variant_q() {
+    if constexpr (L_NN != L_TN) return launch_gemm_pp<L_NN, D_BF16, BM, BN, BK, WGM, WGN, true>;
+    else return nullptr;
+}
 #define V(id, bm, bn, bk, wgm, wgn) \
     {launch_gemm<L_NN, D_BF16, bm, bn, bk, wgm, wgn, false>, launch_gemm<L_NN, D_BF16, bm, bn, bk, wgm, wgn, true>, \
      act_variant_v<id, bm, bn, bk, wgm, wgn>()},
@@ -28,13 +34,16 @@ constexpr launch_fn act_variant_d() {
     {launch_gemm_dmap<L_NN, D_BF16, bm, bn, bk, wgm, wgn, ns, false, false>, \
      launch_gemm_dmap<L_NN, D_BF16, bm, bn, bk, wgm, wgn, ns, true, false>, nullptr},
 #define G(id, bm, bn, bk, fb) {nullptr, nullptr, nullptr},   // launched through gemv_table
+#define Q(id, bm, bn, bk, wgm, wgn, ns, fb) \
+    {launch_gemm_pp<L_NN, D_BF16, bm, bn, bk, wgm, wgn>, nullptr, act_variant_q<bm, bn, bk, wgm, wgn>()},
 #define S(id, bm, bn, bk, wgm, wgn, ns, fb)                                \
     {launch_gemm_dmap<L_NN, D_BF16, bm, bn, bk, wgm, wgn, ns, false, true>, \
      launch_gemm_dmap<L_NN, D_BF16, bm, bn, bk, wgm, wgn, ns, true, true>, nullptr},
-launch_fn launch_table_nn_bf16[MG_NUM_TILES][3] = {MG_TILE_LIST(V, D, P, S, G)};
+launch_fn launch_table_nn_bf16[MG_NUM_TILES][3] = {MG_TILE_LIST(V, D, P, S, G, Q)};
 #undef V
 #undef D
 #undef P
 #undef S
 #undef G
+#undef Q
 }  // namespace mg

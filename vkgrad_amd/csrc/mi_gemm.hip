@@ -48,18 +48,21 @@ struct TileDesc {
     int fallback;   // tile of the same BM x BN with weaker preconditions (self: none)
     int persistent; // 1: grid of resident workgroups looping over tiles; 2: the same with stream-K balancing
     int gemv;       // 1: the skinny-M streaming kernel (no matrix cores), NT layout only
+    int pingpong;   // 1: the two wavefronts of a SIMD alternate between LDS reads and MFMAs (gemm_pp_kernel.h)
 };
-#define V(id, bm, bn, bk, wgm, wgn) {id, bm, bn, bk, wgm, wgn, 0, id, 0, 0},
-#define D(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 0, 0},
-#define P(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 1, 0},
-#define S(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 2, 0},
-#define G(id, bm, bn, bk, fb) {id, bm, bn, bk, 1, GEMV_WAVES, 0, fb, 0, 1},
-static const TileDesc g_tiles[MG_NUM_TILES] = {MG_TILE_LIST(V, D, P, S, G)};
+#define V(id, bm, bn, bk, wgm, wgn) {id, bm, bn, bk, wgm, wgn, 0, id, 0, 0, 0},
+#define D(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 0, 0, 0},
+#define P(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 1, 0, 0},
+#define S(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 2, 0, 0},
+#define G(id, bm, bn, bk, fb) {id, bm, bn, bk, 1, GEMV_WAVES, 0, fb, 0, 1, 0},
+#define Q(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 0, 0, 1},
+static const TileDesc g_tiles[MG_NUM_TILES] = {MG_TILE_LIST(V, D, P, S, G, Q)};
 #undef V
 #undef D
 #undef P
 #undef S
 #undef G
+#undef Q
 
 static thread_local char g_err[512] = "";
 
@@ -198,6 +201,7 @@ static const float g_cost[MG_NUM_TILES][3][2] = {
     {{4.81f, 2.006f}, {7.24f, 1.819f}, {3.05f, 2.002f}},   // 18 mmk_256x256x64_w2x4_s2
     {{5.52f, 0.907f}, {4.46f, 0.944f}, {3.88f, 1.003f}},   // 19 mmk_128x128x64_w2x2_s2
     {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}},                     // 20 mv_4x64x512 (priced by bytes, see plan_cost_us)
+    {{5.69f, 1.230f}, {13.28f, 1.060f}, {4.76f, 1.200f}},   // 21 mmq_256x256x64_w2x4_s2 (tile 10's overhead, its own K-block time)
 };
 
 static int wgs_per_cu(const TileDesc &t, int layout) {
@@ -711,7 +715,8 @@ int mg_tile_info(int id, mg_tile *out) {
         snprintf(out->name, sizeof(out->name), "%s_%dx%dx%d_w%dx%d_s%d", t.persistent == 2 ? "mmk" : "mmp", t.bm, t.bn, t.bk,
                  t.wgm, t.wgn, t.nstage);
     else if (t.nstage > 0)
-        snprintf(out->name, sizeof(out->name), "mmd_%dx%dx%d_w%dx%d_s%d", t.bm, t.bn, t.bk, t.wgm, t.wgn, t.nstage);
+        snprintf(out->name, sizeof(out->name), "%s_%dx%dx%d_w%dx%d_s%d", t.pingpong ? "mmq" : "mmd", t.bm, t.bn, t.bk, t.wgm,
+                 t.wgn, t.nstage);
     else
         snprintf(out->name, sizeof(out->name), "mm_%dx%dx%d_w%dx%d", t.bm, t.bn, t.bk, t.wgm, t.wgn);
     out->stages = t.nstage;

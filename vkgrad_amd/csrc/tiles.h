@@ -20,10 +20,13 @@
 //     G(id, BM, BN, BK, fallback_id) — BM rows of A at most, BN output columns per
 //     workgroup, BK elements of K per register chunk; falls back to a skinny
 //     register-staged tile.
+//   ping-pong direct-to-LDS (gemm_pp_kernel.h): the preconditions of the direct-to-LDS tiles;
+//     the two wavefronts of a SIMD alternate between reading operands and multiplying.
+//     Q(id, BM, BN, BK, WGM, WGN, NSTAGE, fallback_id)
 // WGM x WGN wavefronts of 64 lanes per workgroup.
 #pragma once
 
-#define MG_TILE_LIST(V, D, P, S, G) \
+#define MG_TILE_LIST(V, D, P, S, G, Q) \
     V(0, 256, 256, 64, 2, 2)       \
     V(1, 256, 128, 64, 2, 2)       \
     V(2, 128, 256, 64, 2, 2)       \
@@ -44,6 +47,7 @@
     P(17, 128, 128, 64, 2, 2, 2, 11) \
     S(18, 256, 256, 64, 2, 4, 2, 15) \
     S(19, 128, 128, 64, 2, 2, 2, 17) \
-    G(20, 4, 64, 512, 4)
+    G(20, 4, 64, 512, 4) \
+    Q(21, 256, 256, 64, 2, 4, 2, 10)
 
-#define MG_NUM_TILES 21
+#define MG_NUM_TILES 22
