@@ -219,6 +219,21 @@ int mg_gemm_time(mg_ctx *ctx, const mg_gemm_args *args, int repeat, double *seco
  * reference times a shape on one set of buffers (kernels.py:433-447), which on
  * this chip would time small shapes out of cache. */
 int mg_gemm_time_rotating(mg_ctx *ctx, const mg_gemm_args *args, int nargs, int repeat, double *seconds);
+/* No counterpart in the reference.  mg_gemm for callers that cannot allocate device memory or
+ * create a context: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  Same arguments and results as mg_gemm (bit-identical: the same kernels and plans),
+ * on device `device_index` and on `hip_stream` (a hipStream_t, NULL for the default stream),
+ * which the caller owns and synchronises.  It calls no hipMalloc / hipFree and needs no mg_ctx:
+ * the K slices of a split meet in a workspace that is part of the library's image on every
+ * device, MG_STATIC_WS_BYTES of partial tiles and MG_STATIC_MAX_TILES arrival counters, which
+ * each GPU holds until the process ends.  A GEMM whose K split needs more than that is refused
+ * with MG_ERR_ARG (nothing is launched); MG_FLAG_SPLITK_ATOMIC, split_k = 1 or mg_gemm are the
+ * ways out.  MG_FLAG_SIDE_STREAM is refused.  All calls on one GPU share the one workspace:
+ * calls that may overlap on a GPU (two streams, two threads) race on it - keep them on one
+ * stream or give every concurrent caller but one split_k = 1. */
+#define MG_STATIC_WS_BYTES (32ll << 20)
+#define MG_STATIC_MAX_TILES 16384
+int mg_gemm_static(int device_index, void *hip_stream, const mg_gemm_args *args);
 /* CONFIGS — kernels.py:326-331: the tile table the tuner walks. */
 int mg_tile_count(void);
 int mg_tile_info(int id, mg_tile *out);

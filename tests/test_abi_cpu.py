@@ -363,6 +363,15 @@ def test_documented_ctypes_stub_matches_the_binding():
     assert lib.mg_gemm_check(C.cast(C.byref(args), C.POINTER(L.GemmArgs))) == L.MG_OK, L.last_error()
 
 
+def test_static_entry_point_validates_before_touching_a_device(lib):
+    """mg_gemm_static runs the same argument checks first, so its refusals are testable here."""
+    assert lib.mg_gemm_static(0, None, None) == L.MG_ERR_ARG
+    ga = good_args(k=-1)
+    assert lib.mg_gemm_static(0, None, C.byref(ga)) == L.MG_ERR_ARG and "positive" in L.last_error()
+    ga = good_args(flags=L.MG_FLAG_SIDE_STREAM)
+    assert lib.mg_gemm_static(0, None, C.byref(ga)) == L.MG_ERR_ARG and "SIDE_STREAM" in L.last_error()
+
+
 def test_graph_refuses_replay_after_a_buffer_was_destroyed():
     """A finished graph has device addresses baked in; replaying it on freed memory must
     be refused on the host (no device needed: the check precedes the library call)."""

@@ -14,6 +14,8 @@ MG_ACT_NONE, MG_ACT_GELU, MG_ACT_RELU = 0, 1, 2
 MG_FLAG_TIGHT_BUFFERS = 1
 MG_FLAG_SPLITK_ATOMIC = 2
 MG_FLAG_SIDE_STREAM = 4
+MG_STATIC_WS_BYTES = 32 << 20
+MG_STATIC_MAX_TILES = 16384
 
 DTYPES = {"f16": MG_F16, "bf16": MG_BF16}
 KINDS = {"device": MG_DEVICE, "shared": MG_SHARED, "cached": MG_CACHED, "bar": MG_BAR}
@@ -83,6 +85,7 @@ SIGNATURES = {
     "mg_last_error": (C.c_char_p, []),
     "mg_gemm_check": (C.c_int, [C.POINTER(GemmArgs)]),
     "mg_gemm": (C.c_int, [_P, C.POINTER(GemmArgs)]),
+    "mg_gemm_static": (C.c_int, [C.c_int, _P, C.POINTER(GemmArgs)]),
     "mg_side_fork": (C.c_int, [_P]),
     "mg_side_join": (C.c_int, [_P]),
     "mg_gemm_time": (C.c_int, [_P, C.POINTER(GemmArgs), C.c_int, C.POINTER(C.c_double)]),

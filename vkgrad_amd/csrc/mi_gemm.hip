@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 
 #include "gemm_kernel.h"
@@ -1087,6 +1088,125 @@ int mg_graph_destroy(mg_ctx *ctx, mg_graph *g) {
     (void)hipGraphDestroy(g->graph);
     delete g;
     return MG_OK;
+}
+
+// ---------------------------------------------------------------------------
+// mg_gemm_static: the GEMM for callers that cannot allocate.  Its K slices meet in
+// a workspace that is part of the library's image on every device instead of a
+// hipMalloc'ed one: `scratch` holds MG_STATIC_WS_BYTES of partial tiles followed by
+// MG_STATIC_MAX_TILES arrival counters.  In host code that name is a stand-in, not a
+// device address: each device's copy is looked up with hipGetSymbolAddress, once per
+// device with that device current, and only the pointer it returns is handed to kernels.
+// ---------------------------------------------------------------------------
+}  // extern "C"
+
+static __device__ __align__(256) unsigned char scratch[MG_STATIC_WS_BYTES + MG_STATIC_MAX_TILES * sizeof(int)];
+
+namespace mg {
+__global__ void zero_ints_kernel(int *p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+struct StaticLane {
+    std::atomic<int> ready{0};   // 0: not looked up, 1: ready
+    float *ws = nullptr;
+    int *cnt = nullptr;
+    int cus = 0;
+    int lds_limit = 0;
+    char arch_ok = 0;
+};
+static const int MG_MAX_DEVICES = 64;
+static StaticLane g_static[MG_MAX_DEVICES];
+static std::mutex g_static_mu;
+
+// Looks up this device's copies of the static arrays (with that device current).
+static int static_lane(int device, StaticLane **out) {
+    if (device < 0 || device >= MG_MAX_DEVICES)
+        return fail(MG_ERR_ARG, "mg_gemm_static: device index %d out of range [0, %d)", device, MG_MAX_DEVICES);
+    StaticLane &sl = g_static[device];
+    if (!sl.ready.load(std::memory_order_acquire)) {
+        std::lock_guard<std::mutex> lock(g_static_mu);
+        if (!sl.ready.load(std::memory_order_relaxed)) {
+            void *ptr = nullptr;
+            HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+            int cus = 0, lds = 0;
+            HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+            HIP_TRY(hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, device));
+            hipDeviceProp_t prop;
+            HIP_TRY(hipGetDeviceProperties(&prop, device));
+            sl.arch_ok = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+            sl.ws = (float *)ptr;
+            sl.cnt = (int *)((unsigned char *)ptr + MG_STATIC_WS_BYTES);
+            sl.cus = cus;
+            sl.lds_limit = lds;
+            sl.ready.store(1, std::memory_order_release);
+        }
+    }
+    if (!sl.arch_ok) return fail(MG_ERR_NODEVICE, "mg_gemm_static: device %d is not gfx950", device);
+    *out = &sl;
+    return MG_OK;
+}
+}  // namespace mg
+
+extern "C" {
+
+int mg_gemm_static(int device_index, void *hip_stream, const mg_gemm_args *args) {
+    int rc = check_args(args);
+    if (rc != MG_OK) return rc;
+    if (args->flags & MG_FLAG_SIDE_STREAM)
+        return fail(MG_ERR_ARG, "mg_gemm_static: MG_FLAG_SIDE_STREAM belongs to a context; pass the stream itself");
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        return fail(MG_ERR_NODEVICE, "mg_gemm_static: no HIP device available");
+    }
+    if (device_index < 0 || device_index >= count)
+        return fail(MG_ERR_ARG, "mg_gemm_static: device index %d out of range [0, %d)", device_index, count);
+    HIP_TRY(hipSetDevice(device_index));
+    StaticLane *sl = nullptr;
+    rc = static_lane(device_index, &sl);
+    if (rc != MG_OK) return rc;
+    Lane ln;
+    ln.stream = (hipStream_t)hip_stream;
+    ln.ws = sl->ws;
+    ln.ws_bytes = MG_STATIC_WS_BYTES;
+    ln.cnt = sl->cnt;
+    ln.max_tiles = MG_STATIC_MAX_TILES;
+    ln.cus = sl->cus;
+    ln.lds_limit = sl->lds_limit;
+    Plan pl;
+    pick_plan(*args, ln.cus, pl);
+    const TileDesc &t = g_tiles[pl.tile];
+    // what the K slices (or stream-K pieces) of this plan need of the static workspace
+    const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n * args->nbatch;
+    int64_t need = 0, counted = 0;
+    if (pl.split_k > 1) {
+        need = tiles * pl.split_k * t.bm * t.bn * (int64_t)sizeof(float);
+        counted = tiles;
+    } else if (t.persistent == 2) {
+        const int64_t slots = (int64_t)ln.cus * wgs_per_cu(t, args->layout);
+        const int64_t slots_z = slots / args->nbatch > 0 ? slots / args->nbatch : 1;
+        const StreamK sk = stream_k_partition((int64_t)pl.grid_m * pl.grid_n, args->k / t.bk, slots_z);
+        if (sk.pieces > 1) {
+            need = (int64_t)sk.pieces * sk.rem_tiles * args->nbatch * t.bm * t.bn * (int64_t)sizeof(float);
+            counted = tiles;
+        }
+    }
+    if (!(args->flags & MG_FLAG_SPLITK_ATOMIC) && (need > MG_STATIC_WS_BYTES || counted > MG_STATIC_MAX_TILES))
+        return fail(MG_ERR_ARG,
+                    "mg_gemm_static: this GEMM's K split needs %lld bytes of partial tiles and %lld tile counters; the "
+                    "static workspace holds %lld bytes and %d counters (use mg_gemm, a smaller split_k, or "
+                    "MG_FLAG_SPLITK_ATOMIC)",
+                    (long long)need, (long long)counted, (long long)MG_STATIC_WS_BYTES, MG_STATIC_MAX_TILES);
+    if (counted > 0 && !(args->flags & MG_FLAG_SPLITK_ATOMIC)) {
+        // The array keeps what the last call left: counters must start at zero (a fill kernel, so
+        // that the sequence may be captured into a graph).
+        hipLaunchKernelGGL(zero_ints_kernel, dim3((unsigned)cdiv(counted, 256)), dim3(256), 0, ln.stream, ln.cnt,
+                           (int)counted);
+        HIP_TRY(hipGetLastError());
+    }
+    return enqueue_gemm(ln, args, pl);
 }
 
 }  // extern "C"
