@@ -173,8 +173,11 @@ struct DmaTraits {
     static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;
 };
 
-template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool ACT = false>
-__global__ void __launch_bounds__(WGM *WGN * 64)
+// MINW: wavefronts per SIMD the register allocation must leave room for (1: no constraint).
+// Eight wavefronts of 64 x 64 need fewer than 128 registers, so two such workgroups fit a CU
+// (four wavefronts per SIMD) when the compiler is told to stay below that.
+template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool ACT = false, int MINW = 1>
+__global__ void __launch_bounds__(WGM *WGN * 64, MINW)
 gemm_dma_kernel(const GemmParams p) {
     constexpr bool A_KC = (LAYOUT != L_TN);
     constexpr bool B_KC = (LAYOUT == L_NT);
@@ -685,10 +688,10 @@ gemm_dmap_kernel(const GemmParams p) {
     }
 }
 
-template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool ACT = false>
+template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool ACT = false, int MINW = 1>
 hipError_t launch_gemm_dma(const GemmParams &p, dim3 grid, hipStream_t stream) {
     using TT = DmaTraits<LAYOUT, BM, BN, BK, WGM, WGN, NSTAGE>;
-    auto kern = gemm_dma_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, NSTAGE, ACT>;
+    auto kern = gemm_dma_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, NSTAGE, ACT, MINW>;
     static std::atomic<uint64_t> lds_allowed{0};
     hipError_t e = allow_dynamic_lds((const void *)kern, TT::LDS_BYTES, lds_allowed);
     if (e != hipSuccess) return e;

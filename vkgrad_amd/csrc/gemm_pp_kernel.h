@@ -47,15 +47,6 @@
 
 namespace mg {
 
-#ifdef PP_DEBUG_CLOCKS
-__device__ unsigned long long pp_dbg[4];
-#endif
-#ifdef PP_DEBUG_PHASES
-__device__ unsigned long long pp_ph[2][8];
-#define PP_T(x) const unsigned long long x = clock64();
-#else
-#define PP_T(x)
-#endif
 
 // Where one wavefront's direct loads of an operand tile come from.
 struct PpAddr {
@@ -289,24 +280,12 @@ gemm_pp_kernel(const GemmParams p) {
     }
     __builtin_amdgcn_sched_barrier(0);
 
-#ifdef PP_DEBUG_CLOCKS
-    const unsigned long long dbg_c0 = clock64(), dbg_w0 = wall_clock64();
-#endif
-#ifdef PP_DEBUG_PHASES
-    unsigned long long ph_acc[7] = {0, 0, 0, 0, 0, 0, 0};
-#endif
     for (int i = 0; i < nkb; i++) {
-        PP_T(t0)
         // ---- MEM(i): operands of block i into registers, then the loads that refill what has
         // become free (behind the reads: a direct load is not issued while LDS reads of its
         // wavefront are outstanding, so loads between the reads only serialise the two) ----
         int newest = 0;   // loads issued in this phase
-#ifndef PP_NO_LDS
         read_block(i & 1);
-#else
-        if (i == 0) read_block(0);
-#endif
-#ifndef PP_NO_DMA
         if (grp == 0) {
             if (i >= 1 && i + 1 < nkb) {
                 issue_b((i + 1) & 1);
@@ -322,9 +301,7 @@ gemm_pp_kernel(const GemmParams p) {
                 newest = 2 * NLA;
             }
         }
-#endif
         __builtin_amdgcn_sched_barrier(0);
-        PP_T(t1)
         // Group 1: the upper half of A of block i + 1, which group 0 reads next, has landed -
         // everything older than the loads of this phase.  Group 0 has nothing to confirm here.
         if (grp == 1) {
@@ -332,45 +309,23 @@ gemm_pp_kernel(const GemmParams p) {
             else if (newest == NLA) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLA) : "memory");
             else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
-        PP_T(t2)
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
-        PP_T(t3)
         // ---- MMA(i) ----
         __builtin_amdgcn_s_setprio(1);
         mma_block();
         __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_sched_barrier(0);
-        PP_T(t4)
         // Group 0: B of block i + 1 has landed.  Group 1: the lower half of A of block i + 1, which
         // it reads itself next (every wavefront of the group reads what the others loaded); the
         // upper half of block i + 2 behind it may still be on its way.
         if (grp == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         else if (newest == 2 * NLA) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NLA) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        PP_T(t5)
         if (grp == 0 || i + 1 < nkb) asm volatile("s_barrier" ::: "memory");
-        PP_T(t6)
-#ifdef PP_DEBUG_PHASES
-        if (i > 1 && i + 2 < nkb) {
-            ph_acc[0] += t1 - t0; ph_acc[1] += t2 - t1; ph_acc[2] += t3 - t2;
-            ph_acc[3] += t4 - t3; ph_acc[4] += t5 - t4; ph_acc[5] += t6 - t5; ph_acc[6] += 1;
-        }
-#endif
         __builtin_amdgcn_sched_barrier(0);
     }
 
-#ifdef PP_DEBUG_PHASES
-    if ((tid & 255) == 0)
-        for (int q = 0; q < 7; q++) atomicAdd(&pp_ph[grp][q], ph_acc[q]);
-#endif
-#ifdef PP_DEBUG_CLOCKS
-    if (tid == 0) {
-        atomicAdd(&pp_dbg[0], clock64() - dbg_c0);
-        atomicAdd(&pp_dbg[1], wall_clock64() - dbg_w0);
-        atomicAdd(&pp_dbg[2], (unsigned long long)nkb);
-    }
-#endif
     // Epilogue: shared with the register-staged kernel (store_tile, gemm_kernel.h).
     bool add_bias = p.bias != nullptr && blockIdx.y == 0;
     int mode = p.split_k > 1 ? 2 : (p.beta ? 1 : 0);
@@ -384,14 +339,7 @@ gemm_pp_kernel(const GemmParams p) {
         add_bias = p.bias != nullptr;
         mode = p.beta ? 1 : 0;
     }
-#ifdef PP_DEBUG_CLOCKS
-    const unsigned long long dbg_e0 = clock64();
-#endif
     store_tile<DT, TM, TN, WTM, WTN, ACT>(p, C, acc, m0, n0, wave_m, wave_n, lane, add_bias, mode, interior);
-#ifdef PP_DEBUG_CLOCKS
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (tid == 0) atomicAdd(&pp_dbg[3], clock64() - dbg_e0);
-#endif
 }
 
 template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, bool ACT = false>
