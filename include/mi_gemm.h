@@ -234,6 +234,13 @@ int mg_gemm_time_rotating(mg_ctx *ctx, const mg_gemm_args *args, int nargs, int 
 #define MG_STATIC_WS_BYTES (32ll << 20)
 #define MG_STATIC_MAX_TILES 16384
 int mg_gemm_static(int device_index, void *hip_stream, const mg_gemm_args *args);
+/* What the matrix cores sustain with no memory traffic: two wavefronts per SIMD on every CU run
+ * `iters` rounds of eight back-to-back v_mfma_f32_32x32x16 from registers.  random_operands = 0
+ * multiplies zeros (the chip holds its boost clock), 1 multiplies random 16-bit values (the
+ * power-managed clock drops, and with it the rate every real GEMM is bounded by).  Returns the
+ * rate and the shader clock during the loop.  The reference's counterpart is the hand-measured
+ * WMMA peak it prices its kernels against (bench/RESULTS.md:113-119, 656-659). */
+int mg_probe_mfma(mg_ctx *ctx, int dtype, int random_operands, int iters, double *tflops, double *ghz);
 /* CONFIGS — kernels.py:326-331: the tile table the tuner walks. */
 int mg_tile_count(void);
 int mg_tile_info(int id, mg_tile *out);

@@ -334,3 +334,19 @@ def test_column_sums_and_recordable_copy(dev):
     assert dev._lib.mg_ew_copy(dev._ctx, dst.ptr, src.ptr, 6) != 0     # not a multiple of 4
     src.destroy()
     dst.destroy()
+
+
+def test_mfma_ceiling_probe(dev):
+    """mg_probe_mfma: the register-only MFMA rate, on zero and on random operands.  The rate
+    equals 2 wavefronts x 4 SIMDs x CUs x 1024 FLOP per clock at the clock it reports (the loop
+    has no other instruction), and random operands never run faster than zeros."""
+    from vkgrad_amd.probe import mfma_ceiling
+    z_tf, z_ghz = mfma_ceiling(dev, "bf16", False, seconds=0.05)
+    r_tf, r_ghz = mfma_ceiling(dev, "bf16", True, seconds=0.05)
+    for tf, ghz in ((z_tf, z_ghz), (r_tf, r_ghz)):
+        assert 0.5 < ghz < 3.5 and tf > 100.0
+        per_clock = tf * 1e12 / (ghz * 1e9) / (dev.compute_units * 4)
+        assert 0.85 * 1024 <= per_clock <= 1.02 * 1024, per_clock
+    assert r_tf <= z_tf * 1.03
+    f_tf, _ = mfma_ceiling(dev, "f16", True, seconds=0.05)
+    assert f_tf > 100.0

@@ -1,0 +1,48 @@
+"""MFMA ceiling of the device on zero and on random operands.
+
+    python -m vkgrad_amd.probe [--dtype bf16] [--seconds 0.5]
+
+Prints the rate a register-only MFMA loop sustains on every SIMD of the chip and the shader
+clock it ran at, for all-zero operands (the chip holds its boost clock) and for random ones
+(the power-managed clock drops).  GEMM throughput on real data is bounded by the second
+figure, not by the datasheet peak, which assumes the boost clock.
+"""
+
+import argparse
+import ctypes as C
+import json
+
+from . import _lib as L
+from .vk import Device, _check
+
+
+def mfma_ceiling(dev, dtype="bf16", random_operands=True, seconds=0.5):
+    """(TFLOP/s, GHz) of the register-only MFMA loop; the iteration count is scaled from a
+    short launch so that the timed one lasts about `seconds`."""
+    lib, ctx = dev._lib, dev._ctx
+    tf, ghz = C.c_double(), C.c_double()
+    iters = 20000
+    _check(lib.mg_probe_mfma(ctx, L.DTYPES[dtype], int(bool(random_operands)), iters, C.byref(tf), C.byref(ghz)), "probe")
+    per_iter = dev.compute_units * 8 * 8 * 32768.0 / (tf.value * 1e12)
+    iters = int(max(iters, min(1 << 24, seconds / per_iter)))
+    _check(lib.mg_probe_mfma(ctx, L.DTYPES[dtype], int(bool(random_operands)), iters, C.byref(tf), C.byref(ghz)), "probe")
+    return tf.value, ghz.value
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--dtype", default="bf16", choices=("f16", "bf16"))
+    ap.add_argument("--seconds", type=float, default=0.5)
+    args = ap.parse_args(argv)
+    dev = Device()
+    out = {"device": dev.name, "compute_units": dev.compute_units, "dtype": args.dtype}
+    for name, rnd in (("zeros", False), ("random", True), ("zeros_again", False), ("random_again", True)):
+        tf, ghz = mfma_ceiling(dev, args.dtype, rnd, args.seconds)
+        out[name] = {"tflops": round(tf, 1), "ghz": round(ghz, 3), "of_2500": round(tf / 2500.0, 4)}
+        print(f"{name:13s} {tf:8.1f} TFLOP/s at {ghz:.3f} GHz  ({tf / 25.0:.1f} % of 2.5 PFLOP/s)", flush=True)
+    print(json.dumps(out))
+    dev.destroy()
+
+
+if __name__ == "__main__":
+    main()
