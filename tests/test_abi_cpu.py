@@ -199,12 +199,12 @@ def test_picker_properties(lib):
     info, split, _ = pick(lib, m=1024, n=64, k=1024, lda=1024, ldb=64, ldc=64, nbatch=96,
                           sa=1024 * 1024, sb=1024 * 64, sc=1024 * 64)
     assert split == 1 and info.bn <= 128
-    # the skinny-M streaming tile runs NT with at most 4 rows over K <= 2048 and hands
+    # the skinny-M streaming tile runs NT with at most 8 rows over K <= 2048 and hands
     # everything else to its fallback
     mv = next(i for i in range(lib.mg_tile_count()) if tile_name(lib, i).startswith("mv_"))
     info, split, _ = pick(lib, layout=L.MG_NT, m=3, n=50257, k=768, lda=768, ldb=768, ldc=50257, tile=mv)
     assert info.id == mv and split == 1
-    for kw in (dict(layout=L.MG_NT, m=5, n=4096, k=768, lda=768, ldb=768, ldc=4096),
+    for kw in (dict(layout=L.MG_NT, m=9, n=4096, k=768, lda=768, ldb=768, ldc=4096),
                dict(layout=L.MG_NT, m=1, n=4096, k=4096, lda=4096, ldb=4096, ldc=4096),
                dict(layout=L.MG_NT, m=4, n=4096, k=772, lda=772, ldb=772, ldc=4096),
                dict(layout=L.MG_NN, m=4, n=4096, k=768, lda=768, ldb=4096, ldc=4096)):

@@ -233,16 +233,18 @@ def test_stream_k_tiles_exact(dev, layout):
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_skinny_stream_tile_exact(dev, dtype):
-    """The skinny-M streaming tile (NT, M <= 4, K <= 2048, no matrix cores): every row
-    count 1..4, K of one to four 512-element chunks with ragged ends, N ragged against
-    the 16 rows of a wavefront and the 64 of a workgroup, bias, beta = 1, a padded pitch
-    of C; bit exact on integer data, within tolerance on random data; and the plan must
-    really be that tile."""
+    """The skinny-M streaming tile (NT, M <= 8, K <= 2048, no matrix cores): every row
+    count 1..8, K of one to four 512-element chunks with ragged ends (and the 513..768 class,
+    whose last chunk pairs of rows share), N from one row to more than the resident wavefronts
+    take at once, bias, beta = 1, a padded pitch of C; bit exact on integer data,
+    within tolerance on random data; and the plan must really be that tile."""
     from vkgrad_amd.kernels import CONFIGS, Matmul
     mv = next(t for t in CONFIGS if t["name"].startswith("mv_"))
     mp = Matmul(dev, trans_b=True, dtype=dtype, tile=mv["id"])
     cases = [(1, 50257, 768), (4, 2304, 768), (3, 1000, 1024), (3, 96, 768), (2, 777, 2048), (4, 129, 8),
-             (1, 1, 8), (4, 4097, 520), (4, 63, 1536), (1, 17, 2048), (2, 64, 512), (2, 65, 1032), (4, 300, 2048)]
+             (1, 1, 8), (4, 4097, 520), (4, 63, 1536), (1, 17, 2048), (2, 64, 512), (2, 65, 1032), (4, 300, 2048),
+             (7, 50257, 768), (8, 2304, 768), (5, 96, 768), (6, 100003, 264), (8, 33000, 2048), (7, 31, 1024),
+             (3, 45, 648), (8, 77, 760), (1, 130, 768), (2, 5, 528)]
     for i, (m, n, k) in enumerate(cases):
         assert mp.plan(m, n, k)[0] == mv["id"], (m, n, k)
         r, got, ref = check_case(dev, m, n, k, False, True, dtype, seed=m + n + k, integer=True, tile=mv["id"],
@@ -252,7 +254,7 @@ def test_skinny_stream_tile_exact(dev, dtype):
         r, got, ref = check_case(dev, m, n, k, False, True, dtype, seed=3, tile=mv["id"], bias=True)
         _assert_close(r, f"mv {m}x{n}x{k}")
     # what it cannot run goes to its fallback and is still right
-    r, got, ref = check_case(dev, 5, 300, 768, False, True, dtype, seed=1, integer=True, tile=mv["id"])
+    r, got, ref = check_case(dev, 9, 300, 768, False, True, dtype, seed=1, integer=True, tile=mv["id"])
     assert r["exact"]
     r, got, ref = check_case(dev, 4, 300, 768, False, False, dtype, seed=1, integer=True, tile=mv["id"])
     assert r["exact"]

@@ -127,15 +127,14 @@ struct Plan {
 // Preconditions of the direct-to-LDS kernels (gemm_dma_kernel.h): aligned bases
 // and pitches, K slices that are multiples of BK (the last may be ragged), and
 // row pitches that cover the 16-byte chunk straddling a ragged edge.
-// The skinny-M kernel holds MP >= M rows of A (1, 2 or 4) over NCH >= K / 512 chunks
-// (1, 2 or 4) in registers and reads 16-byte pieces of both operands.
-static bool gemv_shape(const mg_gemm_args &a, int *mp_log2, int *nch_log2) {
-    if (a.m > 4 || a.k > 2048) return false;
-    int lm = 0, lc = 0;
+// The skinny-M kernel holds MP >= M rows of A (1, 2, 4 or 8) over K <= 512, 768, 1024 or
+// 2048 elements in registers and reads 16-byte pieces of both operands.
+static bool gemv_shape(const mg_gemm_args &a, int *mp_log2, int *k_class) {
+    if (a.m > 8 || a.k > 2048) return false;
+    int lm = 0;
     while ((1 << lm) < a.m) lm++;
-    while ((512 << lc) < a.k) lc++;
     if (mp_log2) *mp_log2 = lm;
-    if (nch_log2) *nch_log2 = lc;
+    if (k_class) *k_class = gemv_k_class((int)a.k);
     return true;
 }
 static bool gemv_eligible(const mg_gemm_args &a, int split) {
@@ -201,7 +200,7 @@ static const float g_cost[MG_NUM_TILES][3][2] = {
     {{5.27f, 0.871f}, {3.25f, 0.983f}, {3.08f, 0.980f}},   // 17 mmp_128x128x64_w2x2_s2
     {{4.81f, 2.006f}, {7.24f, 1.819f}, {3.05f, 2.002f}},   // 18 mmk_256x256x64_w2x4_s2
     {{5.52f, 0.907f}, {4.46f, 0.944f}, {3.88f, 1.003f}},   // 19 mmk_128x128x64_w2x2_s2
-    {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}},                     // 20 mv_4x64x512 (priced by bytes, see plan_cost_us)
+    {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}},                     // 20 mv_8x64x512 (priced by bytes, see plan_cost_us)
     {{5.69f, 1.230f}, {13.28f, 1.060f}, {4.76f, 1.200f}},   // 21 mmq_256x256x64_w2x4_s2 (tile 10's overhead, its own K-block time)
 };
 

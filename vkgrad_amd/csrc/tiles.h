@@ -15,7 +15,7 @@
 //     (pieces meet in the context's workspace), so the last round fills the chip too.
 //     S(id, BM, BN, BK, WGM, WGN, NSTAGE, fallback_id) — falls back to the
 //     persistent tile of the same shape (no workspace, or ragged K).
-//   skinny-M stream (gemv_kernel.h): NT layout with at most 4 rows of A and K <= 2048;
+//   skinny-M stream (gemv_kernel.h): NT layout with at most 8 rows of A and K <= 2048;
 //     no matrix cores, B is read once as it lies in memory.
 //     G(id, BM, BN, BK, fallback_id) — BM rows of A at most, BN output columns per
 //     workgroup, BK elements of K per register chunk; falls back to a skinny
@@ -47,7 +47,7 @@
     P(17, 128, 128, 64, 2, 2, 2, 11) \
     S(18, 256, 256, 64, 2, 4, 2, 15) \
     S(19, 128, 128, 64, 2, 2, 2, 17) \
-    G(20, 4, 64, 512, 4) \
+    G(20, 8, 64, 512, 4) \
     Q(21, 256, 256, 64, 2, 4, 2, 10)
 
 #define MG_NUM_TILES 22

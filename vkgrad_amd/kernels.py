@@ -418,9 +418,9 @@ def buffer_sets_for(footprint):
 
 
 def skinny_stream_fits(m, k, layout):
-    """The skinny-M streaming tile (name mv_*): NT layout, at most 4 rows of A and
+    """The skinny-M streaming tile (name mv_*): NT layout, at most 8 rows of A and
     K <= 2048 in whole 8-element pieces."""
-    return layout == L.MG_NT and m <= 4 and k <= 2048 and k % 8 == 0
+    return layout == L.MG_NT and m <= 8 and k <= 2048 and k % 8 == 0
 
 
 def candidate_space(m, n, k, cus=256, nbatch=1, layout=None):
