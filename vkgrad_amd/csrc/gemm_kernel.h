@@ -52,6 +52,10 @@ struct GemmParams {
     int xcd_remap;        // 1: renumber workgroups so neighbours share an XCD
     float *ws;            // split-K workspace (split_k * tiles * BM * BN floats) or null: add with atomics
     int *cnt;             // one arrival counter per tile, zero between launches
+    // Staggered start (ping-pong kernel): the first stagger_blocks workgroups - the ones resident
+    // at once - nap phase / 8 of stagger_clk clocks before they begin, so that the C stores of
+    // a round of short-K tiles do not reach memory in one burst.  0: off.
+    int stagger_clk, stagger_blocks;
     int stream_k;         // stream-K kernel only: cut the tiles of the last, partial round along K
     // stream-K partition, computed by the host for the launched grid: whole rounds of tiles,
     // tiles left over after them, and the number of equal K pieces each of those is cut into

@@ -143,6 +143,21 @@ struct PpLoad {
     }
 };
 
+// With a short K loop the tiles of a round finish together and their C stores meet the HBM
+// write rate all at once (8192 x 3072 x 768: 64 MB in one burst, 11 us of a 27 us round), while
+// memory idles during the K loops.  Spreading the starts of the first round over one K loop
+// spreads the stores of every later round too; the early finishers take the tiles of the
+// partial last round.  Workgroups are handed to the eight XCDs in turn and inside an XCD to
+// its CUs in turn, so id / 8 walks the CUs of an XCD: neighbours get consecutive phases.
+__device__ __forceinline__ void stagger_start(const GemmParams &p) {
+    if (p.stagger_clk <= 0) return;
+    const unsigned bid = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    if (bid >= (unsigned)p.stagger_blocks) return;
+    const unsigned phase = (bid >> 3) & 7;
+    const int naps = (int)(((int64_t)p.stagger_clk * phase) >> 13);   // about 1024 clocks a nap
+    for (int i = 0; i < naps; i++) __builtin_amdgcn_s_sleep(16);
+}
+
 template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, bool ACT = false>
 __global__ void __launch_bounds__(WGM *WGN * 64)
 gemm_pp_kernel(const GemmParams p) {
@@ -173,6 +188,7 @@ gemm_pp_kernel(const GemmParams p) {
     const int wi = wave & (NWI - 1);
     const int grp = wave / NWI;              // == wave_m: group 0 owns the upper half of the tile
 
+    stagger_start(p);
     int pid_m, pid_n;
     tile_coords(p, pid_m, pid_n);
     const int m0 = pid_m * BM, n0 = pid_n * BN;

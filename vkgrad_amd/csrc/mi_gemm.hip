@@ -834,6 +834,17 @@ static int enqueue_gemm(const Lane &ln, const mg_gemm_args *args, const Plan &pl
     p.ws = nullptr;
     p.cnt = nullptr;
     p.stream_k = 0;
+    p.stagger_clk = p.stagger_blocks = 0;
+    if (t.pingpong) {
+        // more than one round of tiles whose K loop is short beside their C store: spread the
+        // starts of the first round over one K loop (2048 MFMA clocks a K-block)
+        const int64_t wgs = (int64_t)pl.grid_m * pl.grid_n * a.nbatch * pl.split_k;
+        const int64_t nkb = cdiv(pl.split_k > 1 ? pl.k_per_split : a.k, t.bk);
+        if (wgs > ln.cus && nkb <= 16) {
+            p.stagger_clk = (int)nkb * 2048;
+            p.stagger_blocks = ln.cus;
+        }
+    }
     p.sk_full_rounds = p.sk_rem_tiles = 0;
     p.sk_pieces = 1;
     if (pl.split_k > 1) {
