@@ -173,11 +173,8 @@ struct DmaTraits {
     static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;
 };
 
-// MINW: wavefronts per SIMD the register allocation must leave room for (1: no constraint).
-// Eight wavefronts of 64 x 64 need fewer than 128 registers, so two such workgroups fit a CU
-// (four wavefronts per SIMD) when the compiler is told to stay below that.
-template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool ACT = false, int MINW = 1>
-__global__ void __launch_bounds__(WGM *WGN * 64, MINW)
+template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool ACT = false>
+__global__ void __launch_bounds__(WGM *WGN * 64)
 gemm_dma_kernel(const GemmParams p) {
     constexpr bool A_KC = (LAYOUT != L_TN);
     constexpr bool B_KC = (LAYOUT == L_NT);
@@ -688,10 +685,10 @@ gemm_dmap_kernel(const GemmParams p) {
     }
 }
 
-template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool ACT = false, int MINW = 1>
+template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool ACT = false>
 hipError_t launch_gemm_dma(const GemmParams &p, dim3 grid, hipStream_t stream) {
     using TT = DmaTraits<LAYOUT, BM, BN, BK, WGM, WGN, NSTAGE>;
-    auto kern = gemm_dma_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, NSTAGE, ACT, MINW>;
+    auto kern = gemm_dma_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, NSTAGE, ACT>;
     static std::atomic<uint64_t> lds_allowed{0};
     hipError_t e = allow_dynamic_lds((const void *)kern, TT::LDS_BYTES, lds_allowed);
     if (e != hipSuccess) return e;
