@@ -238,9 +238,12 @@ int mg_gemm_static(int device_index, void *hip_stream, const mg_gemm_args *args)
  * `iters` rounds of eight back-to-back v_mfma_f32_32x32x16 from registers.  random_operands = 0
  * multiplies zeros (the chip holds its boost clock), 1 multiplies random 16-bit values (the
  * power-managed clock drops, and with it the rate every real GEMM is bounded by).  Returns the
- * rate and the shader clock during the loop.  The reference's counterpart is the hand-measured
- * WMMA peak it prices its kernels against (bench/RESULTS.md:113-119, 656-659). */
-int mg_probe_mfma(mg_ctx *ctx, int dtype, int random_operands, int iters, double *tflops, double *ghz);
+ * rate and the shader clock during the loop.  workgroups = 0 keeps every CU busy; a smaller
+ * positive count keeps that many busy (one workgroup each), which shows how the clock depends on
+ * the number of CUs multiplying.  The reference's counterpart is the hand-measured WMMA peak it
+ * prices its kernels against (bench/RESULTS.md:113-119, 656-659). */
+int mg_probe_mfma(mg_ctx *ctx, int dtype, int random_operands, int iters, int workgroups, double *tflops,
+                  double *ghz);
 /* CONFIGS — kernels.py:326-331: the tile table the tuner walks. */
 int mg_tile_count(void);
 int mg_tile_info(int id, mg_tile *out);

@@ -350,3 +350,9 @@ def test_mfma_ceiling_probe(dev):
     assert r_tf <= z_tf * 1.03
     f_tf, _ = mfma_ceiling(dev, "f16", True, seconds=0.05)
     assert f_tf > 100.0
+    # a quarter of the CUs busy: a quarter of the work per clock, at a clock that is no lower
+    q = dev.compute_units // 4
+    q_tf, q_ghz = mfma_ceiling(dev, "bf16", True, seconds=0.05, busy_cus=q)
+    per_clock = q_tf * 1e12 / (q_ghz * 1e9) / (q * 4)
+    assert 0.85 * 1024 <= per_clock <= 1.02 * 1024, per_clock
+    assert q_ghz >= r_ghz * 0.97

@@ -63,8 +63,9 @@ __global__ void __launch_bounds__(512) k_probe_mfma(int iters, uint32_t seed, in
 
 using namespace mg;
 
-extern "C" int mg_probe_mfma(mg_ctx *ctx, int dtype, int random_operands, int iters, double *tflops, double *ghz) {
-    EW_PRECHECK("mg_probe_mfma", dtype_ok(dtype) && iters > 0 && iters <= (1 << 24) && tflops && ghz);
+extern "C" int mg_probe_mfma(mg_ctx *ctx, int dtype, int random_operands, int iters, int workgroups, double *tflops,
+                             double *ghz) {
+    EW_PRECHECK("mg_probe_mfma", dtype_ok(dtype) && iters > 0 && iters <= (1 << 24) && workgroups >= 0 && tflops && ghz);
     hipStream_t stream = ctx_stream(ctx);
     int dev = 0, cus = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -79,7 +80,9 @@ extern "C" int mg_probe_mfma(mg_ctx *ctx, int dtype, int random_operands, int it
     if (e == hipSuccess) {
         auto kern = dtype == MG_F16 ? k_probe_mfma<D_F16> : k_probe_mfma<D_BF16>;
         float *sink = reinterpret_cast<float *>(clocks + 4);
-        // one workgroup of eight wavefronts per CU: two per SIMD; a short untimed launch first
+        // one workgroup of eight wavefronts per CU (two per SIMD), on all CUs or on the first
+        // `workgroups` the dispatcher picks; a short untimed launch first
+        if (workgroups > 0 && workgroups < cus) cus = workgroups;
         hipLaunchKernelGGL(kern, dim3(cus), dim3(512), 0, stream, iters / 8 + 1, 1u, random_operands, clocks, sink);
         e = hipEventRecord(e0, stream);
         hipLaunchKernelGGL(kern, dim3(cus), dim3(512), 0, stream, iters, 2u, random_operands, clocks, sink);
