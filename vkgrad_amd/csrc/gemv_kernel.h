@@ -94,7 +94,7 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64, gemv_min_waves(MP, NCH, HALF)
     const int kh = NCH * 512 + (lane & 31) * 8;                        // this lane's elements of the half chunk
 
     // the stream first: everything the registers hold goes out before A is touched
-    uint4 b[NG][4][NCH > 0 ? NCH : 1];
+    uint4 b[NG][4][NCH];
     uint4 bh[NG][2];
 #pragma unroll
     for (int g = 0; g < NG; g++) {
@@ -119,7 +119,7 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64, gemv_min_waves(MP, NCH, HALF)
     }
 
     // this lane's elements of every row of A
-    uint4 a[MP][NCH > 0 ? NCH : 1];
+    uint4 a[MP][NCH];
     uint4 ah[MP];
 #pragma unroll
     for (int m = 0; m < MP; m++) {
