@@ -601,6 +601,13 @@ def test_ping_pong_tile(dev, layout, dtype):
         r, got, ref = check_case(dev, m, n, k, ta, tb, dtype, seed=m + n + k, integer=True, tile=pp, bias=(k % 128 == 0),
                                  accumulate=(m % 2 == 1))
         assert r["exact"], f"{layout} {dtype} {m}x{n}x{k}: {int((got != ref).sum())} entries differ"
+    # more workgroups than CUs with a short K loop: the first round starts staggered (ragged
+    # edges; unsplit, and with a K split whose slices make up the surplus)
+    if dtype == "bf16":
+        r, got, ref = check_case(dev, 4344, 4104, 200, ta, tb, dtype, seed=9, integer=True, tile=pp, bias=True)
+        assert r["exact"], f"{layout} staggered: {int((got != ref).sum())} entries differ"
+        r, got, ref = check_case(dev, 2300, 2304, 2048, ta, tb, dtype, seed=10, integer=True, tile=pp, split_k=4, accumulate=True)
+        assert r["exact"], f"{layout} staggered, split: {int((got != ref).sum())} entries differ"
     # padded pitches (the padding holds NaN) and K splits through the workspace and with atomics
     r, got, ref = check_case(dev, 300, 520, 1024, ta, tb, dtype, seed=5, integer=True, tile=pp, split_k=4, bias=True,
                              lda=(304 if ta else 1032), ldb=(1032 if tb else 528), ldc=536)
