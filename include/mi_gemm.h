@@ -285,6 +285,10 @@ int mg_graph_enqueue(mg_ctx *ctx, mg_graph *g);
  * replays and waits; seconds_each[i] = device time of replay i.  The reference times a
  * recorded step by host wall clock around submit (vk.py:877-889, bench/ab.py:36-51). */
 int mg_graph_time(mg_ctx *ctx, mg_graph *g, int repeat, double *seconds_each);
+/* Graph.n_dispatch — vk.py:824, 868, counted where the work is: the kernel launches a recorded
+ * graph replays (one library call may record several: a clear in front of an atomic K split, a
+ * long-K GEMM whose partial last round runs as a second, split launch). */
+int mg_graph_kernel_count(mg_ctx *ctx, mg_graph *g, int *kernels);
 int mg_graph_destroy(mg_ctx *ctx, mg_graph *g);
 
 /* ---- companion elementwise kernels: kernels.make_kernels (kernels.py:699-862) ----

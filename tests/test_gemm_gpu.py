@@ -724,3 +724,42 @@ def test_medium_random(dev, layout, dtype):
     ta, tb = LAYOUTS[layout]
     r, _, _ = check_case(dev, 1024, 768, 1536, ta, tb, dtype, seed=11, bias=True)
     _assert_close(r, f"{layout} {dtype} 1024x768x1536")
+
+
+def test_ping_pong_partial_round_split(dev):
+    """An unsplit ping-pong GEMM with a long K loop whose tiles leave a partial last round runs
+    as two launches - whole rounds of tile rows unsplit, the remaining tile rows with a K split
+    that fills the chip - and the result is what the oracle says (integer data: exact), with
+    ragged edges, a K remainder, bias and beta = 1.  A shape without a partial round, and one
+    whose K loop is too short to pay for the second launch, stay one launch."""
+    from vkgrad_amd.kernels import CONFIGS, Matmul
+    pp = next(t["id"] for t in CONFIGS if t["name"].startswith("mmq_"))
+    cus = dev.compute_units
+    if cus != 256:
+        pytest.skip("shapes below are laid out for 256 CUs")
+
+    def launches(layout, m, n, k):
+        ta, tb = LAYOUTS[layout]
+        a, b = O.make_operands(m, n, k, ta, tb, "bf16", seed=1, integer=True)
+        ba, bb, bc = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), dev.buffer(m * n * 4, "device")
+        mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype="bf16", tile=pp, split_k=1)
+        g = dev.graph("count")
+        try:
+            ba.upload(a); bb.upload(b)
+            mm(ba, bb, bc, m, n, k, graph=g)
+            g.finish()
+            return g.kernel_count()
+        finally:
+            g.destroy(); mm.destroy()
+            for x in (ba, bb, bc):
+                x.destroy()
+
+    # 17 x 16 = 272 tiles: 16 whole tile rows, then 16 tiles cut 8 ways along K = 4096 (+ 8)
+    assert launches("NT", 4352, 4096, 4096) == 2
+    assert launches("NT", 4096, 4096, 4096) == 1          # 256 tiles: whole rounds
+    assert launches("NT", 4352, 4096, 512) == 1           # 8 K-blocks: not worth a second launch
+    for layout in ("NT", "NN", "TN"):
+        ta, tb = LAYOUTS[layout]
+        r, got, ref = check_case(dev, 4352 - 8, 4096 - 24, 4096 + 8, ta, tb, "bf16", seed=21, integer=True, tile=pp, split_k=1,
+                                 bias=True, accumulate=True)
+        assert r["exact"], f"{layout}: {int((got != ref).sum())} entries differ"

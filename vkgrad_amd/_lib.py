@@ -100,6 +100,7 @@ SIGNATURES = {
     "mg_graph_launch": (C.c_int, [_P, _P, C.POINTER(C.c_double)]),
     "mg_graph_enqueue": (C.c_int, [_P, _P]),
     "mg_graph_time": (C.c_int, [_P, _P, C.c_int, C.POINTER(C.c_double)]),
+    "mg_graph_kernel_count": (C.c_int, [_P, _P, C.POINTER(C.c_int)]),
     "mg_graph_destroy": (C.c_int, [_P, _P]),
     "mg_ew_bias_act": (C.c_int, [_P, _P, _P, _P, _P, C.c_int64, C.c_int64, C.c_int, C.c_int]),
     "mg_ew_act_bwd": (C.c_int, [_P, _P, _P, _P, _P, C.c_int64, C.c_int, C.c_int]),

@@ -2,6 +2,8 @@
 // Declarations and the reference interfaces they replace are in include/mi_gemm.h.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
@@ -772,9 +774,57 @@ static int lane_of(mg_ctx *ctx, const mg_gemm_args &a, Lane &ln) {
     return MG_OK;
 }
 
+// The partial last round of an unsplit ping-pong GEMM with a long K loop.  591 tiles on 256 CUs
+// are three rounds of which the last keeps 79 CUs busy; run as two GEMMs over row ranges - whole
+// rounds unsplit, the remaining tile rows with a K split that fills the chip once more - the
+// 50257 x 768 x 8192 dW product takes 538 us instead of 581.  Estimated in K-block times: a round
+// costs the K loop, the split part its slice of it plus 1.7 per slice for the meeting of the
+// partial tiles and 2.5 for the second launch.  Returns the rows of the first GEMM (0: no split).
+static int64_t tail_rows(const Lane &ln, const mg_gemm_args &a, const Plan &pl, const TileDesc &t, int *slices) {
+    if (!t.pingpong || pl.split_k != 1 || a.nbatch != 1 || a.tri != MG_TRI_NONE) return 0;
+    if (!a.c || a.y16 || a.z || a.colsum || a.res || a.p16) return 0;
+    const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n, cus = ln.cus;
+    if (cus < 8 || tiles <= cus || tiles % cus == 0) return 0;
+    const int64_t rows1 = (tiles / cus) * cus / pl.grid_n;            // tile rows of the whole rounds
+    const int64_t rest = (pl.grid_m - rows1) * pl.grid_n;             // tiles left over
+    if (rows1 < 1 || rest < 1) return 0;
+    const int64_t s = std::min<int64_t>(8, cus / rest);
+    const int64_t nkb = cdiv(a.k, t.bk);
+    if (s < 2 || nkb / s < 8) return 0;
+    const double as_is = (double)cdiv(tiles, cus) * nkb;
+    const double cut = (double)cdiv(rows1 * pl.grid_n, cus) * nkb + cdiv(nkb, s) + 1.7 * s + 2.5;
+    if (cut > 0.95 * as_is) return 0;
+    if (!ln.ws || rest * s * t.bm * t.bn * (int64_t)sizeof(float) > ln.ws_bytes || rest > ln.max_tiles) return 0;
+    *slices = (int)s;
+    return rows1 * t.bm;
+}
+
 static int enqueue_gemm(const Lane &ln, const mg_gemm_args *args, const Plan &pl) {
     const mg_gemm_args &a = *args;
     const TileDesc &t = g_tiles[pl.tile];
+    {
+        int slices = 1;
+        const int64_t m1 = tail_rows(ln, a, pl, t, &slices);
+        if (m1 > 0) {
+            mg_gemm_args head = a, tail = a;
+            head.m = m1;
+            head.tile = tail.tile = pl.tile;
+            head.split_k = 1;
+            tail.m = a.m - m1;
+            tail.split_k = slices;
+            tail.flags &= ~MG_FLAG_SPLITK_ATOMIC;
+            tail.a = (const char *)a.a + (a.layout == MG_TN ? m1 : m1 * a.lda) * 2;
+            tail.c = a.c + m1 * a.ldc;
+            Plan ph, pt;
+            pick_plan(head, ln.cus, ph);
+            pick_plan(tail, ln.cus, pt);
+            // (neither part qualifies again: the head is whole rounds, the tail is split)
+            if (ph.tile == pl.tile && pt.tile == pl.tile && ph.split_k == 1 && pt.split_k == slices) {
+                const int rc = enqueue_gemm(ln, &head, ph);
+                return rc != MG_OK ? rc : enqueue_gemm(ln, &tail, pt);
+            }
+        }
+    }
     hipStream_t stream = ln.stream;
     const int64_t lane_bytes = ln.ws_bytes;
     float *lane_ws = ln.ws;
@@ -1089,6 +1139,25 @@ int mg_graph_time(mg_ctx *ctx, mg_graph *g, int repeat, double *seconds_each) {
     for (int i = 0; i < made; i++) (void)hipEventDestroy(ev[i]);
     delete[] ev;
     return rc;
+}
+
+int mg_graph_kernel_count(mg_ctx *ctx, mg_graph *g, int *kernels) {
+    if (!ctx || !g || !kernels) return fail(MG_ERR_ARG, "mg_graph_kernel_count: NULL argument");
+    size_t n = 0;
+    HIP_TRY(hipGraphGetNodes(g->graph, nullptr, &n));
+    hipGraphNode_t *nodes = n ? new (std::nothrow) hipGraphNode_t[n] : nullptr;
+    if (n && !nodes) return fail(MG_ERR_STATE, "mg_graph_kernel_count: out of host memory");
+    int count = 0;
+    hipError_t e = n ? hipGraphGetNodes(g->graph, nodes, &n) : hipSuccess;
+    for (size_t i = 0; e == hipSuccess && i < n; i++) {
+        hipGraphNodeType ty;
+        e = hipGraphNodeGetType(nodes[i], &ty);
+        if (e == hipSuccess && ty == hipGraphNodeTypeKernel) count++;
+    }
+    delete[] nodes;
+    if (e != hipSuccess) return hip_fail(e, "mg_graph_kernel_count");
+    *kernels = count;
+    return MG_OK;
 }
 
 int mg_graph_destroy(mg_ctx *ctx, mg_graph *g) {

@@ -187,6 +187,13 @@ class Graph:
         _check(self.dev._lib.mg_graph_time(self.dev._ctx, self._handle, int(repeat), out), f"{self.name}: time")
         return list(out)
 
+    def kernel_count(self):
+        """Kernel launches one replay makes (a recorded call may stand for several)."""
+        self._check_alive("kernel_count")
+        n = C.c_int()
+        _check(self.dev._lib.mg_graph_kernel_count(self.dev._ctx, self._handle, C.byref(n)), f"{self.name}: kernel_count")
+        return n.value
+
     def destroy(self):
         if self._handle is not None:
             h, self._handle = self._handle, None
