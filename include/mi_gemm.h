@@ -247,6 +247,29 @@ int mg_probe_mfma(mg_ctx *ctx, int dtype, int random_operands, int iters, int wo
 /* CONFIGS — kernels.py:326-331: the tile table the tuner walks. */
 int mg_tile_count(void);
 int mg_tile_info(int id, mg_tile *out);
+/* Kernel.statistics() - vk.py:690-736 (driver-reported VGPRs, LDS and scratch of a compiled
+ * pipeline) and the inputs of occupancy() - kernels.py:384-411.  Reports, for the kernel the
+ * library would launch for `args` (after the picker, the tuned tile/split in args, and every
+ * fallback), what the HIP runtime says about that instantiation on the context's device:
+ * registers per lane, static and dynamic LDS, scratch (spill) bytes per lane, and how many of its
+ * workgroups one CU holds.  `tile` receives the tile that would run.  Launches nothing. */
+typedef struct {
+    int32_t vgprs;             /* registers per lane (hipFuncAttributes.numRegs) */
+    int32_t scratch_bytes;     /* private memory per lane; non-zero means the kernel spills */
+    int32_t static_lds_bytes;
+    int32_t dynamic_lds_bytes;
+    int32_t threads;           /* workgroup size */
+    int32_t wgs_per_cu;        /* resident workgroups per CU for this launch shape */
+    int32_t waves_per_simd;    /* wgs_per_cu * (threads / 64) / 4 SIMDs, rounded up */
+    int32_t max_threads;       /* hipFuncAttributes.maxThreadsPerBlock */
+} mg_kernel_stats;
+int mg_kernel_stats_for(mg_ctx *ctx, const mg_gemm_args *args, int *tile, mg_kernel_stats *out);
+/* The same for one instantiation named directly: tile id, layout (MG_NN..), dtype, and
+ * variant 0 (aligned operands / plain epilogue), 1 (any alignment for register-staged tiles,
+ * bias epilogue for persistent ones) or 2 (fused activation output).  For the skinny-M tile the
+ * variant is 4 * log2(rows of A held) + K class (0: K <= 512, 1: 768, 2: 1024, 3: 2048).
+ * MG_ERR_ARG when the table holds no such instantiation. */
+int mg_tile_kernel_stats(mg_ctx *ctx, int tile, int layout, int dtype, int variant, mg_kernel_stats *out);
 /* Matmul.fits for one tile: 1 if tile `id` can run `args`, else 0. */
 int mg_tile_fits(int id, const mg_gemm_args *args);
 /* pick_config — autograd.py:22-41: heuristic choice without benchmarking; pure.

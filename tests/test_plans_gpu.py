@@ -339,3 +339,68 @@ def test_autotune_batched_shape_and_cache_roundtrip(dev, tmp_path, monkeypatch):
         mm2.destroy()
     finally:
         mm.destroy()
+
+
+# ---------------------------------------------------------------------------
+# Kernel resource statistics (Kernel.statistics, /root/reference/vk.py:690-736; occupancy,
+# /root/reference/kernels.py:384-411): no instantiation spills, and each tile holds the
+# workgroups per CU its design and the picker's cost model assume.
+# ---------------------------------------------------------------------------
+
+# workgroups per CU by tile name: two for the four-wave tiles whose ring takes at most half the
+# LDS, one for the 256 x 256 tiles and the register-staged tiles with more than half the LDS
+_WGS_PER_CU = {
+    "mm_256x256x32_w2x4": 1, "mm_256x128x64_w2x2": 1, "mm_128x256x64_w2x2": 1, "mm_128x128x64_w2x2": 2,
+    "mm_64x256x64_w1x4": 1, "mm_32x256x64_w1x4": 1, "mm_256x64x64_w4x1": 1, "mm_256x32x64_w4x1": 1,
+    "mmd_256x256x32_w2x4_s4": 1, "mmd_256x256x64_w2x4_s2": 1, "mmd_128x128x64_w2x2_s2": 2,
+    "mmd_128x256x32_w2x2_s3": 2, "mmd_256x128x32_w2x2_s3": 2, "mmd_128x128x32_w2x2_s3": 2,
+    "mmp_256x256x64_w2x4_s2": 1, "mmp_256x256x32_w2x4_s4": 1, "mmp_128x128x64_w2x2_s2": 2,
+    "mmk_256x256x64_w2x4_s2": 1, "mmk_128x128x64_w2x2_s2": 2, "mmq_256x256x64_w2x4_s2": 1,
+}
+
+
+def test_no_instantiation_spills_and_occupancy_is_as_designed(dev):
+    from vkgrad_amd import kernels as K
+    seen = 0
+    for t in K.CONFIGS:
+        skinny = t["name"].startswith("mv_")
+        for layout in (K.L.MG_NN, K.L.MG_NT, K.L.MG_TN):
+            for dtype in ("f16", "bf16"):
+                for variant in (range(16) if skinny else range(3)):
+                    st = K.tile_statistics(dev, t["id"], layout, dtype, variant)
+                    if st is None:
+                        continue
+                    seen += 1
+                    what = (t["name"], layout, dtype, variant, st)
+                    assert st["scratchMemUsageInBytes"] == 0, what
+                    assert 0 < st["numUsedVgprs"] <= 512, what
+                    assert st["workgroupThreads"] == t["threads"], what
+                    assert st["workgroupsPerCU"] >= 1, what
+                    if skinny:
+                        continue
+                    assert st["ldsUsageSizeInBytes"] <= 160 * 1024, what
+                    if t["name"] in _WGS_PER_CU:
+                        assert st["workgroupsPerCU"] == _WGS_PER_CU[t["name"]], what
+                    else:
+                        assert t["name"] == "mm_64x64x64_w2x2" and st["workgroupsPerCU"] >= 3, what
+                    occ, reason = K.occupancy(dev, st)
+                    assert reason is None and occ == st["wavesPerSimd"], what
+    # 22 tiles x 3 layouts x 2 dtypes, most with two or three variants
+    assert seen > 250
+
+
+def test_statistics_of_a_planned_gemm_and_tuner_fields(dev):
+    """Matmul.statistics names the kernel the call would launch; the tuner records vgpr and
+    occupancy with its pick as the reference does (kernels.py:527-529)."""
+    from vkgrad_amd.kernels import Matmul, autotune_matmul, CONFIGS
+    mm = Matmul(dev, trans_b=True, dtype="bf16", tile=21)
+    st = mm.statistics(8192, 3072, 768)
+    assert CONFIGS[st["tile_id"]]["name"] == "mmq_256x256x64_w2x4_s2"
+    assert st["workgroupThreads"] == 512 and st["ldsUsageSizeInBytes"] == 131072 and st["workgroupsPerCU"] == 1
+    # unaligned operands: the plan falls back to the register-staged 256 x 256 tile
+    st = mm.statistics(8192, 3072, 770, lda=771, ldb=771)
+    assert CONFIGS[st["tile_id"]]["name"] == "mm_256x256x32_w2x4" and st["scratchMemUsageInBytes"] == 0
+    mm.destroy()
+    mm, best = autotune_matmul(dev, 512, 512, 512, reps=1, use_cache=False, dtype="bf16")
+    assert best["vgpr"] and best["vgpr"] <= 512 and best["occupancy"] >= 1 and best["spilling"] == []
+    mm.destroy()

@@ -60,6 +60,14 @@ class Tile(C.Structure):
     ]
 
 
+class KernelStats(C.Structure):
+    _fields_ = [
+        ("vgprs", C.c_int32), ("scratch_bytes", C.c_int32), ("static_lds_bytes", C.c_int32),
+        ("dynamic_lds_bytes", C.c_int32), ("threads", C.c_int32), ("wgs_per_cu", C.c_int32),
+        ("waves_per_simd", C.c_int32), ("max_threads", C.c_int32),
+    ]
+
+
 class DeviceInfo(C.Structure):
     _fields_ = [
         ("name", C.c_char * 128), ("arch", C.c_char * 64),
@@ -94,6 +102,8 @@ SIGNATURES = {
     "mg_tile_count": (C.c_int, []),
     "mg_tile_info": (C.c_int, [C.c_int, C.POINTER(Tile)]),
     "mg_tile_fits": (C.c_int, [C.c_int, C.POINTER(GemmArgs)]),
+    "mg_kernel_stats_for": (C.c_int, [_P, C.POINTER(GemmArgs), C.POINTER(C.c_int), C.POINTER(KernelStats)]),
+    "mg_tile_kernel_stats": (C.c_int, [_P, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(KernelStats)]),
     "mg_pick": (C.c_int, [C.POINTER(GemmArgs), C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "mg_graph_begin": (C.c_int, [_P]),
     "mg_graph_end": (C.c_int, [_P, C.POINTER(_P)]),

@@ -173,8 +173,18 @@ struct DmaTraits {
     static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;
 };
 
+// Four-wave workgroups whose accumulators take 128 registers a lane and whose ring takes at most
+// half the LDS are meant to run two to a CU: the second launch bound keeps the register
+// allocator under 256, which it otherwise exceeds for the 256 x 128 and 128 x 256 tiles (348
+// registers, one workgroup per CU, 60.6 against 51.2 us at 8192 x 3072 x 768).  The smaller
+// four-wave tiles stay under 256 by themselves and are left to the allocator.
+template <int BM, int BN, int BK, int WGM, int WGN, int NSTAGE>
+constexpr int dma_waves_per_simd() {
+    return (WGM * WGN == 4 && BM * BN == 256 * 128 && NSTAGE * (BM + BN) * BK * 2 <= 81920) ? 2 : 1;
+}
+
 template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool ACT = false>
-__global__ void __launch_bounds__(WGM *WGN * 64)
+__global__ void __launch_bounds__(WGM *WGN * 64, (dma_waves_per_simd<BM, BN, BK, WGM, WGN, NSTAGE>()))
 gemm_dma_kernel(const GemmParams p) {
     constexpr bool A_KC = (LAYOUT != L_TN);
     constexpr bool B_KC = (LAYOUT == L_NT);
@@ -686,24 +696,26 @@ gemm_dmap_kernel(const GemmParams p) {
 }
 
 template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool ACT = false>
-hipError_t launch_gemm_dma(const GemmParams &p, dim3 grid, hipStream_t stream) {
+hipError_t launch_gemm_dma(const GemmParams &p, dim3 grid, hipStream_t stream, KernelQuery *query = nullptr) {
     using TT = DmaTraits<LAYOUT, BM, BN, BK, WGM, WGN, NSTAGE>;
     auto kern = gemm_dma_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, NSTAGE, ACT>;
     static std::atomic<uint64_t> lds_allowed{0};
     hipError_t e = allow_dynamic_lds((const void *)kern, TT::LDS_BYTES, lds_allowed);
     if (e != hipSuccess) return e;
+    if (query) return query_kernel((const void *)kern, TT::NTHREADS, TT::LDS_BYTES, query);
     hipLaunchKernelGGL(kern, grid, dim3(TT::NTHREADS), TT::LDS_BYTES, stream, p);
     return hipGetLastError();
 }
 
 // Persistent launcher: grid.x is the number of resident workgroups the host chose.
 template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, int NSTAGE, bool EPI_LOADS, bool STREAMK>
-hipError_t launch_gemm_dmap(const GemmParams &p, dim3 grid, hipStream_t stream) {
+hipError_t launch_gemm_dmap(const GemmParams &p, dim3 grid, hipStream_t stream, KernelQuery *query = nullptr) {
     using TT = DmaTraits<LAYOUT, BM, BN, BK, WGM, WGN, NSTAGE>;
     auto kern = gemm_dmap_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, NSTAGE, EPI_LOADS, STREAMK>;
     static std::atomic<uint64_t> lds_allowed{0};
     hipError_t e = allow_dynamic_lds((const void *)kern, TT::LDS_BYTES, lds_allowed);
     if (e != hipSuccess) return e;
+    if (query) return query_kernel((const void *)kern, TT::NTHREADS, TT::LDS_BYTES, query);
     hipLaunchKernelGGL(kern, grid, dim3(TT::NTHREADS), TT::LDS_BYTES, stream, p);
     return hipGetLastError();
 }

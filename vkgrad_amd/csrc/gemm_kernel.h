@@ -692,7 +692,26 @@ gemm_kernel(const GemmParams p) {
     store_tile<DT, TM, TN, WTM, WTN, ACT>(p, C, acc, m0, n0, wave_m, wave_n, lane, add_bias, mode, interior);
 }
 
-typedef hipError_t (*launch_fn)(const GemmParams &, dim3 grid, hipStream_t);
+// What the runtime reports for one kernel instantiation on the current device (the counterpart of
+// the reference's Kernel.statistics(), vk.py:690-736): registers, static LDS and scratch from
+// hipFuncGetAttributes, the workgroups of this launch shape a CU holds from the occupancy query.
+struct KernelQuery {
+    hipFuncAttributes attr;
+    int threads;        // workgroup size the launcher uses
+    int dynamic_lds;    // dynamic LDS bytes it asks for
+    int wgs_per_cu;     // hipOccupancyMaxActiveBlocksPerMultiprocessor for that launch shape
+};
+inline hipError_t query_kernel(const void *kern, int threads, int dynamic_lds, KernelQuery *q) {
+    hipError_t e = hipFuncGetAttributes(&q->attr, kern);
+    if (e != hipSuccess) return e;
+    q->threads = threads;
+    q->dynamic_lds = dynamic_lds;
+    q->wgs_per_cu = 0;
+    return hipOccupancyMaxActiveBlocksPerMultiprocessor(&q->wgs_per_cu, kern, threads, (size_t)dynamic_lds);
+}
+
+// A launcher enqueues its kernel, or - with `query` set - only reports on it.
+typedef hipError_t (*launch_fn)(const GemmParams &, dim3 grid, hipStream_t, KernelQuery *query);
 
 // More than 64 KiB of dynamic LDS has to be allowed per kernel and per device; `done`
 // remembers, one bit per device index, where that has happened for the calling launcher.
@@ -709,12 +728,13 @@ inline hipError_t allow_dynamic_lds(const void *kern, int bytes, std::atomic<uin
 }
 
 template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, bool GENERAL, bool ACT = false>
-hipError_t launch_gemm(const GemmParams &p, dim3 grid, hipStream_t stream) {
+hipError_t launch_gemm(const GemmParams &p, dim3 grid, hipStream_t stream, KernelQuery *query = nullptr) {
     using TT = TileTraits<LAYOUT, BM, BN, BK, WGM, WGN>;
     auto kern = gemm_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, GENERAL, ACT>;
     static std::atomic<uint64_t> lds_allowed{0};
     hipError_t e = allow_dynamic_lds((const void *)kern, TT::LDS_BYTES, lds_allowed);
     if (e != hipSuccess) return e;
+    if (query) return query_kernel((const void *)kern, TT::NTHREADS, TT::LDS_BYTES, query);
     hipLaunchKernelGGL(kern, grid, dim3(TT::NTHREADS), TT::LDS_BYTES, stream, p);
     return hipGetLastError();
 }

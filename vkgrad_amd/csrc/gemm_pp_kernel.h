@@ -373,12 +373,13 @@ gemm_pp_kernel(const GemmParams p) {
 }
 
 template <int LAYOUT, int DT, int BM, int BN, int BK, int WGM, int WGN, bool ACT = false>
-hipError_t launch_gemm_pp(const GemmParams &p, dim3 grid, hipStream_t stream) {
+hipError_t launch_gemm_pp(const GemmParams &p, dim3 grid, hipStream_t stream, KernelQuery *query = nullptr) {
     using TT = DmaTraits<LAYOUT, BM, BN, BK, WGM, WGN, 2>;
     auto kern = gemm_pp_kernel<LAYOUT, DT, BM, BN, BK, WGM, WGN, ACT>;
     static std::atomic<uint64_t> lds_allowed{0};
     hipError_t e = allow_dynamic_lds((const void *)kern, TT::LDS_BYTES, lds_allowed);
     if (e != hipSuccess) return e;
+    if (query) return query_kernel((const void *)kern, TT::NTHREADS, TT::LDS_BYTES, query);
     hipLaunchKernelGGL(kern, grid, dim3(TT::NTHREADS), TT::LDS_BYTES, stream, p);
     return hipGetLastError();
 }

@@ -210,10 +210,11 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64, gemv_min_waves(MP, NCH, HALF)
     }
 }
 
-typedef hipError_t (*gemv_launch_fn)(const GemvParams &, dim3 grid, hipStream_t);
+typedef hipError_t (*gemv_launch_fn)(const GemvParams &, dim3 grid, hipStream_t, KernelQuery *query);
 
 template <int DT, int MP, int NCH, bool HALF>
-hipError_t launch_gemv(const GemvParams &p, dim3 grid, hipStream_t stream) {
+hipError_t launch_gemv(const GemvParams &p, dim3 grid, hipStream_t stream, KernelQuery *query = nullptr) {
+    if (query) return query_kernel((const void *)gemv_nt_kernel<DT, MP, NCH, HALF>, GEMV_WAVES * 64, 0, query);
     hipLaunchKernelGGL((gemv_nt_kernel<DT, MP, NCH, HALF>), grid, dim3(GEMV_WAVES * 64), 0, stream, p);
     return hipGetLastError();
 }

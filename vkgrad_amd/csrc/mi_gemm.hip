@@ -171,8 +171,10 @@ static bool dma_eligible(const mg_gemm_args &a, const TileDesc &t, int64_t k_per
         if (a.tri) return false;                   // the unit loop knows nothing of skipped tiles or K ranges
     }
     if (t.persistent == 2 && split > 1) return false;   // stream-K cuts K itself
-    // the 256 x 256 stream-K kernel with the bias epilogue does not fit the register file
+    // the 256 x 256 stream-K kernel with the bias epilogue does not fit the register file, nor does
+    // the persistent 256 x 256 x 64 one in the NN layout (neither is instantiated)
     if (t.persistent == 2 && a.bias && t.bm * t.bn > 128 * 128) return false;
+    if (t.persistent && a.bias && t.bm * t.bn > 128 * 128 && t.bk >= 64 && a.layout == MG_NN) return false;
     return true;
 }
 
@@ -182,7 +184,7 @@ static bool dma_eligible(const mg_gemm_args &a, const TileDesc &t, int64_t k_per
 // {per-workgroup overhead in us, time per K-block in us} by tile and layout NN, NT, TN.
 // It only has to rank candidates; the tuner measures.
 static const float g_cost[MG_NUM_TILES][3][2] = {
-    {{6.63f, 1.813f}, {12.84f, 1.644f}, {5.81f, 1.695f}},   // 0 mm_256x256x64_w2x2
+    {{6.63f, 0.906f}, {12.84f, 0.822f}, {5.81f, 0.848f}},   // 0 mm_256x256x32_w2x4 (half the fitted block time of its 64-wide form)
     {{5.29f, 1.046f}, {12.32f, 0.779f}, {3.73f, 1.029f}},   // 1 mm_256x128x64_w2x2
     {{5.21f, 0.991f}, {11.72f, 0.771f}, {3.63f, 1.042f}},   // 2 mm_128x256x64_w2x2
     {{4.60f, 1.014f}, {7.81f, 0.781f}, {2.82f, 0.975f}},   // 3 mm_128x128x64_w2x2
@@ -747,6 +749,43 @@ int mg_pick(const mg_gemm_args *args, int compute_units, int *tile, int *split_k
     return MG_OK;
 }
 
+static int fill_stats(const KernelQuery &q, mg_kernel_stats *out) {
+    memset(out, 0, sizeof(*out));
+    out->vgprs = q.attr.numRegs;
+    out->scratch_bytes = (int32_t)q.attr.localSizeBytes;
+    out->static_lds_bytes = (int32_t)q.attr.sharedSizeBytes;
+    out->dynamic_lds_bytes = q.dynamic_lds;
+    out->threads = q.threads;
+    out->wgs_per_cu = q.wgs_per_cu;
+    out->waves_per_simd = (q.wgs_per_cu * (q.threads / 64) + 3) / 4;
+    out->max_threads = q.attr.maxThreadsPerBlock;
+    return MG_OK;
+}
+
+int mg_tile_kernel_stats(mg_ctx *ctx, int tile, int layout, int dtype, int variant, mg_kernel_stats *out) {
+    if (!ctx || !out) return fail(MG_ERR_ARG, "mg_tile_kernel_stats: NULL argument");
+    if (tile < 0 || tile >= MG_NUM_TILES) return fail(MG_ERR_ARG, "mg_tile_kernel_stats: unknown tile id %d", tile);
+    if (layout < MG_NN || layout > MG_TN) return fail(MG_ERR_ARG, "mg_tile_kernel_stats: unknown layout %d", layout);
+    if (dtype != MG_F16 && dtype != MG_BF16) return fail(MG_ERR_ARG, "mg_tile_kernel_stats: unknown dtype %d", dtype);
+    HIP_TRY(hipSetDevice(ctx->device));
+    KernelQuery q;
+    memset(&q, 0, sizeof(q));
+    const TileDesc &t = g_tiles[tile];
+    if (t.gemv) {
+        if (layout != MG_NT || variant < 0 || variant >= 16 || !gemv_table[dtype][variant / 4][variant % 4])
+            return fail(MG_ERR_ARG, "mg_tile_kernel_stats: the skinny-M tile has no instantiation %d for this layout", variant);
+        GemvParams g{};
+        HIP_TRY(gemv_table[dtype][variant / 4][variant % 4](g, dim3(1), nullptr, &q));
+        return fill_stats(q, out);
+    }
+    if (variant < 0 || variant > 2) return fail(MG_ERR_ARG, "mg_tile_kernel_stats: variant %d out of range", variant);
+    launch_fn fn = table_for(layout, dtype)[tile][variant];
+    if (!fn) return fail(MG_ERR_ARG, "mg_tile_kernel_stats: tile %d has no variant %d in this layout", tile, variant);
+    GemmParams p{};
+    HIP_TRY(fn(p, dim3(1), nullptr, &q));
+    return fill_stats(q, out);
+}
+
 // Where a GEMM runs and what it may use there: a stream, that stream's share of the split-K
 // workspace (partial tiles and per-tile arrival counters), and the limits of the device.
 struct Lane {
@@ -797,6 +836,15 @@ static int64_t tail_rows(const Lane &ln, const mg_gemm_args &a, const Plan &pl, 
     if (!ln.ws || rest * s * t.bm * t.bn * (int64_t)sizeof(float) > ln.ws_bytes || rest > ln.max_tiles) return 0;
     *slices = (int)s;
     return rows1 * t.bm;
+}
+
+// Which instantiation of a tile serves a call.  Direct-to-LDS tiles: eligibility was settled by
+// the plan; register-staged tiles: the any-alignment instantiation unless every chunk is aligned
+// and whole; persistent tiles: [1] is the epilogue with bias; [2] everywhere the fused activation.
+static int variant_for(const mg_gemm_args &a, const TileDesc &t) {
+    if (t.persistent) return a.bias != nullptr ? 1 : 0;
+    if (a.y16) return 2;
+    return t.nstage > 0 ? 0 : (operands_aligned(a) ? 0 : 1);
 }
 
 static int enqueue_gemm(const Lane &ln, const mg_gemm_args *args, const Plan &pl) {
@@ -861,7 +909,7 @@ static int enqueue_gemm(const Lane &ln, const mg_gemm_args *args, const Plan &pl
         g.sa = p.sa; g.sb = p.sb; g.sc = p.sc;
         g.M = p.M; g.N = p.N; g.K = p.K; g.beta = p.beta;
         const dim3 grid((unsigned)cdiv(a.n, GEMV_ROWS_PER_WG), 1, (unsigned)a.nbatch);
-        hipError_t e = gemv_table[a.dtype][lm][lc](g, grid, stream);
+        hipError_t e = gemv_table[a.dtype][lm][lc](g, grid, stream, nullptr);
         if (e != hipSuccess) return hip_fail(e, "mg_gemm: kernel launch");
         return MG_OK;
     }
@@ -930,14 +978,9 @@ static int enqueue_gemm(const Lane &ln, const mg_gemm_args *args, const Plan &pl
                            p.sc, vec);
         HIP_TRY(hipGetLastError());
     }
-    // direct-to-LDS tiles: eligibility was settled by the plan; register-staged
-    // tiles: the any-alignment instantiation unless every chunk is aligned and whole
-    int general = t.nstage > 0 ? 0 : (operands_aligned(a) ? 0 : 1);
-    if (a.y16) general = 2;   // the variant with the fused activation output
+    int general = variant_for(a, t);
     dim3 grid((unsigned)(pl.grid_m * pl.grid_n), (unsigned)pl.split_k, (unsigned)a.nbatch);
     if (t.persistent) {
-        // resident workgroups loop over (slice, tile) units; [1] = epilogue with bias
-        general = a.bias != nullptr ? 1 : 0;
         const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n;
         const int64_t slots = (int64_t)ln.cus * wgs_per_cu(t, a.layout);
         // stream-K cuts tiles only when the batches together leave resident slots idle: every batch
@@ -966,7 +1009,7 @@ static int enqueue_gemm(const Lane &ln, const mg_gemm_args *args, const Plan &pl
     }
     launch_fn fn = table_for(a.layout, a.dtype)[pl.tile][general];
     if (!fn) return fail(MG_ERR_STATE, "mg_gemm: tile %d has no kernel for this alignment", pl.tile);
-    hipError_t e = fn(p, grid, stream);
+    hipError_t e = fn(p, grid, stream, nullptr);
     if (e != hipSuccess) return hip_fail(e, "mg_gemm: kernel launch");
     return MG_OK;
 }
@@ -981,6 +1024,22 @@ int mg_gemm(mg_ctx *ctx, const mg_gemm_args *args) {
     Plan pl;
     pick_plan(*args, ln.cus, pl);
     return enqueue_gemm(ln, args, pl);
+}
+
+int mg_kernel_stats_for(mg_ctx *ctx, const mg_gemm_args *args, int *tile, mg_kernel_stats *out) {
+    if (!ctx || !out) return fail(MG_ERR_ARG, "mg_kernel_stats_for: NULL argument");
+    int rc = check_args(args);
+    if (rc != MG_OK) return rc;
+    Plan pl;
+    pick_plan(*args, ctx->prop.multiProcessorCount, pl);
+    const TileDesc &t = g_tiles[pl.tile];
+    if (tile) *tile = pl.tile;
+    if (t.gemv) {
+        int lm = 0, lc = 0;
+        if (!gemv_shape(*args, &lm, &lc)) return fail(MG_ERR_STATE, "mg_kernel_stats_for: the skinny-M tile cannot run this call");
+        return mg_tile_kernel_stats(ctx, pl.tile, args->layout, args->dtype, 4 * lm + lc, out);
+    }
+    return mg_tile_kernel_stats(ctx, pl.tile, args->layout, args->dtype, variant_for(*args, t), out);
 }
 
 int mg_gemm_time(mg_ctx *ctx, const mg_gemm_args *args, int repeat, double *seconds) {

@@ -27,7 +27,7 @@
 #pragma once
 
 #define MG_TILE_LIST(V, D, P, S, G, Q) \
-    V(0, 256, 256, 64, 2, 2)       \
+    V(0, 256, 256, 32, 2, 4)       \
     V(1, 256, 128, 64, 2, 2)       \
     V(2, 128, 256, 64, 2, 2)       \
     V(3, 128, 128, 64, 2, 2)       \

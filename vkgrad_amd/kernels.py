@@ -280,6 +280,26 @@ class Matmul:
                self.name)
         return t.value, s.value, g.value
 
+    def statistics(self, m, n, k, nbatch=1, lda=None, ldb=None, ldc=None):
+        """Runtime-reported resource usage of the kernel this Matmul launches for a shape
+        (Kernel.statistics, vk.py:690-736), with the reference's key names where they have a
+        counterpart: numUsedVgprs, ldsUsageSizeInBytes, scratchMemUsageInBytes, plus
+        workgroupThreads, workgroupsPerCU, wavesPerSimd and the tile id that would run."""
+        ga = L.GemmArgs()
+        ga.struct_size = C.sizeof(L.GemmArgs)
+        ga.layout, ga.dtype = self.layout, L.DTYPES[self.dtype]
+        ga.m, ga.n, ga.k = int(m), int(n), int(k)
+        ga.a = ga.b = ga.c = 16     # placeholders: nothing is launched
+        ga.lda = int(lda) if lda is not None else (m if self.trans_a else k)
+        ga.ldb = int(ldb) if ldb is not None else (k if self.trans_b else n)
+        ga.ldc = int(ldc) if ldc is not None else n
+        ga.nbatch, ga.tile = (int(nbatch) if self.batched else 1), self.tile
+        ga.sc = m * ga.ldc
+        ga.split_k, ga.group_m = self.split_k, self.group_m
+        st, tile = L.KernelStats(), C.c_int()
+        _check(self.dev._lib.mg_kernel_stats_for(self.dev._ctx, C.byref(ga), C.byref(tile), C.byref(st)), self.name)
+        return stats_dict(st, tile.value)
+
     def traffic_bytes(self, m, n, k, nbatch=1, bias=False, accumulate=False):
         """Algorithmic (compulsory) bytes: each operand once.  The reference's
         upper bound (kernels.py:299-309) counts per-tile re-reads instead; with
@@ -298,6 +318,41 @@ class Matmul:
 # --------------------------------------------------------------------------
 # autotuner
 # --------------------------------------------------------------------------
+
+def stats_dict(st, tile):
+    return {"numUsedVgprs": st.vgprs, "ldsUsageSizeInBytes": st.static_lds_bytes + st.dynamic_lds_bytes,
+            "scratchMemUsageInBytes": st.scratch_bytes, "workgroupThreads": st.threads,
+            "workgroupsPerCU": st.wgs_per_cu, "wavesPerSimd": st.waves_per_simd, "tile_id": tile}
+
+
+def tile_statistics(dev, tile, layout, dtype="f16", variant=0):
+    """statistics() of one instantiation named directly (tile id, layout MG_NN.., dtype,
+    variant 0 aligned / 1 any alignment or bias epilogue / 2 fused activation); None when the
+    library holds no such instantiation."""
+    st = L.KernelStats()
+    rc = dev._lib.mg_tile_kernel_stats(dev._ctx, int(tile), int(layout), L.DTYPES[dtype], int(variant), C.byref(st))
+    if rc == L.MG_ERR_ARG:
+        return None
+    _check(rc, "tile_statistics")
+    return stats_dict(st, int(tile))
+
+
+def occupancy(dev, stats, workgroup_threads=None, min_waves=1):
+    """Waves resident per SIMD for a compiled kernel, and why it is not worth timing (or
+    None) - the reference's pruning signal (kernels.py:384-411).  There the reason is too
+    few waves to hide DRAM latency on a 12-CU part; the kernels here are built for one or two
+    wavefronts per SIMD with explicit prefetch, so the default bar is one wave, and the
+    reason that does prune is a register spill: a kernel that uses scratch memory turns
+    accumulator traffic into vector memory operations inside the K loop."""
+    waves = stats.get("wavesPerSimd")
+    if not stats.get("numUsedVgprs") or waves is None:
+        return None, None          # unknown: benchmark it rather than guess
+    if stats.get("scratchMemUsageInBytes", 0) > 0:
+        return waves, f"spills {stats['scratchMemUsageInBytes']} bytes of scratch per lane (vgpr={stats['numUsedVgprs']})"
+    if waves < min_waves:
+        return waves, f"only {waves} waves/SIMD (vgpr={stats['numUsedVgprs']})"
+    return waves, None
+
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # Shipped table of tuned picks for MI355X, consulted read-only after the user cache.
@@ -514,6 +569,21 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
                  for at in ((False, True) if s > 1 else (False,))]
         if not cands:
             raise VkError(f"no matmul config fits {m}x{n}x{k}")
+        # resource usage of each candidate's kernel; a spilling one is not timed (kernels.py:478-503)
+        info, pruned = {}, []
+        if sets is not None:
+            kept = []
+            for x in cands:
+                st = x.statistics(m, n, k, nb, lda, ldb, ldc)
+                occ, reason = occupancy(dev, st)
+                info[id(x)] = (st["numUsedVgprs"], occ)
+                if reason:
+                    pruned.append((x.tile, x.split_k, reason))
+                    if verbose:
+                        print(f"    tile {x.bm:3d}x{x.bn:3d} split_k={x.split_k:2d}  pruned: {reason}")
+                else:
+                    kept.append(x)
+            cands = kept or cands
 
         def measure(mms):
             warm = {id(x): timer(x, 1) for x in mms}
@@ -531,9 +601,12 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
             tf = x.flops(m, n, k) * nb / t / 1e12
             results.append({"config": [x.bm, x.bn, x.bk], "lds": True, "tflops": tf, "ms": t * 1e3,
                             "tile": [x.bm, x.bn], "tile_id": x.tile, "split_k": x.split_k,
-                            "atomic_split": x.atomic_split})
+                            "atomic_split": x.atomic_split, "vgpr": info.get(id(x), (None, None))[0],
+                            "occupancy": info.get(id(x), (None, None))[1]})
             if verbose:
-                print(f"    tile {x.bm:3d}x{x.bn:3d} split_k={x.split_k:2d}  {tf:8.2f} TFLOPS  {t * 1e6:9.1f} us")
+                v, o = info.get(id(x), (None, None))
+                print(f"    tile {x.bm:3d}x{x.bn:3d} id={x.tile:2d} split_k={x.split_k:2d}{' at' if x.atomic_split else '   '}  "
+                      f"{tf:8.2f} TFLOPS  {t * 1e6:9.1f} us  vgpr={v or '?'} waves={o or '?'}")
         results.sort(key=lambda r: -r["tflops"])
         best = dict(results[0])
 
@@ -548,6 +621,7 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
         tf, g = scored[0]
         best.update(tflops=tf, ms=2.0 * m * n * k * nb / tf / 1e9, group_m=g)
         best["pruned"] = len(CONFIGS) * 1 - len({c.tile for c in cands})
+        best["spilling"] = [list(x) for x in pruned]
         best["evaluated"] = len(results)
         if use_cache:
             cache = _load_cache()
