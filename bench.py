@@ -141,27 +141,83 @@ def cpu_baseline(min_seconds=10.0):
     except AttributeError:
         cores = os.cpu_count() or 1
     threads = int(os.environ.get("OPENBLAS_NUM_THREADS") or os.environ.get("OMP_NUM_THREADS") or cores)
+    mlp = cpu_mlp_step()
     return {"value": round(flops / secs / 1e12, 4), "unit": "TFLOP/s", "cores": min(threads, cores),
-            "kind": "port",
+            "kind": "port", "mnist_mlp_step_ms": mlp,
             "sample": f"{steps} whole steps of the benchmark workload (147 GEMMs, 6.07 TFLOP each), numpy float32 matmul "
                       f"of bf16-rounded operands, {secs:.1f} s of matmul time"}
 
 
+MLP_SIZES, MLP_BATCH, MLP_CLASSES = (784, 512, 512), 128, 10
+
+
+def mlp_step_device(dev, steps=300):
+    """BASELINE configs[0] on the device: the synthetic-MNIST MLP train step (batch 128, 784 ->
+    512 -> 512 -> 10, ReLU, He-normal weights, f16, fwd + dX + dW + bias gradients + AdamW)
+    recorded once and replayed as one HIP graph; microseconds per step including the read-back
+    of the loss, as the reference's TrainStep measures it (bench/mnist-repro.json:5-24)."""
+    from vkgrad_amd.autograd import AdamW, Ctx, MLP, TrainStep
+    rng = np.random.default_rng(0)
+    ctx = Ctx(dev, dtype="f16", fuse_bias=True)
+    try:
+        model = MLP(ctx, MLP_BATCH, list(MLP_SIZES), MLP_CLASSES, pad_classes=MLP_CLASSES, activation="relu")
+        widths = list(MLP_SIZES) + [MLP_CLASSES]
+        for layer, fin, fout in zip(model.layers, widths[:-1], widths[1:]):
+            layer.W.set((rng.standard_normal((fin, fout)) * np.sqrt(2.0 / fin)).astype(np.float32))
+            layer.b.set(np.zeros(fout, np.float32))
+        xb = ctx.buf(MLP_BATCH * MLP_SIZES[0] * 2, "shared")
+        xb.array(np.float16, (MLP_BATCH, MLP_SIZES[0]))[:] = rng.random((MLP_BATCH, MLP_SIZES[0]),
+                                                                        dtype=np.float32).astype(np.float16)
+        yb = ctx.buf(MLP_BATCH * 4, "shared")
+        yb.array(np.uint32, (MLP_BATCH,))[:] = rng.integers(0, MLP_CLASSES, MLP_BATCH)
+        step = TrainStep(model, AdamW(ctx, model.params(), lr=1e-3), xb, yb)
+        first = step()[0]
+        for _ in range(20):
+            step()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            loss, _ = step()
+        dt = (time.perf_counter() - t0) / steps
+        return {"us_per_step": round(dt * 1e6, 1), "kernels_per_step": step.n_dispatch, "steps": steps,
+                "loss_first": round(float(first), 4), "loss_last": round(float(loss), 4),
+                "what": "graph replay + loss read-back, batch 128, 784-512-512-10, ReLU, f16, AdamW"}
+    finally:
+        ctx.destroy()
+
+
+def cpu_mlp_step(steps=30):
+    """The numpy model of the configs[0] train step (oracle/ref_mlp.py, the restatement of the
+    reference's numpy path) on this host: milliseconds per step."""
+    from oracle import ref_mlp
+    Ws, bs = ref_mlp.he_init(list(MLP_SIZES) + [MLP_CLASSES], 0)
+    ref = ref_mlp.RefMLP(MLP_SIZES, MLP_CLASSES, MLP_CLASSES, act="relu", dtype="f16")
+    ref.set_params(Ws, bs)
+    _, xf, y = ref_mlp.synthetic_batch(MLP_BATCH, MLP_SIZES[0], MLP_CLASSES, 0, "f16")
+    for _ in range(3):
+        ref.train_step(xf, y, lr=1e-3)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ref.train_step(xf, y, lr=1e-3)
+    return round((time.perf_counter() - t0) / steps * 1e3, 3)
+
+
 def other_workloads(dev):
     """Compact figures for the workloads the headline does not cover (the reference's
-    bench/matmul_sweep.py:60-107 writes one record with every size): the largest square
-    of configs[1] in the three layouts, one optimiser step of the d_model-1024 decoder of
-    configs[3] (every distinct GEMM timed, weighted by its count), and the two skinniest
-    memory-bound cases of configs[4].  Median of 3 batches of >= 10 ms each per GEMM."""
+    bench/matmul_sweep.py:60-107 writes one record with every size): the MLP train step of
+    configs[0], the squares of configs[1] in the three layouts (8192^3 timed over batches of
+    >= 0.1 s so that it runs at the sustained clock), one optimiser step of the d_model-1024
+    decoder of configs[3] (every distinct GEMM timed, weighted by its count), the char-LM
+    GEMMs of configs[4] and its N = 50257 skinny rows.  Median of the batches per GEMM."""
     from vkgrad_amd import sweep
     r = sweep.Runner(dev=dev, warm=False)
-    out = {}
+    out = {"mnist_mlp_step_f16": mlp_step_device(dev)}
     sq = {}
     for c in sweep.cases_for("square"):
-        if c["m"] == 8192:
-            row = r.time_case(c, samples=3, min_seconds=0.01)
-            sq[c["layout"]] = {"tflops": row["tflops"], "frac_mfma": row["frac_mfma"], "us": row["us"], "tile": row["tile"]}
-    out["square_8192_f16"] = sq
+        big = c["m"] == 8192
+        row = r.time_case(c, samples=4 if big else 3, min_seconds=0.1 if big else 0.01)
+        sq.setdefault(str(c["m"]), {})[c["layout"]] = {"tflops": row["tflops"], "frac_mfma": row["frac_mfma"],
+                                                       "us": row["us"], "tile": row["tile"]}
+    out["square_f16"] = sq
     rows = [r.time_case(c, samples=3, min_seconds=0.01) for c in sweep.cases_for("decoder")]
     us = sum(x["us"] * x["count"] for x in rows)
     fl = sum(2.0 * x["m"] * x["n"] * x["k"] * x["count"] for x in rows)
@@ -169,9 +225,14 @@ def other_workloads(dev):
         "gemms": sum(x["count"] for x in rows), "tflop": round(fl / 1e12, 2), "gemm_ms": round(us / 1e3, 2),
         "tflops": round(fl / us / 1e6, 1), "frac_mfma": round(fl / us / 1e6 / PEAK_TFLOPS, 4),
         "dw": "beta = 1 over 4 micro-batches (the first overwrites)"}
+    rows = [r.time_case(c, samples=3, min_seconds=0.005) for c in sweep.cases_for("charlm")]
+    us = sum(x["us"] for x in rows)
+    fl = sum(2.0 * x["m"] * x["n"] * x["k"] for x in rows)
+    out["charlm_gemms_f16"] = {"gemms": len(rows), "total_us": round(us, 1), "tflops": round(fl / us / 1e6, 1),
+                               "what": "d_model 256, vocabulary 96, 16384 rows: fwd + dX + dW of 5 linears"}
     sk = {}
     for c in sweep.cases_for("skinny"):
-        if c["n"] == VOCAB and c["m"] in (1, 7):
+        if c["n"] == VOCAB:
             row = r.time_case(c, samples=3, min_seconds=0.01)
             sk[f"{c['m']}x{c['n']}x{c['k']}"] = {"us": row["us"], "gbps": row["gbps"], "frac_hbm": row["frac_hbm"],
                                                  "tile": row["tile"]}
@@ -376,7 +437,7 @@ def main():
     tflops = step_flops / (dt / args.steps) / 1e12
 
     # Per-shape launch durations with HIP events on the library's stream
-    # (mg_gemm_time_rotating): best of 3 batches of back-to-back launches that rotate
+    # (mg_gemm_time_rotating): median of 5 batches of back-to-back launches that rotate
     # through the step's buffer sets, so a layer GEMM reads its operands from HBM as
     # it does inside the step.
     per_shape = []
@@ -388,12 +449,14 @@ def main():
         rot = [tuple(g[x] for x in role_bufs[role]) for g in groups]
         t1 = mm.time_rotating(rot, m, n, k, repeat=len(rot), **kw) / len(rot)
         rep = max(1, int(0.02 / max(t1, 1e-6)) // len(rot)) * len(rot)
-        sec = min(mm.time_rotating(rot, m, n, k, repeat=rep, **kw) / rep for _ in range(3))
+        secs = sorted(mm.time_rotating(rot, m, n, k, repeat=rep, **kw) / rep for _ in range(5))
+        sec = secs[2]
         fl = 2.0 * m * n * k
         by = 2.0 * (m * k + k * n) + 4.0 * m * n
         tile, split, gm = mm.plan(m, n, k, **kw)
         per_shape.append({"gemm": name, "layout": layout, "m": m, "n": n, "k": k, "count": count,
-                          "us": round(sec * 1e6, 2), "tflops": round(fl / sec / 1e12, 1),
+                          "us": round(sec * 1e6, 2), "us_min": round(secs[0] * 1e6, 2), "us_max": round(secs[-1] * 1e6, 2),
+                          "tflops": round(fl / sec / 1e12, 1),
                           "frac_mfma": round(fl / sec / 1e12 / PEAK_TFLOPS, 4),
                           "gbps": round(by / sec / 1e9, 1), "tile": tile, "split_k": split})
     dom = max(per_shape, key=lambda r: r["us"] * r["count"])

@@ -94,15 +94,20 @@ def _run_mm(dev, mm, a, b, m, n, k, lda=None, ldb=None, ldc=None, c_in=None, nba
 # ---------------------------------------------------------------------------
 
 def _bench_cases():
+    """Every GEMM of the benchmark step, and the three LM-head GEMMs once more with logits
+    rows exactly 50257 elements apart (the step bench.py reports as `dense_head`)."""
     import bench
-    return [(name, layout, m, n, k) for name, layout, m, n, k, _ in bench.gemm_list()]
+    cases = [(name, layout, m, n, k, False) for name, layout, m, n, k, _ in bench.gemm_list()]
+    return cases + [c[:5] + (True,) for c in cases if c[0].startswith("head")]
 
 
-@pytest.mark.parametrize("name,layout,m,n,k", _bench_cases(), ids=[c[0] for c in _bench_cases()])
-def test_benchmark_plan_at_full_size(dev, name, layout, m, n, k):
+@pytest.mark.parametrize("name,layout,m,n,k,dense", _bench_cases(),
+                         ids=[c[0] + (".dense" if c[5] else "") for c in _bench_cases()])
+def test_benchmark_plan_at_full_size(dev, name, layout, m, n, k, dense):
     import bench
-    vpitch = bench.head_pitch(False)
+    vpitch = bench.head_pitch(dense)
     mm, kw = bench.plan_for(dev, name, layout, m, n, k, vpitch)
+    assert (kw == {}) == (dense or not name.startswith("head"))
     if os.path.exists(os.path.join(ROOT, "vkgrad_amd", "tuned_mi355x.json")) and dev.name.startswith("gfx950"):
         assert mm.tile >= 0, f"{name}: the tuned table has no plan for this shape (the benchmark would run the picker)"
     ta, tb = LAY[layout]
@@ -117,16 +122,6 @@ def test_benchmark_plan_at_full_size(dev, name, layout, m, n, k):
     _sample_check(got, a, b, m, n, k, ta, tb, "bf16")
     _checksum_check(got, a, b, ta, tb, "bf16")
     mm.destroy()
-
-
-def test_benchmark_step_has_a_plan_for_the_dense_head_too(dev):
-    """bench.py also reports the step with logits rows exactly 50257 elements apart."""
-    import bench
-    for name, layout, m, n, k, _ in bench.gemm_list():
-        if name.startswith("head"):
-            mm, kw = bench.plan_for(dev, name, layout, m, n, k, VOCAB)
-            assert kw == {}
-            mm.destroy()
 
 
 # ---------------------------------------------------------------------------
