@@ -459,6 +459,22 @@ def main():
                           "tflops": round(fl / sec / 1e12, 1),
                           "frac_mfma": round(fl / sec / 1e12 / PEAK_TFLOPS, 4),
                           "gbps": round(by / sec / 1e9, 1), "tile": tile, "split_k": split})
+    # The same GEMMs timed inside the step: the step's calls in order, eagerly, a HIP event behind
+    # each (mg_gemm_time_each); per GEMM the median over its occurrences in 5 passes.
+    from vkgrad_amd.kernels import time_sequence
+    order = [f"{nm}.{role}" for _ in range(LAYERS) for nm, _, _ in LINEARS for role in ("fwd", "dX", "dW")]
+    order += ["head.fwd", "head.dX", "head.dW"]
+    time_sequence(dev, calls)
+    seen, passes = {}, []
+    for _ in range(5):
+        one_pass = time_sequence(dev, calls)
+        passes.append(sum(one_pass))
+        for nm, t in zip(order, one_pass):
+            seen.setdefault(nm, []).append(t)
+    for r in per_shape:
+        ts = sorted(seen[r["gemm"]])
+        r["us_in_step"] = round(ts[len(ts) // 2] * 1e6, 2)
+    in_step_ms = sorted(passes)[2] * 1e3
     dom = max(per_shape, key=lambda r: r["us"] * r["count"])
     mt = MEASURED_TRAFFIC.get(dom["gemm"])
     traffic = None
@@ -487,6 +503,7 @@ def main():
         "frac_of_mfma_peak": round(tflops / PEAK_TFLOPS, 4),
         "sustained_warmup_s": round(warm_s, 2),
         "sum_of_event_timed_gemms_ms": round(events_ms, 4),
+        "step_with_an_event_after_every_gemm_ms": round(in_step_ms, 4),
         "roofline": roofline,
         "device": {"name": dev.name, "compute_units": dev.compute_units, "clock_khz": dev.clock_khz,
                    "derived_peak_tflops": round(dev.compute_units * 4 * 1024 * dev.clock_khz * 1e3 / 1e12, 1)},

@@ -140,7 +140,9 @@ typedef struct {
  * context's workspace and are summed in slice order by the slice that finishes last: no
  * clear of C, bit-reproducible.  This flag makes them add into C with float atomics instead
  * (after a clear kernel when beta == 0), which is also what happens when the partial tiles
- * do not fit the workspace; it can be faster when C is large and the split is deep. */
+ * do not fit the workspace; it can be faster when C is large and the split is deep.  A call
+ * with this flag uses no workspace at all: the library does not cut a partial last round of
+ * tiles into K slices for it either, and a stream-K tile runs as a plain persistent one. */
 #define MG_FLAG_SPLITK_ATOMIC 2
 /* Run this GEMM on the context's side stream (see mg_side_fork): it overlaps with whatever the
  * main stream runs until mg_side_join.  The side stream has its own half of the split-K
@@ -219,21 +221,51 @@ int mg_gemm_time(mg_ctx *ctx, const mg_gemm_args *args, int repeat, double *seco
  * reference times a shape on one set of buffers (kernels.py:433-447), which on
  * this chip would time small shapes out of cache. */
 int mg_gemm_time_rotating(mg_ctx *ctx, const mg_gemm_args *args, int nargs, int repeat, double *seconds);
+/* A whole sequence of different GEMMs (1..4096), each behind the previous one on the context's
+ * stream with a HIP event between them: seconds_each[i] is the time from the end of GEMM i - 1
+ * to the end of GEMM i, i.e. what GEMM i costs inside the sequence, launch gap included.  The
+ * reference times dispatches one at a time (Device.run, vk.py:1295-1340) and has no
+ * in-sequence timer; this one shows what a training step's order costs each GEMM. */
+int mg_gemm_time_each(mg_ctx *ctx, const mg_gemm_args *args, int nargs, double *seconds_each);
 /* No counterpart in the reference.  mg_gemm for callers that cannot allocate device memory or
  * create a context: code under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc.  Same arguments and results as mg_gemm (bit-identical: the same kernels and plans),
- * on device `device_index` and on `hip_stream` (a hipStream_t, NULL for the default stream),
- * which the caller owns and synchronises.  It calls no hipMalloc / hipFree and needs no mg_ctx:
- * the K slices of a split meet in a workspace that is part of the library's image on every
- * device, MG_STATIC_WS_BYTES of partial tiles and MG_STATIC_MAX_TILES arrival counters, which
- * each GPU holds until the process ends.  A GEMM whose K split needs more than that is refused
- * with MG_ERR_ARG (nothing is launched); MG_FLAG_SPLITK_ATOMIC, split_k = 1 or mg_gemm are the
- * ways out.  MG_FLAG_SIDE_STREAM is refused.  All calls on one GPU share the one workspace:
- * calls that may overlap on a GPU (two streams, two threads) race on it - keep them on one
- * stream or give every concurrent caller but one split_k = 1. */
+ * hipMalloc.  Same arguments, kernels and plans as mg_gemm, on device `device_index` and on
+ * `hip_stream` (a hipStream_t, NULL for the default stream), which the caller owns and
+ * synchronises; the caller's current device is left as it was.  It calls no hipMalloc /
+ * hipFree and needs no mg_ctx: the K slices of a split meet in a workspace that is part of the
+ * library's image on every device, MG_STATIC_WS_BYTES of partial tiles and MG_STATIC_MAX_TILES
+ * arrival counters, which each GPU holds until the process ends.
+ *   Results are those of mg_gemm bit for bit whenever both take the same plan, which is always
+ * the case for an explicit tile and split_k whose partial tiles fit MG_STATIC_WS_BYTES.  Where
+ * the library itself decides to use its workspace - a partial last round of ping-pong tiles cut
+ * into K slices, the K pieces of a stream-K tile - that decision depends on what fits, so a
+ * shape whose partial tiles need between 32 MiB and the context's workspace is summed in a
+ * different order here (same values on integer data, within tolerance otherwise): a stream-K
+ * tile then runs as a plain persistent one and the partial round stays uncut.
+ *   A K split that the caller or the picker chose and whose partial tiles or counters do not
+ * fit is refused with MG_ERR_ARG (nothing is launched); MG_FLAG_SPLITK_ATOMIC, a smaller
+ * split_k or mg_gemm are the ways out.  MG_FLAG_SIDE_STREAM is refused.
+ *   All calls on one GPU share the one workspace, which keeps what the last call left: the
+ * counters a launch uses are cleared by a fill kernel in front of it, and calls that may
+ * overlap on a GPU (two streams, two threads) race on it.  Keep them on one stream, or pass
+ * MG_FLAG_SPLITK_ATOMIC on every concurrent call but one: with that flag a call touches
+ * neither the partial tiles nor the counters (its slices add into C with atomics, a partial
+ * round is not cut, a stream-K tile runs plain).
+ *   Under stream capture: the first call on a device looks up the workspace address and the
+ * device's limits and raises the dynamic-LDS limit of the kernel it launches, which the
+ * runtime may refuse while a capture is under way - make one call of the same tile, layout and
+ * dtype outside the capture first. */
 #define MG_STATIC_WS_BYTES (32ll << 20)
 #define MG_STATIC_MAX_TILES 16384
 int mg_gemm_static(int device_index, void *hip_stream, const mg_gemm_args *args);
+/* How many kernels mg_gemm_static would launch for `args` (GEMM kernels, counter clears, the
+ * clear of C before an atomic split); launches nothing. */
+int mg_gemm_static_launches(int device_index, const mg_gemm_args *args, int *kernels);
+/* The same question without a device, for a lane described by its numbers: CUs, bytes of
+ * partial-tile workspace (0: none), arrival counters, and whether counters are cleared in front
+ * of a launch (1 for a workspace that persists between calls).  Pure arithmetic. */
+int mg_launch_count(const mg_gemm_args *args, int compute_units, int64_t workspace_bytes, int64_t counters,
+                    int clear_counters, int *kernels);
 /* What the matrix cores sustain with no memory traffic: two wavefronts per SIMD on every CU run
  * `iters` rounds of eight back-to-back v_mfma_f32_32x32x16 from registers.  random_operands = 0
  * multiplies zeros (the chip holds its boost clock), 1 multiplies random 16-bit values (the

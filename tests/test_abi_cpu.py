@@ -397,3 +397,68 @@ def test_graph_refuses_replay_after_a_buffer_was_destroyed():
     g2 = Graph(FakeDev(), "g2")
     with pytest.raises(VkError, match="destroyed"):
         g2.record(lambda: None, [dead], name="k")
+
+
+def _tiles(lib):
+    out = []
+    for i in range(lib.mg_tile_count()):
+        t = L.Tile()
+        assert lib.mg_tile_info(i, C.byref(t)) == L.MG_OK
+        out.append(dict(id=t.id, name=t.name.decode(), fallback=t.fallback))
+    return out
+
+
+def _count(lib, ga, ws_mb, counters=1 << 18, clear=0, cus=256):
+    n = C.c_int(-1)
+    assert lib.mg_launch_count(C.byref(ga), cus, int(ws_mb) << 20, counters, clear, C.byref(n)) == L.MG_OK, L.last_error()
+    return n.value
+
+
+def test_atomic_flag_keeps_a_call_off_the_workspace(lib):
+    """What include/mi_gemm.h promises concurrent callers: with MG_FLAG_SPLITK_ATOMIC a call
+    touches neither partial tiles nor counters.  Counted without a device (mg_launch_count):
+    the ping-pong tile with a partial last round records two GEMM launches when it may use the
+    workspace (whole rounds unsplit, the rest cut into K slices) and one with the flag; a
+    stream-K tile and an explicit split record no counter clear with the flag."""
+    pp = next(t["id"] for t in _tiles(lib) if t["name"].startswith("mmq_"))
+    sk = next(t["id"] for t in _tiles(lib) if t["name"].startswith("mmk_128"))
+    # 50257 x 768 x 8192 TN: 591 tiles of 256 x 256 on 256 CUs, the LM-head dW of the benchmark
+    ga = good_args(layout=L.MG_TN, dtype=L.MG_BF16, m=50257, n=768, k=8192, lda=50304, ldb=768, ldc=768, tile=pp, split_k=1)
+    assert _count(lib, ga, 256) == 2
+    assert _count(lib, ga, 256, clear=1) == 3          # + the clear of the tail's counters
+    assert _count(lib, ga, 32, clear=1) == 1           # 81 tiles x 3 slices x 256 KiB do not fit 32 MiB: no cut
+    assert _count(lib, ga, 0) == 1
+    ga.flags = L.MG_FLAG_SPLITK_ATOMIC
+    assert _count(lib, ga, 256, clear=1) == 1
+    # explicit split: slices meet in the workspace (clear + GEMM), or add atomically (clear of C + GEMM)
+    ga = good_args(layout=L.MG_TN, dtype=L.MG_BF16, m=768, n=768, k=8192, lda=768, ldb=768, ldc=768, tile=pp, split_k=4)
+    assert _count(lib, ga, 256, clear=1) == 2 and _count(lib, ga, 256, clear=0) == 1
+    ga.flags = L.MG_FLAG_SPLITK_ATOMIC
+    assert _count(lib, ga, 256, clear=1) == 2          # zero_c + GEMM, no counter clear
+    ga.beta = 1
+    assert _count(lib, ga, 256, clear=1) == 1
+    # stream-K tile: pieces meet in the workspace unless the flag forbids it
+    ga = good_args(layout=L.MG_NN, dtype=L.MG_BF16, m=8192, n=1152, k=2304, lda=2304, ldb=1152, ldc=1152, tile=sk, split_k=1)
+    assert _count(lib, ga, 256, clear=1) == 2
+    ga.flags = L.MG_FLAG_SPLITK_ATOMIC
+    assert _count(lib, ga, 256, clear=1) == 1
+
+
+def test_ping_pong_tile_is_refused_where_its_lane_offsets_would_overflow(lib):
+    """The ping-pong kernel addresses a lane's load as scalar base + 32-bit offset; a row pitch
+    that pushes 7 rows (K-contiguous) or 1 row (M/N-contiguous) past 2^32 bytes must fall back."""
+    tiles = _tiles(lib)
+    pp = next(t for t in tiles if t["name"].startswith("mmq_"))
+    def picked(**kw):
+        ga = good_args(dtype=L.MG_BF16, tile=pp["id"], split_k=1, **kw)
+        t, s, g = C.c_int(), C.c_int(), C.c_int()
+        assert lib.mg_pick(C.byref(ga), 256, C.byref(t), C.byref(s), C.byref(g)) == L.MG_OK, L.last_error()
+        return t.value
+    ok_ld = 300_000_000         # 7 * ld * 2 + 128 < 2^32
+    bad_ld = 310_000_000        # >= 2^32
+    assert picked(layout=L.MG_NT, m=512, n=512, k=512, lda=ok_ld, ldb=512, ldc=512) == pp["id"]
+    assert picked(layout=L.MG_NT, m=512, n=512, k=512, lda=bad_ld, ldb=512, ldc=512) == pp["fallback"]
+    assert picked(layout=L.MG_NT, m=512, n=512, k=512, lda=512, ldb=bad_ld, ldc=512) == pp["fallback"]
+    # M/N-contiguous operand: one row of pitch
+    assert picked(layout=L.MG_TN, m=512, n=512, k=512, lda=2_000_000_000, ldb=512, ldc=512) == pp["id"]
+    assert picked(layout=L.MG_TN, m=512, n=512, k=512, lda=2_147_483_400, ldb=512, ldc=512) == pp["fallback"]

@@ -1,10 +1,12 @@
 """mg_gemm_static: the GEMM entry point that allocates nothing (no context, the caller's
 stream, K slices meeting in a workspace that is part of the library's image).
 
-It must give what mg_gemm gives, bit for bit (same kernels, same plans, and the workspace
-split sums its slices in slice order), on two calls in a row - the second on a smaller
-problem, so that whatever the first left in the shared workspace and its counters shows if
-it is not cleared - and must refuse a K split that needs more than the static workspace.
+It must give what mg_gemm gives, bit for bit where both take the same plan (same kernels, and
+the workspace split sums its slices in slice order), on two calls in a row - the second on a
+smaller problem, so that whatever the first left in the shared workspace and its counters
+shows if it is not cleared - must refuse a K split that needs more than the static workspace,
+must clear the counters of the launches the library splits by itself, and must work when
+captured into a graph on a stream the caller owns.
 Collected last (by its file name), so a failure here hides no other test.
 """
 
@@ -107,3 +109,121 @@ def test_static_entry_point_refuses_what_does_not_fit(dev):
         mm.destroy()
         for x in (ba, bb, bc):
             x.destroy()
+
+
+def test_static_ping_pong_partial_round_and_dirty_counters(dev):
+    """The ping-pong tile with a partial last round: the library cuts the remaining tile rows
+    into K slices that meet in the workspace, and that second launch is planned unsplit at the
+    top level - its counters must be cleared all the same.  Integer data, exact against the
+    oracle, after another split call has used the workspace and twice in a row."""
+    from vkgrad_amd import _lib as L
+    from vkgrad_amd.kernels import Matmul
+    lib = dev._lib
+    # 67 x 4 = 268 tiles of 256 x 256 on 256 CUs: one whole round and 12 tiles more, cut into 8
+    # K slices of 8 K-blocks each (24 MiB of partial tiles: fits the static workspace)
+    m, n, k = 67 * 256, 1024, 4096
+    a, b = O.make_operands(m, n, k, True, False, "bf16", 41, integer=True)
+    ba, bb, bc = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), dev.buffer(m * n * 4, "device")
+    mm = Matmul(dev, trans_a=True, dtype="bf16", tile=21, split_k=1)
+    try:
+        ba.upload(a)
+        bb.upload(b)
+        ga = mm._args(ba, bb, bc, m, n, k, 1, (0, 0, 0), None, False, None, None, None)
+        nk = C.c_int()
+        assert lib.mg_gemm_static_launches(0, C.byref(ga), C.byref(nk)) == L.MG_OK, L.last_error()
+        if dev.compute_units == 256:
+            assert nk.value == 3, nk.value      # whole rounds, clear of the tail's counters, the tail's slices
+        # a split call on a small problem first: it leaves its partial tiles in the workspace
+        small = Matmul(dev, trans_a=True, dtype="bf16", tile=11, split_k=2)
+        sa, sb = O.make_operands(128, 128, 256, True, False, "bf16", 42, integer=True)
+        bsa, bsb, bsc = dev.buffer(sa.nbytes, "device"), dev.buffer(sb.nbytes, "device"), dev.buffer(128 * 128 * 4, "device")
+        bsa.upload(sa)
+        bsb.upload(sb)
+        gs = small._args(bsa, bsb, bsc, 128, 128, 256, 1, (0, 0, 0), None, False, None, None, None)
+        assert lib.mg_gemm_static(0, None, C.byref(gs)) == L.MG_OK, L.last_error()
+        for _ in range(2):                      # twice: the second finds what the first left
+            bc.upload(np.full((m, n), np.nan, np.float32))
+            assert lib.mg_gemm_static(0, None, C.byref(ga)) == L.MG_OK, L.last_error()
+            assert _hip().hipDeviceSynchronize() == 0
+            got = bc.download(np.float32, (m, n))
+            assert np.array_equal(got, O.ref_gemm(a, b, True, False, "bf16"))
+        # with the atomic flag the same call is one launch and touches no workspace
+        ga.flags |= L.MG_FLAG_SPLITK_ATOMIC
+        assert lib.mg_gemm_static_launches(0, C.byref(ga), C.byref(nk)) == L.MG_OK and nk.value == 1
+        bc.upload(np.full((m, n), np.nan, np.float32))
+        assert lib.mg_gemm_static(0, None, C.byref(ga)) == L.MG_OK, L.last_error()
+        assert _hip().hipDeviceSynchronize() == 0
+        assert np.array_equal(bc.download(np.float32, (m, n)), O.ref_gemm(a, b, True, False, "bf16"))
+        small.destroy()
+        for x in (bsa, bsb, bsc):
+            x.destroy()
+    finally:
+        mm.destroy()
+        for x in (ba, bb, bc):
+            x.destroy()
+
+
+def test_static_entry_point_under_stream_capture(dev):
+    """What the entry point is for: after one priming call outside the capture, a split and an
+    unsplit GEMM are captured on a stream the caller owns, instantiated as a graph and replayed
+    twice, with eager work and synchronisations between the replays; every replay is exact
+    against the oracle, and the caller's current device is left alone."""
+    from vkgrad_amd import _lib as L
+    from vkgrad_amd.kernels import Matmul
+    lib, hip = dev._lib, _hip()
+    hip.hipStreamCreate.argtypes = [C.POINTER(C.c_void_p)]
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip.hipStreamSynchronize.argtypes = [C.c_void_p]
+    hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+    hip.hipGraphDestroy.argtypes = [C.c_void_p]
+    hip.hipStreamDestroy.argtypes = [C.c_void_p]
+    hip.hipGetDevice.argtypes = [C.POINTER(C.c_int)]
+    cases = [(768, 512, 4096, True, False, 11, 4), (300, 264, 520, False, True, 11, 1)]   # split, unsplit
+    bufs, mms, gas, refs = [], [], [], []
+    for i, (m, n, k, ta, tb, tile, split) in enumerate(cases):
+        a, b = O.make_operands(m, n, k, ta, tb, "bf16", 50 + i, integer=True)
+        ba, bb, bc = dev.buffer(a.nbytes, "device"), dev.buffer(b.nbytes, "device"), dev.buffer(m * n * 4, "device")
+        ba.upload(a)
+        bb.upload(b)
+        mm = Matmul(dev, trans_a=ta, trans_b=tb, dtype="bf16", tile=tile, split_k=split)
+        gas.append(mm._args(ba, bb, bc, m, n, k, 1, (0, 0, 0), None, False, None, None, None))
+        bufs.append((ba, bb, bc, m, n))
+        mms.append(mm)
+        refs.append(O.ref_gemm(a, b, ta, tb, "bf16"))
+    stream, graph, gexec = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    try:
+        before = C.c_int(-1)
+        assert hip.hipGetDevice(C.byref(before)) == 0
+        for ga in gas:                                       # priming calls, outside the capture
+            assert lib.mg_gemm_static(0, None, C.byref(ga)) == L.MG_OK, L.last_error()
+        assert hip.hipDeviceSynchronize() == 0
+        assert hip.hipStreamCreate(C.byref(stream)) == 0
+        assert hip.hipStreamBeginCapture(stream, 2) == 0     # hipStreamCaptureModeRelaxed
+        for ga in gas:
+            assert lib.mg_gemm_static(0, stream, C.byref(ga)) == L.MG_OK, L.last_error()
+        assert hip.hipStreamEndCapture(stream, C.byref(graph)) == 0
+        assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+        after = C.c_int(-2)
+        assert hip.hipGetDevice(C.byref(after)) == 0 and after.value == before.value
+        for replay in range(3):
+            for ba, bb, bc, m, n in bufs:
+                bc.upload(np.full((m, n), np.nan, np.float32))      # eager work between the replays
+            assert hip.hipGraphLaunch(gexec, stream) == 0
+            assert hip.hipStreamSynchronize(stream) == 0
+            for (ba, bb, bc, m, n), ref in zip(bufs, refs):
+                assert np.array_equal(bc.download(np.float32, (m, n)), ref), f"replay {replay}"
+    finally:
+        if gexec:
+            hip.hipGraphExecDestroy(gexec)
+        if graph:
+            hip.hipGraphDestroy(graph)
+        if stream:
+            hip.hipStreamDestroy(stream)
+        for mm in mms:
+            mm.destroy()
+        for ba, bb, bc, m, n in bufs:
+            for x in (ba, bb, bc):
+                x.destroy()

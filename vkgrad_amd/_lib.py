@@ -94,10 +94,13 @@ SIGNATURES = {
     "mg_gemm_check": (C.c_int, [C.POINTER(GemmArgs)]),
     "mg_gemm": (C.c_int, [_P, C.POINTER(GemmArgs)]),
     "mg_gemm_static": (C.c_int, [C.c_int, _P, C.POINTER(GemmArgs)]),
+    "mg_gemm_static_launches": (C.c_int, [C.c_int, C.POINTER(GemmArgs), C.POINTER(C.c_int)]),
+    "mg_launch_count": (C.c_int, [C.POINTER(GemmArgs), C.c_int, C.c_int64, C.c_int64, C.c_int, C.POINTER(C.c_int)]),
     "mg_side_fork": (C.c_int, [_P]),
     "mg_side_join": (C.c_int, [_P]),
     "mg_gemm_time": (C.c_int, [_P, C.POINTER(GemmArgs), C.c_int, C.POINTER(C.c_double)]),
     "mg_gemm_time_rotating": (C.c_int, [_P, C.POINTER(GemmArgs), C.c_int, C.c_int, C.POINTER(C.c_double)]),
+    "mg_gemm_time_each": (C.c_int, [_P, C.POINTER(GemmArgs), C.c_int, C.POINTER(C.c_double)]),
     "mg_probe_mfma": (C.c_int, [_P, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "mg_tile_count": (C.c_int, []),
     "mg_tile_info": (C.c_int, [C.c_int, C.POINTER(Tile)]),

@@ -45,6 +45,12 @@ __global__ void zero_c_kernel(float *C, int64_t ldc, int M, int N, int64_t sc, i
     }
 }
 
+// Arrival counters back to zero (a fill kernel, so that the sequence may be captured into a graph).
+__global__ void zero_ints_kernel(int *p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
 struct TileDesc {
     int id, bm, bn, bk, wgm, wgn;
     int nstage;     // 0: register-staged kernel; >0: direct-to-LDS ring depth
@@ -165,6 +171,13 @@ static bool dma_eligible(const mg_gemm_args &a, const TileDesc &t, int64_t k_per
     // beyond the matrix, so the caller must own it (MG_FLAG_TIGHT_BUFFERS says it does not).
     const bool ragged = (a_kc ? (a.k & 7) : (a.m & 7)) || (b_kc ? (a.k & 7) : (a.n & 7));
     if (ragged && (a.flags & MG_FLAG_TIGHT_BUFFERS)) return false;
+    if (t.pingpong) {
+        // its loads address a lane as scalar base + 32-bit offset of up to 7 rows (K-contiguous
+        // operand, 8 rows of 128 bytes per instruction) or 1 row (M/N-contiguous, 2 rows of 512)
+        const int64_t lim = (int64_t)1 << 32;
+        if ((a_kc ? 7 * a.lda * 2 + 128 : a.lda * 2 + 512) >= lim) return false;
+        if ((b_kc ? 7 * a.ldb * 2 + 128 : a.ldb * 2 + 512) >= lim) return false;
+    }
     if (t.persistent) {
         if (a.k % t.bk != 0 || k_per_split % t.bk != 0) return false;
         if (a.res && a.res != a.c) return false;   // their beta = 1 is an atomic add into C
@@ -796,7 +809,23 @@ struct Lane {
     int64_t max_tiles;    // arrival counters available
     int cus;
     int lds_limit;        // LDS bytes a workgroup may use
+    // The counters a launch uses are cleared by a fill kernel in front of it: for a workspace
+    // that keeps what the last call left (mg_gemm_static).  A context's counters are zero
+    // between launches by construction and need none.
+    bool clear_counters = false;
+    // Dry run: nothing is launched, every kernel that would be is counted here.
+    int *dry_count = nullptr;
 };
+
+// MG_FLAG_SPLITK_ATOMIC keeps a call off the workspace altogether: no slices meeting there, no
+// partial round cut into slices, no stream-K pieces.
+static Lane lane_without_ws(Lane ln) {
+    ln.ws = nullptr;
+    ln.cnt = nullptr;
+    ln.ws_bytes = 0;
+    ln.max_tiles = 0;
+    return ln;
+}
 
 static int lane_of(mg_ctx *ctx, const mg_gemm_args &a, Lane &ln) {
     const bool on_side = (a.flags & MG_FLAG_SIDE_STREAM) != 0;
@@ -847,9 +876,10 @@ static int variant_for(const mg_gemm_args &a, const TileDesc &t) {
     return t.nstage > 0 ? 0 : (operands_aligned(a) ? 0 : 1);
 }
 
-static int enqueue_gemm(const Lane &ln, const mg_gemm_args *args, const Plan &pl) {
+static int enqueue_gemm(const Lane &lane, const mg_gemm_args *args, const Plan &pl) {
     const mg_gemm_args &a = *args;
     const TileDesc &t = g_tiles[pl.tile];
+    const Lane ln = (a.flags & MG_FLAG_SPLITK_ATOMIC) ? lane_without_ws(lane) : lane;
     {
         int slices = 1;
         const int64_t m1 = tail_rows(ln, a, pl, t, &slices);
@@ -909,6 +939,10 @@ static int enqueue_gemm(const Lane &ln, const mg_gemm_args *args, const Plan &pl
         g.sa = p.sa; g.sb = p.sb; g.sc = p.sc;
         g.M = p.M; g.N = p.N; g.K = p.K; g.beta = p.beta;
         const dim3 grid((unsigned)cdiv(a.n, GEMV_ROWS_PER_WG), 1, (unsigned)a.nbatch);
+        if (ln.dry_count) {
+            ++*ln.dry_count;
+            return MG_OK;
+        }
         hipError_t e = gemv_table[a.dtype][lm][lc](g, grid, stream, nullptr);
         if (e != hipSuccess) return hip_fail(e, "mg_gemm: kernel launch");
         return MG_OK;
@@ -974,9 +1008,13 @@ static int enqueue_gemm(const Lane &ln, const mg_gemm_args *args, const Plan &pl
         unsigned gx = (unsigned)cdiv(zn, 1024);
         unsigned gy = (unsigned)(zm < 4096 ? zm : 4096);
         if (gx > 65535u * 16u) return fail(MG_ERR_ARG, "mg_gemm: C too large for the split-K clear");
-        hipLaunchKernelGGL(zero_c_kernel, dim3(gx, gy, (unsigned)zb), dim3(256), 0, stream, a.c, a.ldc, zm, zn,
-                           p.sc, vec);
-        HIP_TRY(hipGetLastError());
+        if (ln.dry_count) {
+            ++*ln.dry_count;
+        } else {
+            hipLaunchKernelGGL(zero_c_kernel, dim3(gx, gy, (unsigned)zb), dim3(256), 0, stream, a.c, a.ldc, zm, zn,
+                               p.sc, vec);
+            HIP_TRY(hipGetLastError());
+        }
     }
     int general = variant_for(a, t);
     dim3 grid((unsigned)(pl.grid_m * pl.grid_n), (unsigned)pl.split_k, (unsigned)a.nbatch);
@@ -1009,6 +1047,21 @@ static int enqueue_gemm(const Lane &ln, const mg_gemm_args *args, const Plan &pl
     }
     launch_fn fn = table_for(a.layout, a.dtype)[pl.tile][general];
     if (!fn) return fail(MG_ERR_STATE, "mg_gemm: tile %d has no kernel for this alignment", pl.tile);
+    if (p.cnt && ln.clear_counters) {
+        // one counter per tile of this launch (all batches)
+        const int64_t counted = (int64_t)pl.grid_m * pl.grid_n * a.nbatch;
+        if (ln.dry_count) {
+            ++*ln.dry_count;
+        } else {
+            hipLaunchKernelGGL(zero_ints_kernel, dim3((unsigned)cdiv(counted, 256)), dim3(256), 0, stream, p.cnt,
+                               (int)counted);
+            HIP_TRY(hipGetLastError());
+        }
+    }
+    if (ln.dry_count) {
+        ++*ln.dry_count;
+        return MG_OK;
+    }
     hipError_t e = fn(p, grid, stream, nullptr);
     if (e != hipSuccess) return hip_fail(e, "mg_gemm: kernel launch");
     return MG_OK;
@@ -1097,6 +1150,54 @@ int mg_gemm_time_rotating(mg_ctx *ctx, const mg_gemm_args *args, int nargs, int 
     HIP_TRY(hipEventElapsedTime(&ms, ctx->ev0, ctx->ev1));
     *seconds = (double)ms * 1e-3;
     return MG_OK;
+}
+
+int mg_gemm_time_each(mg_ctx *ctx, const mg_gemm_args *args, int nargs, double *seconds_each) {
+    if (!ctx || !args || !seconds_each) return fail(MG_ERR_ARG, "mg_gemm_time_each: NULL argument");
+    if (nargs < 1 || nargs > 4096) return fail(MG_ERR_ARG, "mg_gemm_time_each: nargs must be 1..4096");
+    if (ctx->capturing) return fail(MG_ERR_STATE, "mg_gemm_time_each: not allowed while a graph is being recorded");
+    Plan *pl = new (std::nothrow) Plan[nargs];
+    hipEvent_t *ev = new (std::nothrow) hipEvent_t[nargs + 1]();
+    if (!pl || !ev) {
+        delete[] pl;
+        delete[] ev;
+        return fail(MG_ERR_NOMEM, "mg_gemm_time_each: out of host memory");
+    }
+    int rc = MG_OK, made = 0;
+    Lane ln;
+    for (int i = 0; i < nargs && rc == MG_OK; i++) {
+        rc = check_args(&args[i]);
+        if (rc == MG_OK && (args[i].flags & MG_FLAG_SIDE_STREAM))
+            rc = fail(MG_ERR_ARG, "mg_gemm_time_each: timing runs on the main stream");
+        if (rc == MG_OK) pick_plan(args[i], ctx->prop.multiProcessorCount, pl[i]);
+    }
+    if (rc == MG_OK) rc = lane_of(ctx, args[0], ln);
+    if (rc == MG_OK && hipSetDevice(ctx->device) != hipSuccess) rc = fail(MG_ERR_HIP, "mg_gemm_time_each: hipSetDevice");
+    for (; rc == MG_OK && made <= nargs; made++) {
+        hipError_t e = hipEventCreate(&ev[made]);
+        if (e != hipSuccess) {
+            rc = hip_fail(e, "mg_gemm_time_each: hipEventCreate");
+            break;
+        }
+    }
+    if (rc == MG_OK) {
+        hipError_t e = hipEventRecord(ev[0], ctx->stream);
+        for (int i = 0; i < nargs && e == hipSuccess && rc == MG_OK; i++) {
+            rc = enqueue_gemm(ln, &args[i], pl[i]);
+            if (rc == MG_OK) e = hipEventRecord(ev[i + 1], ctx->stream);
+        }
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        for (int i = 0; i < nargs && e == hipSuccess && rc == MG_OK; i++) {
+            float ms = 0.f;
+            e = hipEventElapsedTime(&ms, ev[i], ev[i + 1]);
+            seconds_each[i] = (double)ms * 1e-3;
+        }
+        if (e != hipSuccess && rc == MG_OK) rc = hip_fail(e, "mg_gemm_time_each");
+    }
+    for (int i = 0; i < made; i++) (void)hipEventDestroy(ev[i]);
+    delete[] ev;
+    delete[] pl;
+    return rc;
 }
 
 int mg_graph_begin(mg_ctx *ctx) {
@@ -1241,11 +1342,6 @@ int mg_graph_destroy(mg_ctx *ctx, mg_graph *g) {
 static __device__ __align__(256) unsigned char scratch[MG_STATIC_WS_BYTES + MG_STATIC_MAX_TILES * sizeof(int)];
 
 namespace mg {
-__global__ void zero_ints_kernel(int *p, int n) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = 0;
-}
-
 struct StaticLane {
     std::atomic<int> ready{0};   // 0: not looked up, 1: ready
     float *ws = nullptr;
@@ -1289,61 +1385,100 @@ static int static_lane(int device, StaticLane **out) {
 
 extern "C" {
 
-int mg_gemm_static(int device_index, void *hip_stream, const mg_gemm_args *args) {
+// Number of HIP devices, asked once: the count cannot change while the process runs, and the
+// question must not be put while a stream of the caller is being captured.
+static int static_device_count() {
+    static std::atomic<int> cached{-1};
+    int n = cached.load(std::memory_order_acquire);
+    if (n >= 0) return n;
+    if (hipGetDeviceCount(&n) != hipSuccess || n < 0) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    cached.store(n, std::memory_order_release);
+    return n;
+}
+
+static int static_gemm(int device_index, hipStream_t stream, const mg_gemm_args *args, int *dry_count) {
     int rc = check_args(args);
     if (rc != MG_OK) return rc;
     if (args->flags & MG_FLAG_SIDE_STREAM)
         return fail(MG_ERR_ARG, "mg_gemm_static: MG_FLAG_SIDE_STREAM belongs to a context; pass the stream itself");
-    int count = 0;
-    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
-        (void)hipGetLastError();
-        return fail(MG_ERR_NODEVICE, "mg_gemm_static: no HIP device available");
-    }
+    const int count = static_device_count();
+    if (count <= 0) return fail(MG_ERR_NODEVICE, "mg_gemm_static: no HIP device available");
     if (device_index < 0 || device_index >= count)
         return fail(MG_ERR_ARG, "mg_gemm_static: device index %d out of range [0, %d)", device_index, count);
-    HIP_TRY(hipSetDevice(device_index));
+    // the caller's current device is left as it was
+    int before = -1;
+    HIP_TRY(hipGetDevice(&before));
+    if (before != device_index) HIP_TRY(hipSetDevice(device_index));
+    struct Restore {
+        int dev, now;
+        ~Restore() {
+            if (dev >= 0 && dev != now) (void)hipSetDevice(dev);
+        }
+    } restore{before, device_index};
     StaticLane *sl = nullptr;
     rc = static_lane(device_index, &sl);
     if (rc != MG_OK) return rc;
     Lane ln;
-    ln.stream = (hipStream_t)hip_stream;
+    ln.stream = stream;
     ln.ws = sl->ws;
     ln.ws_bytes = MG_STATIC_WS_BYTES;
     ln.cnt = sl->cnt;
     ln.max_tiles = MG_STATIC_MAX_TILES;
     ln.cus = sl->cus;
     ln.lds_limit = sl->lds_limit;
+    ln.clear_counters = true;   // the array keeps what the last call left
+    ln.dry_count = dry_count;
     Plan pl;
     pick_plan(*args, ln.cus, pl);
     const TileDesc &t = g_tiles[pl.tile];
-    // what the K slices (or stream-K pieces) of this plan need of the static workspace
-    const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n * args->nbatch;
-    int64_t need = 0, counted = 0;
-    if (pl.split_k > 1) {
-        need = tiles * pl.split_k * t.bm * t.bn * (int64_t)sizeof(float);
-        counted = tiles;
-    } else if (t.persistent == 2) {
-        const int64_t slots = (int64_t)ln.cus * wgs_per_cu(t, args->layout);
-        const int64_t slots_z = slots / args->nbatch > 0 ? slots / args->nbatch : 1;
-        const StreamK sk = stream_k_partition((int64_t)pl.grid_m * pl.grid_n, args->k / t.bk, slots_z);
-        if (sk.pieces > 1) {
-            need = (int64_t)sk.pieces * sk.rem_tiles * args->nbatch * t.bm * t.bn * (int64_t)sizeof(float);
-            counted = tiles;
-        }
+    // A K split the caller or the picker chose must fit the static workspace (a stream-K tile whose
+    // pieces do not fit runs as a plain persistent one, a partial round is cut only if it fits).
+    if (pl.split_k > 1 && !(args->flags & MG_FLAG_SPLITK_ATOMIC)) {
+        const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n * args->nbatch;
+        const int64_t need = tiles * pl.split_k * t.bm * t.bn * (int64_t)sizeof(float);
+        if (need > MG_STATIC_WS_BYTES || tiles > MG_STATIC_MAX_TILES)
+            return fail(MG_ERR_ARG,
+                        "mg_gemm_static: this GEMM's K split needs %lld bytes of partial tiles and %lld tile counters; the "
+                        "static workspace holds %lld bytes and %d counters (use mg_gemm, a smaller split_k, or "
+                        "MG_FLAG_SPLITK_ATOMIC)",
+                        (long long)need, (long long)tiles, (long long)MG_STATIC_WS_BYTES, MG_STATIC_MAX_TILES);
     }
-    if (!(args->flags & MG_FLAG_SPLITK_ATOMIC) && (need > MG_STATIC_WS_BYTES || counted > MG_STATIC_MAX_TILES))
-        return fail(MG_ERR_ARG,
-                    "mg_gemm_static: this GEMM's K split needs %lld bytes of partial tiles and %lld tile counters; the "
-                    "static workspace holds %lld bytes and %d counters (use mg_gemm, a smaller split_k, or "
-                    "MG_FLAG_SPLITK_ATOMIC)",
-                    (long long)need, (long long)counted, (long long)MG_STATIC_WS_BYTES, MG_STATIC_MAX_TILES);
-    if (counted > 0 && !(args->flags & MG_FLAG_SPLITK_ATOMIC)) {
-        // The array keeps what the last call left: counters must start at zero (a fill kernel, so
-        // that the sequence may be captured into a graph).
-        hipLaunchKernelGGL(zero_ints_kernel, dim3((unsigned)cdiv(counted, 256)), dim3(256), 0, ln.stream, ln.cnt,
-                           (int)counted);
-        HIP_TRY(hipGetLastError());
-    }
+    return enqueue_gemm(ln, args, pl);
+}
+
+int mg_gemm_static(int device_index, void *hip_stream, const mg_gemm_args *args) {
+    return static_gemm(device_index, (hipStream_t)hip_stream, args, nullptr);
+}
+
+int mg_gemm_static_launches(int device_index, const mg_gemm_args *args, int *kernels) {
+    if (!kernels) return fail(MG_ERR_ARG, "mg_gemm_static_launches: kernels is NULL");
+    *kernels = 0;
+    return static_gemm(device_index, nullptr, args, kernels);
+}
+
+int mg_launch_count(const mg_gemm_args *args, int compute_units, int64_t workspace_bytes, int64_t counters,
+                    int clear_counters, int *kernels) {
+    if (!kernels) return fail(MG_ERR_ARG, "mg_launch_count: kernels is NULL");
+    *kernels = 0;
+    int rc = check_args(args);
+    if (rc != MG_OK) return rc;
+    if (workspace_bytes < 0 || counters < 0) return fail(MG_ERR_ARG, "mg_launch_count: negative workspace size");
+    Lane ln;
+    ln.stream = nullptr;
+    // any non-null address: a dry run never dereferences it
+    ln.ws = workspace_bytes > 0 ? reinterpret_cast<float *>(uintptr_t(256)) : nullptr;
+    ln.ws_bytes = workspace_bytes;
+    ln.cnt = workspace_bytes > 0 ? reinterpret_cast<int *>(uintptr_t(256)) : nullptr;
+    ln.max_tiles = counters;
+    ln.cus = compute_units > 0 ? compute_units : 256;
+    ln.lds_limit = 160 * 1024;
+    ln.clear_counters = clear_counters != 0;
+    ln.dry_count = kernels;
+    Plan pl;
+    pick_plan(*args, ln.cus, pl);
     return enqueue_gemm(ln, args, pl);
 }
 

@@ -319,6 +319,19 @@ class Matmul:
 # autotuner
 # --------------------------------------------------------------------------
 
+def time_sequence(dev, calls):
+    """Seconds each GEMM of a sequence costs inside it: every call behind the previous one on
+    the device's stream, HIP events between them.  calls: (mm, a, b, c, m, n, k, kwargs) with
+    kwargs from lda / ldb / ldc / bias / accumulate."""
+    arr = (L.GemmArgs * len(calls))()
+    for i, (mm, a, b, c, m, n, k, kw) in enumerate(calls):
+        arr[i] = mm._args(a, b, c, m, n, k, 1, (0, 0, 0), kw.get("bias"), kw.get("accumulate", False),
+                          kw.get("lda"), kw.get("ldb"), kw.get("ldc"))
+    out = (C.c_double * len(calls))()
+    _check(dev._lib.mg_gemm_time_each(dev._ctx, arr, len(calls), out), "time_sequence")
+    return list(out)
+
+
 def stats_dict(st, tile):
     return {"numUsedVgprs": st.vgprs, "ldsUsageSizeInBytes": st.static_lds_bytes + st.dynamic_lds_bytes,
             "scratchMemUsageInBytes": st.scratch_bytes, "workgroupThreads": st.threads,
