@@ -137,12 +137,12 @@ def test_tile_table(lib):
         assert t.lds_bytes <= 160 * 1024
         assert 0 <= t.fallback < n
         seen.add(t.name)
-        if t.name.startswith(b"mv_"):
-            # the skinny-M streaming tile uses no matrix cores and no LDS; what it
-            # cannot run goes to a register-staged tile
+        if t.name.startswith((b"mv_", b"ms_")):
+            # the skinny-M streaming tiles (mv_: no matrix cores, no LDS; ms_: matrix cores, A in
+            # LDS); what they cannot run goes to a register-staged tile
             fb = L.Tile()
             lib.mg_tile_info(t.fallback, C.byref(fb))
-            assert t.lds_bytes == 0 and fb.stages == 0 and fb.fallback == fb.id
+            assert (t.lds_bytes == 0) == t.name.startswith(b"mv_") and fb.stages == 0 and fb.fallback == fb.id
             continue
         assert t.bm % (32 * t.waves_m) == 0 and t.bn % (32 * t.waves_n) == 0
         # the fallback chain ends at a register-staged tile of the same BM x BN

@@ -261,6 +261,40 @@ def test_skinny_stream_tile_exact(dev, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_skinny_matrix_core_tile_exact(dev, dtype):
+    """The skinny-M tile on the matrix cores (NT, M <= 64, A whole in LDS, every wavefront
+    streaming 32 rows of B through its own LDS buffer): row counts around the 32-row blocks,
+    K of one 8-element piece up to what fits LDS with ragged ends (K not a multiple of the
+    64-element phase, nor of 16), N from one column to more than a round of workgroups,
+    padded pitches of A, B and C with NaN / sentinel padding, bias, beta = 1; bit exact on
+    integer data, within tolerance on random data; the plan must really be that tile, and
+    what it cannot run goes to its fallback."""
+    from vkgrad_amd.kernels import CONFIGS, Matmul
+    ms = next(t for t in CONFIGS if t["name"].startswith("ms_"))
+    mp = Matmul(dev, trans_b=True, dtype=dtype, tile=ms["id"])
+    cases = [(5, 50257, 768), (7, 50257, 768), (8, 2304, 768), (9, 96, 768), (31, 4097, 768), (32, 1000, 1024),
+             (33, 777, 520), (63, 50257, 768), (64, 2304, 768), (64, 300, 960), (1, 1, 8), (17, 129, 8), (20, 127, 24),
+             (32, 128, 2176), (12, 257, 2048), (40, 255, 72), (64, 33, 136), (6, 100003, 264), (48, 513, 648)]
+    for i, (m, n, k) in enumerate(cases):
+        assert mp.plan(m, n, k)[0] == ms["id"], (m, n, k)
+        r, got, ref = check_case(dev, m, n, k, False, True, dtype, seed=m + n + k, integer=True, tile=ms["id"],
+                                 bias=bool(i & 1), accumulate=bool(i & 2), ldc=(n + 5 if i % 3 == 0 else None),
+                                 lda=(k + 8 if i % 4 == 1 else None), ldb=(k + 16 if i % 5 == 2 else None))
+        assert r["exact"], f"{m}x{n}x{k}: max diff {np.abs(got - ref).max()}"
+    for m, n, k in [(7, 50257, 768), (63, 3000, 768), (24, 2000, 1536)]:
+        r, got, ref = check_case(dev, m, n, k, False, True, dtype, seed=3, tile=ms["id"], bias=True)
+        _assert_close(r, f"ms {m}x{n}x{k}")
+    # what it cannot run goes to its fallback and is still right: too many rows, A too large for
+    # LDS, K not in whole 8-element pieces, another layout
+    for m, n, k, ta, tb in [(65, 300, 768, False, True), (64, 300, 1024, False, True), (33, 200, 2048, False, True),
+                            (16, 300, 516, False, True), (16, 304, 768, False, False)]:
+        assert mp.plan(m, n, k)[0] != ms["id"] or (ta, tb) != (False, True), (m, n, k)
+        r, got, ref = check_case(dev, m, n, k, ta, tb, dtype, seed=1, integer=True, tile=ms["id"])
+        assert r["exact"], (m, n, k)
+    mp.destroy()
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("layout", ["NN", "NT"])
 def test_fused_activation_output(dev, layout, dtype):
     """Forward epilogue with the activated 16-bit output (the reference's separate

@@ -37,6 +37,8 @@ def pick_config(m, n, k, trans_a=False, trans_b=False, min_groups=256):
     callers that used the reference function directly."""
     best = None
     for t in CONFIGS:
+        if t["name"].startswith(("mv_", "ms_")):
+            continue   # the skinny-M streams serve one layout and few rows; the library's picker knows when
         gm, gn = -(-m // t["bm"]), -(-n // t["bn"])
         groups = gm * gn
         useful = (m * n) / (gm * t["bm"] * gn * t["bn"])

@@ -43,16 +43,18 @@ constexpr launch_fn bias_variant_p() {
     {launch_gemm_dmap<L_NN, D_F16, bm, bn, bk, wgm, wgn, ns, false, false>, \
      bias_variant_p<bm, bn, bk, wgm, wgn, ns, false>(), nullptr},
 #define G(id, bm, bn, bk, fb) {nullptr, nullptr, nullptr},   // launched through gemv_table
+#define W(id, bm, bn, bk, fb) {nullptr, nullptr, nullptr},   // launched through skinny_table
 #define Q(id, bm, bn, bk, wgm, wgn, ns, fb) \
     {launch_gemm_pp<L_NN, D_F16, bm, bn, bk, wgm, wgn>, nullptr, act_variant_q<bm, bn, bk, wgm, wgn>()},
 #define S(id, bm, bn, bk, wgm, wgn, ns, fb)                                \
     {launch_gemm_dmap<L_NN, D_F16, bm, bn, bk, wgm, wgn, ns, false, true>, \
      bias_variant_p<bm, bn, bk, wgm, wgn, ns, true>(), nullptr},
-launch_fn launch_table_nn_f16[MG_NUM_TILES][3] = {MG_TILE_LIST(V, D, P, S, G, Q)};
+launch_fn launch_table_nn_f16[MG_NUM_TILES][3] = {MG_TILE_LIST(V, D, P, S, G, Q, W)};
 #undef V
 #undef D
 #undef P
 #undef S
 #undef G
 #undef Q
+#undef W
 }  // namespace mg

@@ -14,6 +14,7 @@
 
 #include "gemm_kernel.h"
 #include "gemv_kernel.h"
+#include "skinny_kernel.h"
 #include "mi_gemm.h"
 #include "tiles.h"
 
@@ -56,7 +57,7 @@ struct TileDesc {
     int nstage;     // 0: register-staged kernel; >0: direct-to-LDS ring depth
     int fallback;   // tile of the same BM x BN with weaker preconditions (self: none)
     int persistent; // 1: grid of resident workgroups looping over tiles; 2: the same with stream-K balancing
-    int gemv;       // 1: the skinny-M streaming kernel (no matrix cores), NT layout only
+    int gemv;       // 1: the skinny-M streaming kernel (no matrix cores), 2: the one on the matrix cores; NT layout only
     int pingpong;   // 1: the two wavefronts of a SIMD alternate between LDS reads and MFMAs (gemm_pp_kernel.h)
 };
 #define V(id, bm, bn, bk, wgm, wgn) {id, bm, bn, bk, wgm, wgn, 0, id, 0, 0, 0},
@@ -65,13 +66,15 @@ struct TileDesc {
 #define S(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 2, 0, 0},
 #define G(id, bm, bn, bk, fb) {id, bm, bn, bk, 1, GEMV_WAVES, 0, fb, 0, 1, 0},
 #define Q(id, bm, bn, bk, wgm, wgn, ns, fb) {id, bm, bn, bk, wgm, wgn, ns, fb, 0, 0, 1},
-static const TileDesc g_tiles[MG_NUM_TILES] = {MG_TILE_LIST(V, D, P, S, G, Q)};
+#define W(id, bm, bn, bk, fb) {id, bm, bn, bk, 1, 4, 0, fb, 0, 2, 0},
+static const TileDesc g_tiles[MG_NUM_TILES] = {MG_TILE_LIST(V, D, P, S, G, Q, W)};
 #undef V
 #undef D
 #undef P
 #undef S
 #undef G
 #undef Q
+#undef W
 
 static thread_local char g_err[512] = "";
 
@@ -105,6 +108,7 @@ static launch_fn (*table_for(int layout, int dtype))[3] {
 }
 
 static int lds_bytes_for(const TileDesc &t, int layout) {
+    if (t.gemv == 2) return skinny_lds_bytes(1, skinny_waves(1), SKINNY_KP, 768);   // for K = 768; grows with K
     if (t.gemv) return 0;
     if (t.nstage > 0) return t.nstage * (t.bm + t.bn) * t.bk * 2;
     const bool a_kc = layout != MG_TN, b_kc = layout == MG_NT;
@@ -156,7 +160,23 @@ static bool gemv_eligible(const mg_gemm_args &a, int split) {
     return true;
 }
 
+// The skinny-M kernel on the matrix cores: one or two blocks of 32 rows of A, held in LDS over
+// all of K beside the wavefronts' phase buffers of B; 16-byte pieces of both operands.
+static int skinny_blocks(const mg_gemm_args &a) { return (int)((a.m + 31) / 32); }
+static bool skinny_eligible(const mg_gemm_args &a, int split) {
+    if (a.layout != MG_NT || split > 1 || a.nbatch != 1) return false;
+    if (a.m > 32 * SKINNY_MAX_TMB || a.k > 8192) return false;
+    const int tmb = skinny_blocks(a);
+    if (skinny_lds_bytes(tmb, skinny_waves(tmb), SKINNY_KP, (int)a.k) > SKINNY_LDS_LIMIT) return false;
+    if (((uintptr_t)a.a | (uintptr_t)a.b) & 15) return false;
+    if ((a.lda | a.ldb | a.k) & 7) return false;
+    if (a.res && a.res != a.c) return false;   // its beta = 1 reads C
+    if (a.tri || a.y16) return false;
+    return true;
+}
+
 static bool dma_eligible(const mg_gemm_args &a, const TileDesc &t, int64_t k_per_split, int split) {
+    if (t.gemv == 2) return skinny_eligible(a, split);
     if (t.gemv) return gemv_eligible(a, split);
     if (t.nstage == 0) return true;
     const bool a_kc = a.layout != MG_TN, b_kc = a.layout == MG_NT;
@@ -219,9 +239,11 @@ static const float g_cost[MG_NUM_TILES][3][2] = {
     {{5.52f, 0.907f}, {4.46f, 0.944f}, {3.88f, 1.003f}},   // 19 mmk_128x128x64_w2x2_s2
     {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}},                     // 20 mv_8x64x512 (priced by bytes, see plan_cost_us)
     {{5.69f, 1.230f}, {13.28f, 1.060f}, {4.76f, 1.200f}},   // 21 mmq_256x256x64_w2x4_s2 (tile 10's overhead, its own K-block time)
+    {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}},                     // 22 ms_64x128x64 (priced by bytes, see plan_cost_us)
 };
 
 static int wgs_per_cu(const TileDesc &t, int layout) {
+    if (t.gemv == 2) return 2;
     if (t.gemv) return 8;
     const int by_lds = 163840 / lds_bytes_for(t, layout);
     const int acc_regs = t.bm * t.bn / (t.wgm * t.wgn * 64);          // per lane
@@ -268,6 +290,14 @@ static int64_t persistent_grid(const TileDesc &t, int64_t tiles, int split, int6
 // workgroups, each paying its overhead plus its K-blocks; a CU that holds fewer
 // workgroups than it could runs each of them faster, down to a latency floor.
 static double plan_cost_us(const mg_gemm_args &a, const TileDesc &t, int split, int cus) {
+    if (t.gemv == 2) {
+        // a stream over B at about 4.5 TB/s once the columns fill the chip (128 or 256 per
+        // workgroup), the writes of C behind it, and a start-up of a few microseconds
+        const double bytes = 2.0 * ((double)a.m * a.k + (double)a.k * a.n) + 4.0 * a.m * a.n * (a.beta ? 2.0 : 1.0);
+        const double wgs = (double)cdiv(a.n, 32 * skinny_waves(skinny_blocks(a)));
+        const double fill = wgs < cus / 2 ? (cus / 2) / wgs : 1.0;   // few workgroups: each streams alone
+        return 4.5 + bytes / 4.5e6 * (fill > 4.0 ? 4.0 : fill);
+    }
     if (t.gemv) {
         // a stream over B at about 5 TB/s once enough wavefronts are in flight, plus the
         // multiply-adds, which grow with the rows of A
@@ -727,7 +757,7 @@ int mg_tile_info(int id, mg_tile *out) {
     out->lds_bytes = lds_bytes_for(t, MG_NT);
     out->min_m = 1;
     if (t.gemv)
-        snprintf(out->name, sizeof(out->name), "mv_%dx%dx%d", t.bm, t.bn, t.bk);
+        snprintf(out->name, sizeof(out->name), "%s_%dx%dx%d", t.gemv == 2 ? "ms" : "mv", t.bm, t.bn, t.bk);
     else if (t.persistent)
         snprintf(out->name, sizeof(out->name), "%s_%dx%dx%d_w%dx%d_s%d", t.persistent == 2 ? "mmk" : "mmp", t.bm, t.bn, t.bk,
                  t.wgm, t.wgn, t.nstage);
@@ -784,6 +814,14 @@ int mg_tile_kernel_stats(mg_ctx *ctx, int tile, int layout, int dtype, int varia
     KernelQuery q;
     memset(&q, 0, sizeof(q));
     const TileDesc &t = g_tiles[tile];
+    if (t.gemv == 2) {
+        if (layout != MG_NT || variant < 0 || variant >= SKINNY_MAX_TMB)
+            return fail(MG_ERR_ARG, "mg_tile_kernel_stats: the skinny-M matrix-core tile has no instantiation %d for this layout", variant);
+        SkinnyParams g{};
+        const int tmb = variant + 1, nw = skinny_waves(tmb);
+        HIP_TRY(skinny_table[dtype][variant](g, dim3(1), skinny_lds_bytes(tmb, nw, SKINNY_KP, 768), nullptr, &q));
+        return fill_stats(q, out);
+    }
     if (t.gemv) {
         if (layout != MG_NT || variant < 0 || variant >= 16 || !gemv_table[dtype][variant / 4][variant % 4])
             return fail(MG_ERR_ARG, "mg_tile_kernel_stats: the skinny-M tile has no instantiation %d for this layout", variant);
@@ -929,6 +967,22 @@ static int enqueue_gemm(const Lane &lane, const mg_gemm_args *args, const Plan &
     p.k_per_split = pl.k_per_split;
     p.xcd_remap = pl.xcd_remap;
     if ((int64_t)pl.grid_m * pl.grid_n > 0x7fffffffLL) return fail(MG_ERR_ARG, "mg_gemm: grid too large");
+    if (t.gemv == 2) {
+        if (!skinny_eligible(a, pl.split_k)) return fail(MG_ERR_STATE, "mg_gemm: the skinny-M matrix-core tile cannot run this call");
+        const int tmb = skinny_blocks(a), nw = skinny_waves(tmb);
+        SkinnyParams g;
+        g.A = p.A; g.B = p.B; g.C = p.C; g.bias = p.bias;
+        g.lda = p.lda; g.ldb = p.ldb; g.ldc = p.ldc;
+        g.M = p.M; g.N = p.N; g.K = p.K; g.beta = p.beta;
+        if (ln.dry_count) {
+            ++*ln.dry_count;
+            return MG_OK;
+        }
+        hipError_t e = skinny_table[a.dtype][tmb - 1](g, dim3((unsigned)cdiv(a.n, 32 * nw)), skinny_lds_bytes(tmb, nw, SKINNY_KP, p.K),
+                                                       stream, nullptr);
+        if (e != hipSuccess) return hip_fail(e, "mg_gemm: kernel launch");
+        return MG_OK;
+    }
     if (t.gemv) {
         int lm = 0, lc = 0;
         if (!gemv_eligible(a, pl.split_k) || !gemv_shape(a, &lm, &lc) || !gemv_table[a.dtype][lm][lc])
@@ -1087,6 +1141,7 @@ int mg_kernel_stats_for(mg_ctx *ctx, const mg_gemm_args *args, int *tile, mg_ker
     pick_plan(*args, ctx->prop.multiProcessorCount, pl);
     const TileDesc &t = g_tiles[pl.tile];
     if (tile) *tile = pl.tile;
+    if (t.gemv == 2) return mg_tile_kernel_stats(ctx, pl.tile, args->layout, args->dtype, skinny_blocks(*args) - 1, out);
     if (t.gemv) {
         int lm = 0, lc = 0;
         if (!gemv_shape(*args, &lm, &lc)) return fail(MG_ERR_STATE, "mg_kernel_stats_for: the skinny-M tile cannot run this call");

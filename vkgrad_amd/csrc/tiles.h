@@ -23,10 +23,13 @@
 //   ping-pong direct-to-LDS (gemm_pp_kernel.h): the preconditions of the direct-to-LDS tiles;
 //     the two wavefronts of a SIMD alternate between reading operands and multiplying.
 //     Q(id, BM, BN, BK, WGM, WGN, NSTAGE, fallback_id)
+//   skinny-M stream on the matrix cores (skinny_kernel.h): NT layout, at most BM rows of A, which
+//     sits in LDS whole; every wavefront streams 32 rows of B by itself, BK elements of K at a time.
+//     W(id, bm, bn, bk, fallback_id) - BN output columns per workgroup of four wavefronts
 // WGM x WGN wavefronts of 64 lanes per workgroup.
 #pragma once
 
-#define MG_TILE_LIST(V, D, P, S, G, Q) \
+#define MG_TILE_LIST(V, D, P, S, G, Q, W) \
     V(0, 256, 256, 32, 2, 4)       \
     V(1, 256, 128, 64, 2, 2)       \
     V(2, 128, 256, 64, 2, 2)       \
@@ -48,6 +51,7 @@
     S(18, 256, 256, 64, 2, 4, 2, 15) \
     S(19, 128, 128, 64, 2, 2, 2, 17) \
     G(20, 8, 64, 512, 4) \
-    Q(21, 256, 256, 64, 2, 4, 2, 10)
+    Q(21, 256, 256, 64, 2, 4, 2, 10) \
+    W(22, 64, 128, 64, 4)
 
-#define MG_NUM_TILES 22
+#define MG_NUM_TILES 23

@@ -491,6 +491,16 @@ def skinny_stream_fits(m, k, layout):
     return layout == L.MG_NT and m <= 8 and k <= 2048 and k % 8 == 0
 
 
+def skinny_mfma_fits(m, k, layout):
+    """The skinny-M tile on the matrix cores (name ms_*): NT layout, at most 64 rows of A,
+    which must fit LDS whole beside the phase buffers of B (K <= 2176 for up to 32 rows,
+    K <= 960 for up to 64), K in whole 8-element pieces."""
+    kpad = -(-k // 64) * 64
+    blocks = -(-m // 32)
+    lds = (4 if blocks == 1 else 8) * 32 * (64 * 2 + 16) + blocks * 32 * (kpad * 2 + 16)
+    return layout == L.MG_NT and m <= 64 and k % 8 == 0 and lds <= 160 * 1024
+
+
 def candidate_space(m, n, k, cus=256, nbatch=1, layout=None):
     """(tile, split_k) pairs worth timing for a shape: every tile whose padding
     waste is tolerable, with K splits that bring an under-filled grid up to
@@ -499,10 +509,12 @@ def candidate_space(m, n, k, cus=256, nbatch=1, layout=None):
         gm, gn = -(-m // t["bm"]), -(-n // t["bn"])
         return (m * n) / (gm * t["bm"] * gn * t["bn"])
 
-    tiled = [t for t in CONFIGS if not t["name"].startswith("mv_")]
+    tiled = [t for t in CONFIGS if not t["name"].startswith(("mv_", "ms_"))]
     # skinny problems waste most of every tile: keep the tiles that waste least
     floor = min(0.45, 0.45 * max(useful_of(t) for t in tiled))
     out = [(t["id"], 1) for t in CONFIGS if t["name"].startswith("mv_") and skinny_stream_fits(m, k, layout)]
+    if nbatch == 1:
+        out += [(t["id"], 1) for t in CONFIGS if t["name"].startswith("ms_") and skinny_mfma_fits(m, k, layout)]
     for t in tiled:
         gm, gn = -(-m // t["bm"]), -(-n // t["bn"])
         if useful_of(t) < floor and len(tiled) > 1:
