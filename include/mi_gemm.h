@@ -276,6 +276,12 @@ int mg_launch_count(const mg_gemm_args *args, int compute_units, int64_t workspa
  * prices its kernels against (bench/RESULTS.md:113-119, 656-659). */
 int mg_probe_mfma(mg_ctx *ctx, int dtype, int random_operands, int iters, int workgroups, double *tflops,
                   double *ghz);
+/* What a launch shaped like the skinny-M stream reads from, or writes to, HBM when it does nothing
+ * else: `repeat` back-to-back launches over `nsets` rotating buffers of `nbytes` each (enough
+ * sets overflow the 256 MB last-level cache), microseconds per launch for the read-only and for
+ * the fill-only kernel.  The floor under the memory-bound skinny GEMMs; the counterpart of the
+ * reference's read and copy bandwidth probes (bench/roofline.py:27-50). */
+int mg_probe_stream(mg_ctx *ctx, int64_t nbytes, int nsets, int repeat, double *read_us, double *fill_us);
 /* CONFIGS — kernels.py:326-331: the tile table the tuner walks. */
 int mg_tile_count(void);
 int mg_tile_info(int id, mg_tile *out);

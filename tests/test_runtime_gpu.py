@@ -356,3 +356,16 @@ def test_mfma_ceiling_probe(dev):
     per_clock = q_tf * 1e12 / (q_ghz * 1e9) / (q * 4)
     assert 0.85 * 1024 <= per_clock <= 1.02 * 1024, per_clock
     assert q_ghz >= r_ghz * 0.97
+
+
+def test_stream_floor_probe(dev):
+    """mg_probe_stream: a read-only and a fill-only launch over the bytes of the 50257 x 768 f16
+    weight matrix, shaped like the skinny-M stream.  Between a tenth of the HBM peak and the
+    peak; a buffer 16 bytes long still runs (one partly filled wavefront)."""
+    from vkgrad_amd.probe import stream_floor
+    nbytes = 50257 * 768 * 2
+    r, f = stream_floor(dev, nbytes, nsets=8, repeat=50)
+    for us in (r, f):
+        assert 0.8e12 <= nbytes / (us * 1e-6) <= 8.0e12, us
+    r, f = stream_floor(dev, 16, nsets=1, repeat=3)
+    assert r > 0 and f > 0

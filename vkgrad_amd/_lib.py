@@ -102,6 +102,7 @@ SIGNATURES = {
     "mg_gemm_time_rotating": (C.c_int, [_P, C.POINTER(GemmArgs), C.c_int, C.c_int, C.POINTER(C.c_double)]),
     "mg_gemm_time_each": (C.c_int, [_P, C.POINTER(GemmArgs), C.c_int, C.POINTER(C.c_double)]),
     "mg_probe_mfma": (C.c_int, [_P, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "mg_probe_stream": (C.c_int, [_P, C.c_int64, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "mg_tile_count": (C.c_int, []),
     "mg_tile_info": (C.c_int, [C.c_int, C.POINTER(Tile)]),
     "mg_tile_fits": (C.c_int, [C.c_int, C.POINTER(GemmArgs)]),

@@ -59,9 +59,78 @@ __global__ void __launch_bounds__(512) k_probe_mfma(int iters, uint32_t seed, in
     }
 }
 
+// mg_probe_stream: what a launch shaped like the skinny-M stream can read from, or write to, HBM
+// when it does nothing else - four wavefronts to a workgroup, every wavefront one contiguous
+// 24 KB span (16 rows of 768 16-bit elements) with all 24 loads (or stores) of a lane issued
+// before anything is used.  The floor under the 1 x N x 768 forward GEMM.
+__global__ void __launch_bounds__(256) k_probe_read(const uint4 *src, int64_t n16, unsigned *sink) {
+    const int lane = threadIdx.x & 63;
+    const int64_t span = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 1536;   // 16-byte pieces per wavefront
+    uint4 v[24];
+#pragma unroll
+    for (int i = 0; i < 24; i++) {
+        const int64_t at = span + i * 64 + lane;
+        v[i] = at < n16 ? src[at] : uint4{0u, 0u, 0u, 0u};
+    }
+    unsigned acc = 0;
+#pragma unroll
+    for (int i = 0; i < 24; i++) acc ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+    if (acc == 0x9e3779b9u) *sink = acc;   // never true for the fill pattern: keeps the loads alive
+}
+__global__ void __launch_bounds__(256) k_probe_fill(uint4 *dst, int64_t n16, unsigned value) {
+    const int lane = threadIdx.x & 63;
+    const int64_t span = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 1536;
+#pragma unroll
+    for (int i = 0; i < 24; i++) {
+        const int64_t at = span + i * 64 + lane;
+        if (at < n16) dst[at] = uint4{value, value + 1, value + 2, value + 3};
+    }
+}
+
 }  // namespace mg
 
 using namespace mg;
+
+extern "C" int mg_probe_stream(mg_ctx *ctx, int64_t nbytes, int nsets, int repeat, double *read_us, double *fill_us) {
+    EW_PRECHECK("mg_probe_stream", nbytes >= 16 && nbytes <= ((int64_t)1 << 32) && nsets >= 1 && nsets <= 64 &&
+                                       repeat >= 1 && repeat <= 100000 && read_us && fill_us);
+    hipStream_t stream = ctx_stream(ctx);
+    const int64_t n16 = nbytes / 16;
+    const unsigned wgs = (unsigned)((n16 + 4 * 1536 - 1) / (4 * 1536));
+    uint4 *buf[64] = {nullptr};
+    unsigned *sink = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t e = hipMalloc((void **)&sink, 64);
+    for (int i = 0; i < nsets && e == hipSuccess; i++) e = hipMalloc((void **)&buf[i], (size_t)n16 * 16);
+    if (e == hipSuccess) e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    float ms_read = 0.f, ms_fill = 0.f;
+    if (e == hipSuccess) {
+        // enough rotating buffers make every launch find its bytes in HBM, not in the last-level cache
+        for (int i = 0; i < nsets; i++) hipLaunchKernelGGL(k_probe_fill, dim3(wgs), dim3(256), 0, stream, buf[i], n16, 7u * i);
+        e = hipEventRecord(e0, stream);
+        for (int r = 0; r < repeat; r++)
+            hipLaunchKernelGGL(k_probe_read, dim3(wgs), dim3(256), 0, stream, buf[r % nsets], n16, sink);
+        if (e == hipSuccess) e = hipEventRecord(e1, stream);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms_read, e0, e1);
+        if (e == hipSuccess) e = hipEventRecord(e0, stream);
+        for (int r = 0; r < repeat; r++)
+            hipLaunchKernelGGL(k_probe_fill, dim3(wgs), dim3(256), 0, stream, buf[r % nsets], n16, (unsigned)r);
+        if (e == hipSuccess) e = hipEventRecord(e1, stream);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms_fill, e0, e1);
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    for (int i = 0; i < nsets; i++)
+        if (buf[i]) (void)hipFree(buf[i]);
+    if (sink) (void)hipFree(sink);
+    if (e != hipSuccess) return ctx_hip_fail(e, "mg_probe_stream");
+    *read_us = (double)ms_read * 1e3 / repeat;
+    *fill_us = (double)ms_fill * 1e3 / repeat;
+    return MG_OK;
+}
 
 extern "C" int mg_probe_mfma(mg_ctx *ctx, int dtype, int random_operands, int iters, int workgroups, double *tflops,
                              double *ghz) {

@@ -1,6 +1,6 @@
 """MFMA ceiling of the device on zero and on random operands.
 
-    python -m vkgrad_amd.probe [--dtype bf16] [--seconds 0.5] [--busy-cus 256 192 128 64]
+    python -m vkgrad_amd.probe [--dtype bf16] [--seconds 0.5] [--busy-cus 256 192 128 64] [--stream-bytes B]
 
 Prints the rate a register-only MFMA loop sustains on every SIMD of the chip and the shader
 clock it ran at, for all-zero operands (the chip holds its boost clock) and for random ones
@@ -32,12 +32,23 @@ def mfma_ceiling(dev, dtype="bf16", random_operands=True, seconds=0.5, busy_cus=
     return tf.value, ghz.value
 
 
+def stream_floor(dev, nbytes, nsets=8, repeat=400):
+    """(read us, fill us) per launch of a kernel that only reads / only writes `nbytes`, shaped
+    like the skinny-M stream (24 KB per wavefront, everything in flight), over rotating buffers."""
+    r, f = C.c_double(), C.c_double()
+    _check(dev._lib.mg_probe_stream(dev._ctx, int(nbytes), int(nsets), int(repeat), C.byref(r), C.byref(f)), "probe")
+    return r.value, f.value
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--dtype", default="bf16", choices=("f16", "bf16"))
     ap.add_argument("--seconds", type=float, default=0.5)
     ap.add_argument("--busy-cus", type=int, nargs="*", default=[], metavar="N",
                     help="also run the random-operand loop with only N CUs multiplying")
+    ap.add_argument("--stream-bytes", type=int, default=0, metavar="B",
+                    help="also time a read-only and a fill-only kernel over B bytes, shaped like the skinny-M "
+                         "stream (e.g. 77194752 = the 50257 x 768 f16 weights)")
     args = ap.parse_args(argv)
     dev = Device()
     out = {"device": dev.name, "compute_units": dev.compute_units, "dtype": args.dtype}
@@ -49,6 +60,12 @@ def main(argv=None):
         tf, ghz = mfma_ceiling(dev, args.dtype, True, args.seconds, busy_cus=n)
         out[f"random_{n}_cus"] = {"tflops": round(tf, 1), "ghz": round(ghz, 3)}
         print(f"random, {n:3d} CUs busy {tf:8.1f} TFLOP/s at {ghz:.3f} GHz", flush=True)
+    if args.stream_bytes:
+        r, f = stream_floor(dev, args.stream_bytes)
+        out["stream"] = {"bytes": args.stream_bytes, "read_us": round(r, 2), "read_gbps": round(args.stream_bytes / r / 1e3, 1),
+                         "fill_us": round(f, 2), "fill_gbps": round(args.stream_bytes / f / 1e3, 1)}
+        print(f"stream of {args.stream_bytes} bytes: read-only {r:.2f} us ({args.stream_bytes / r / 1e3:.0f} GB/s), "
+              f"fill-only {f:.2f} us ({args.stream_bytes / f / 1e3:.0f} GB/s)", flush=True)
     print(json.dumps(out))
     dev.destroy()
 
