@@ -294,6 +294,31 @@ def test_skinny_matrix_core_tile_exact(dev, dtype):
     mp.destroy()
 
 
+@pytest.mark.parametrize("tile", [3, 4, 11, 13, 21])
+def test_xcd_major_order_and_rotated_walk_cover_every_tile(dev, tile):
+    """The tiled kernels renumber workgroups XCD-major - XCD x takes the x-th eighth of the
+    tile order, the first (tiles % 8) XCDs one tile more - and with MG_FLAG_XCD_ROTATE each XCD
+    starts elsewhere in its share.  Either way every output tile must be computed exactly once:
+    tile counts with every remainder modulo 8, fewer tiles than XCDs, bands that do not divide
+    the rows, with and without a K split (which keeps the renumbering only for whole eights),
+    on integer data where a tile computed twice or not at all cannot hide (beta = 1 doubles the
+    first, NaN poison shows the second)."""
+    from vkgrad_amd.kernels import CONFIGS
+    t = CONFIGS[tile]
+    bm, bn = t["bm"], t["bn"]
+    grids = [(1, 1), (3, 1), (2, 4), (3, 3), (5, 2), (11, 1), (3, 4), (13, 1), (7, 2), (5, 3), (4, 4), (17, 1),
+             (3, 6), (19, 1), (5, 4), (7, 3), (11, 2), (23, 1), (6, 4), (9, 5), (8, 8)]
+    for i, (gm, gn) in enumerate(grids):
+        m, n = gm * bm - (i % 3) * 8, gn * bn - (i % 2) * 8
+        for rot in (False, True):
+            for split, acc in ((0, False), (1, True), (2, False)):
+                k = 256 if split != 2 else 512
+                r, got, ref = check_case(dev, m, n, k, i % 3 == 2, i % 3 == 1, "bf16", seed=i, integer=True,
+                                         tile=tile, split_k=split, group_m=(0, 1, 3, 4)[i % 4], accumulate=acc,
+                                         xcd_rotate=rot)
+                assert r["exact"], (tile, gm, gn, rot, split, float(np.abs(got - ref).max()))
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("layout", ["NN", "NT"])
 def test_fused_activation_output(dev, layout, dtype):

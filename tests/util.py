@@ -23,7 +23,7 @@ def pad_pitch(x, ld, fill):
 
 def run_gemm(dev, a, b, m, n, k, trans_a=False, trans_b=False, dtype="f16", bias=None,
              c_in=None, tile=None, split_k=0, group_m=0, kind="device", poison=True,
-             lda=None, ldb=None, ldc=None):
+             lda=None, ldb=None, ldc=None, xcd_rotate=False):
     """a, b: stored operands (f16 arrays or bf16 bit patterns).  Returns C (m,n) f32.
     lda/ldb: upload the operand with that row pitch; the padding holds NaN so that
     anything read from it and used shows.  ldc: C has that row pitch; its padding
@@ -41,7 +41,7 @@ def run_gemm(dev, a, b, m, n, k, trans_a=False, trans_b=False, dtype="f16", bias
     bbias = None
     SENT = np.float32(-12345.5)
     mm = Matmul(dev, trans_a=trans_a, trans_b=trans_b, tile=tile, dtype=dtype, split_k=split_k,
-                group_m=group_m)
+                group_m=group_m, xcd_rotate=xcd_rotate)
     try:
         ba.upload(a)
         bb.upload(b)
@@ -65,7 +65,8 @@ def run_gemm(dev, a, b, m, n, k, trans_a=False, trans_b=False, dtype="f16", bias
 
 
 def check_case(dev, m, n, k, trans_a=False, trans_b=False, dtype="f16", seed=0, bias=False,
-               accumulate=False, tile=None, split_k=0, integer=False, group_m=0, lda=None, ldb=None, ldc=None):
+               accumulate=False, tile=None, split_k=0, integer=False, group_m=0, lda=None, ldb=None, ldc=None,
+               xcd_rotate=False):
     """Run one seeded case and compare with the oracle.  Returns metrics dict."""
     a, b = O.make_operands(m, n, k, trans_a, trans_b, dtype, seed, integer=integer)
     rng = np.random.default_rng(seed + 1000)
@@ -77,7 +78,7 @@ def check_case(dev, m, n, k, trans_a=False, trans_b=False, dtype="f16", seed=0, 
         bias_v = (rng.standard_normal(n) * 3 + np.arange(n) % 7 + 1).astype(np.float32) if bias else None
         c_in = rng.standard_normal((m, n)).astype(np.float32) * 5 if accumulate else None
     got = run_gemm(dev, a, b, m, n, k, trans_a, trans_b, dtype, bias_v, c_in, tile, split_k, group_m,
-                   lda=lda, ldb=ldb, ldc=ldc)
+                   lda=lda, ldb=ldb, ldc=ldc, xcd_rotate=xcd_rotate)
     ref = O.ref_gemm(a, b, trans_a, trans_b, dtype, bias_v, c_in)
     out = dict(maxrel=O.err_maxrel(got, ref), fro=O.err_fro(got, ref),
                exact=bool(np.array_equal(got, ref)), finite=bool(np.isfinite(got).all()),

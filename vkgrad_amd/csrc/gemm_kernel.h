@@ -49,7 +49,7 @@ struct GemmParams {
     int group_m;          // rasterisation band height in tiles (>= 1)
     int split_k;          // number of K slices (gridDim.y)
     int k_per_split;      // K elements per slice, a multiple of BK
-    int xcd_remap;        // 1: renumber workgroups so neighbours share an XCD
+    int xcd_remap;        // 1: renumber workgroups so neighbours share an XCD; 2: and rotate each XCD's walk
     float *ws;            // split-K workspace (split_k * tiles * BM * BN floats) or null: add with atomics
     int *cnt;             // one arrival counter per tile, zero between launches
     // Staggered start (ping-pong kernel): the first stagger_blocks workgroups - the ones resident
@@ -104,16 +104,31 @@ __device__ __forceinline__ u32x2 lds_read_tr(const uint16_t *p) {
 
 // Workgroup -> output tile.  Consecutive hardware workgroup ids land on
 // different XCDs (8 per chip, one L2 each); renumbering them XCD-major keeps
-// tiles that share operand panels behind one L2.  Inside that order, bands of
-// `group_m` row-blocks are walked column by column (the reference's grouped
-// rasterisation, kernels.py:72-94).
+// tiles that share operand panels behind one L2: XCD x takes the x-th eighth of
+// the tile order (the first total % 8 XCDs one tile more).  Inside that order,
+// bands of `group_m` row-blocks are walked column by column (the reference's
+// grouped rasterisation, kernels.py:72-94).
+//
+// xcd_remap == 2 also rotates every XCD's walk: XCD x starts x eighths into its
+// own run of tiles and wraps around.  Without it the eight XCDs walk their bands
+// in step and ask for the same panel of the shared operand at the same moment;
+// when that panel is not in the last-level cache each of them fetches it from
+// HBM (8192 x 50257 x 768 after kernels that left nothing of its operands in
+// cache: 717 us in step, 628 us rotated; with the operands in cache 590 / 620).
 __device__ __forceinline__ void tile_coords(const GemmParams &p, int &pid_m, int &pid_n) {
     int pid = blockIdx.x;
     const int total = p.grid_m * p.grid_n;
     if (p.xcd_remap) {
         constexpr int NXCD = 8;
-        const int per = total / NXCD;   // host guarantees total % 8 == 0 when xcd_remap
-        pid = (pid % NXCD) * per + pid / NXCD;
+        const int q = total / NXCD, r = total % NXCD;
+        const int xcd = pid % NXCD;
+        int local = pid / NXCD;
+        const int count = q + (xcd < r ? 1 : 0);
+        if (p.xcd_remap == 2) {
+            local += (int)(((int64_t)count * xcd) / NXCD);
+            if (local >= count) local -= count;
+        }
+        pid = xcd * q + min(xcd, r) + local;
     }
     const int in_group = p.group_m * p.grid_n;
     const int gid = pid / in_group;

@@ -375,7 +375,11 @@ static void finish_plan(const mg_gemm_args &a, int tile, int split, Plan &pl) {
     if (gm <= 0) gm = 8;
     if (gm > pl.grid_m) gm = pl.grid_m;
     pl.group_m = gm;
-    pl.xcd_remap = ((int64_t)pl.grid_m * pl.grid_n) % 8 == 0 ? 1 : 0;
+    // XCD-major renumbering needs workgroup id % 8 to be the XCD in every K slice and batch:
+    // a tile count in whole eights, or a grid that is nothing but tiles
+    const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n;
+    pl.xcd_remap = (tiles % 8 == 0 || (split == 1 && a.nbatch <= 1 && tiles >= 16)) ? 1 : 0;
+    if (pl.xcd_remap && (a.flags & MG_FLAG_XCD_ROTATE)) pl.xcd_remap = 2;
 }
 
 // Heuristic choice of tile, K split and rasterisation band (the reference's
@@ -507,7 +511,7 @@ static int check_args(const mg_gemm_args *a) {
     if (a->tile < -1 || a->tile >= MG_NUM_TILES) return fail(MG_ERR_ARG, "mg_gemm: unknown tile id %d", a->tile);
     if (a->split_k < 0 || a->split_k > 65535) return fail(MG_ERR_ARG, "mg_gemm: split_k %d out of range", a->split_k);
     if (a->group_m < 0) return fail(MG_ERR_ARG, "mg_gemm: group_m %d is negative", a->group_m);
-    if (a->flags & ~(MG_FLAG_TIGHT_BUFFERS | MG_FLAG_SPLITK_ATOMIC | MG_FLAG_SIDE_STREAM))
+    if (a->flags & ~(MG_FLAG_TIGHT_BUFFERS | MG_FLAG_SPLITK_ATOMIC | MG_FLAG_SIDE_STREAM | MG_FLAG_XCD_ROTATE))
         return fail(MG_ERR_ARG, "mg_gemm: unknown flags 0x%x", a->flags);
     return MG_OK;
 }

@@ -63,7 +63,7 @@ class Matmul:
 
     def __init__(self, dev, sg=None, wm=None, wn=None, trans_a=False, trans_b=False,
                  capture_stats=False, lds=True, bk=64, batched=False, acc16=False,
-                 group_m=0, *, tile=None, dtype="f16", split_k=0, atomic_split=False):
+                 group_m=0, *, tile=None, dtype="f16", split_k=0, atomic_split=False, xcd_rotate=False):
         if acc16:
             raise VkError("acc16 (f16 output) is not provided: no call site of the path uses it")
         if dtype not in L.DTYPES:
@@ -78,6 +78,7 @@ class Matmul:
         self.dtype = dtype
         self.split_k = int(split_k)
         self.atomic_split = bool(atomic_split)   # K slices add into C with atomics, not via the workspace
+        self.xcd_rotate = bool(xcd_rotate)       # every XCD starts elsewhere in its share of the tiles
         if tile is None and sg is not None:
             tile = _nearest_tile(sg * (wm or 1) * 16, (wn or 1) * 16)
         if tile is not None and not 0 <= tile < len(CONFIGS):
@@ -92,7 +93,8 @@ class Matmul:
             base = "mm_auto"
         self.name = (f"{base}_{dtype}{'_ta' if trans_a else ''}{'_tb' if trans_b else ''}"
                      f"{'_bat' if batched else ''}{'_g' + str(group_m) if group_m else ''}"
-                     f"{'_s' + str(split_k) if split_k > 1 else ''}{'_at' if atomic_split else ''}")
+                     f"{'_s' + str(split_k) if split_k > 1 else ''}{'_at' if atomic_split else ''}"
+                     f"{'_rot' if xcd_rotate else ''}")
         self._keep = []
 
     def fits(self, m, n, k):
@@ -138,6 +140,8 @@ class Matmul:
             ga.flags |= L.MG_FLAG_SPLITK_ATOMIC
         if side:
             ga.flags |= L.MG_FLAG_SIDE_STREAM
+        if self.xcd_rotate:
+            ga.flags |= L.MG_FLAG_XCD_ROTATE
         if act not in L.ACTS:
             raise VkError(f"{self.name}: unknown activation {act!r}; use None, 'gelu', 'relu', "
                           f"'gelu_grad', 'relu_grad' or 'softmax_grad'")
@@ -430,7 +434,7 @@ def tuned_matmul(dev, m, n, k, trans_a=False, trans_b=False, dtype="f16", batche
         return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, dtype=dtype), "picker"
     return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, dtype=dtype, tile=e["tile_id"],
                   split_k=e.get("split_k", 0), group_m=e.get("group_m", 0),
-                  atomic_split=e.get("atomic_split", False)), "tuned table"
+                  atomic_split=e.get("atomic_split", False), xcd_rotate=e.get("xcd_rotate", False)), "tuned table"
 
 
 _WARMED = set()
@@ -476,13 +480,19 @@ def _repeat_for(t_one):
 LAST_LEVEL_CACHE_BYTES = 256 << 20
 
 
-def buffer_sets_for(footprint):
-    """How many operand sets a timing loop rotates through: one when a single set
-    already overflows the last-level cache twice over, otherwise enough that a
-    rotation spans three cache sizes (3 to 8 sets)."""
-    if footprint >= 2 * LAST_LEVEL_CACHE_BYTES:
+MAX_OPERAND_SETS = 32
+
+
+def buffer_sets_for(read_bytes):
+    """How many operand sets a timing loop rotates through so that no launch finds what it
+    reads in the last-level cache: the sets between two uses of one set are read in between,
+    and together they are twice the cache (3 to MAX_OPERAND_SETS sets; one when a single set
+    already is).  Only what a GEMM reads counts: the results it writes pass through that
+    cache without displacing operands (8192 x 50257 x 768 finds its 90 MB of operands there
+    after the 1.65 GB of logits of the previous launch)."""
+    if read_bytes >= 2 * LAST_LEVEL_CACHE_BYTES:
         return 1
-    return max(3, min(8, -(-3 * LAST_LEVEL_CACHE_BYTES // max(1, footprint))))
+    return max(3, min(MAX_OPERAND_SETS, -(-2 * LAST_LEVEL_CACHE_BYTES // max(1, read_bytes)) + 1))
 
 
 def skinny_stream_fits(m, k, layout):
@@ -547,7 +557,7 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
     only, re-measuring group_m's default alongside (kernels.py:539-584).
     `timer(mm, repeat) -> seconds` replaces the device for tests of the logic.
     Returns (Matmul, best) with best keys config, lds, tflops, ms, tile,
-    evaluated, pruned, group_m, split_k, tile_id.
+    evaluated, pruned, group_m, xcd_rotate, split_k, tile_id.
     """
     key = tune_key(dev.name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate, lda, ldb, ldc)
     if use_cache:
@@ -555,7 +565,7 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
         if e is not None:
             return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=e["tile_id"],
                           dtype=dtype, split_k=e.get("split_k", 0), group_m=e.get("group_m", 0),
-                          atomic_split=e.get("atomic_split", False)), e
+                          atomic_split=e.get("atomic_split", False), xcd_rotate=e.get("xcd_rotate", False)), e
 
     nb = nbatch if batched else 1
     pa = int(lda) if lda is not None else (m if trans_a else k)      # row pitches
@@ -567,12 +577,14 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
     sets = None
     if timer is None:
         warmup(dev)
-        footprint = nb * (2 * (ea + eb) + 4 * ec)
+        read_bytes = nb * (2 * (ea + eb) + (4 * ec if accumulate else 0))
         K = make_kernels(dev, dtype)
-        sets = []
-        for s in range(buffer_sets_for(footprint)):
-            st = (dev.buffer(nb * ea * 2, "device"), dev.buffer(nb * eb * 2, "device"),
-                  dev.buffer(nb * ec * 4, "device"))
+        sets, outs = [], []
+        for s in range(buffer_sets_for(read_bytes)):
+            # results that are only written share three buffers: they do not displace operands
+            if accumulate or s < 3:
+                outs.append(dev.buffer(nb * ec * 4, "device"))
+            st = (dev.buffer(nb * ea * 2, "device"), dev.buffer(nb * eb * 2, "device"), outs[s % len(outs)])
             sets.append(st)
             # random operands: zeros or garbage bit patterns misstate the timing (data
             # toggling sets MFMA power and with it the clock)
@@ -588,7 +600,7 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
     try:
         # a K split is timed both ways: slices meeting in the workspace, and adding atomically
         cands = [Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=t, dtype=dtype,
-                        split_k=s, group_m=0, atomic_split=at)
+                        split_k=s, group_m=0, atomic_split=at, xcd_rotate=True)
                  for t, s in candidate_space(m, n, k, getattr(dev, "compute_units", 256), nb,
                                              layout_of(trans_a, trans_b))
                  for at in ((False, True) if s > 1 else (False,))]
@@ -635,16 +647,19 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
         results.sort(key=lambda r: -r["tflops"])
         best = dict(results[0])
 
+        # stage two: rasterisation band and the walk of the XCDs (in step or rotated) on the winner
         variants = [Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=best["tile_id"],
-                           dtype=dtype, split_k=best["split_k"], group_m=g, atomic_split=best["atomic_split"])
-                    for g in (0, 1, 2, 4, 16)]
+                           dtype=dtype, split_k=best["split_k"], group_m=g, atomic_split=best["atomic_split"],
+                           xcd_rotate=rot)
+                    for g in (0, 1, 2, 4, 16) for rot in (True, False)]
         gt = measure(variants)
-        scored = sorted(((v.flops(m, n, k) * nb / gt[id(v)] / 1e12, v.group_m) for v in variants), reverse=True)
+        scored = sorted(((v.flops(m, n, k) * nb / gt[id(v)] / 1e12, v.group_m, v.xcd_rotate) for v in variants),
+                        reverse=True)
         if verbose:
-            for tf, g in scored:
-                print(f"    group_m={g:2d} on winning tile   {tf:8.2f} TFLOPS")
-        tf, g = scored[0]
-        best.update(tflops=tf, ms=2.0 * m * n * k * nb / tf / 1e9, group_m=g)
+            for tf, g, rot in scored:
+                print(f"    group_m={g:2d}{' rotated' if rot else '        '} on winning tile   {tf:8.2f} TFLOPS")
+        tf, g, rot = scored[0]
+        best.update(tflops=tf, ms=2.0 * m * n * k * nb / tf / 1e9, group_m=g, xcd_rotate=rot)
         best["pruned"] = len(CONFIGS) * 1 - len({c.tile for c in cands})
         best["spilling"] = [list(x) for x in pruned]
         best["evaluated"] = len(results)
@@ -654,11 +669,10 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
             _save_cache(cache)
         return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=best["tile_id"],
                       dtype=dtype, split_k=best["split_k"], group_m=best["group_m"],
-                      atomic_split=best["atomic_split"]), best
+                      atomic_split=best["atomic_split"], xcd_rotate=best["xcd_rotate"]), best
     finally:
-        for st in sets or ():
-            for x in st:
-                x.destroy()
+        for x in {id(b): b for st in sets or () for b in st}.values():
+            x.destroy()
 
 
 # --------------------------------------------------------------------------
