@@ -255,6 +255,10 @@ def main():
                     help="forward pass, then the backward pass with the dW GEMMs of the layers on the library's "
                          "second stream beside the dX chain; default: every GEMM behind the previous one on one "
                          "stream (forward, dX, dW per linear), which measured 1-2 %% faster for the whole step")
+    ap.add_argument("--pair-dw", action="store_true",
+                    help="default order, but dX and dW of a linear side by side: dW on the library's second "
+                         "stream, forked before the pair and joined behind it (measured 3-5 %% slower for the "
+                         "whole step: the fork and join of every pair cost more than the overlap gains)")
     ap.add_argument("--dense-head", action="store_true",
                     help="row pitch of logits/dlogits = 50257 exactly (rows then start at odd addresses) instead of "
                          "the next multiple of 64")
@@ -369,6 +373,12 @@ def main():
         (autograd.py:218-227), so the dW GEMMs of a layer go to the library's second stream once
         that layer's dX chain is done and overlap the next layer's dX chain; the streams join at
         the end of the step.  Entries: ("gemm", call, on_side_stream) | ("fork",) | ("join",)"""
+        if args.pair_dw:
+            out = []
+            for i in range(0, len(calls), 3):
+                fwd, dx, dw = calls[i:i + 3]
+                out += [("gemm", fwd, False), ("fork",), ("gemm", dx, False), ("gemm", dw, True), ("join",)]
+            return out
         if not args.overlap_dw:
             return [("gemm", c, False) for c in calls]
         per_linear = [calls[i:i + 3] for i in range(0, len(calls), 3)]     # (fwd, dX, dW) per linear, head last

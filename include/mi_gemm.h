@@ -149,14 +149,17 @@ typedef struct {
  * workspace, so GEMMs of the two streams never meet there. */
 #define MG_FLAG_SIDE_STREAM 4
 /* The tiled kernels hand every XCD (8 per chip, an L2 each) a contiguous eighth of the tile
- * order.  With this flag XCD x starts x eighths into its share and wraps around, so that the
+ * order.  Rotated walk: XCD x starts x eighths into its share and wraps around, so that the
  * XCDs do not ask for the same operand panel at the same moment.  That moment costs when the
  * operands are not in the last-level cache - a GEMM inside a training step, whose operands
- * were last touched a whole step ago - because every XCD then fetches the panel from HBM.
- * With operands resident in that cache the in-step walk is the faster one by a few percent.
- * Ignored by the persistent, stream-K and skinny tiles and by grids the renumbering does not
- * apply to.  No counterpart in the reference (one L2 on its target). */
+ * were last touched a whole step ago - because every XCD then fetches the panel from HBM
+ * (up to 15 % of a GEMM's time).  In-step walk: all XCDs start at the beginning of their
+ * share; with operands resident in that cache it is the faster one by a few percent.
+ * Neither flag: the library decides (today: rotated).  Both: MG_ERR_ARG.  Ignored by the
+ * persistent, stream-K and skinny tiles and by grids the renumbering does not apply to.
+ * No counterpart in the reference (one L2 on its target). */
 #define MG_FLAG_XCD_ROTATE 8
+#define MG_FLAG_XCD_IN_STEP 16
 
 typedef struct {
     int32_t id;

@@ -73,7 +73,7 @@ def test_validation_accepts_ragged_shapes(lib):
     (dict(lda=63), "lda"), (dict(ldb=95), "ldb"), (dict(ldc=95), "ldc"),
     (dict(nbatch=0), "nbatch"), (dict(nbatch=2, sc=0), "overwrite"), (dict(nbatch=2, sc=10), "overlap"),
     (dict(tile=999), "tile"), (dict(split_k=-1), "split_k"), (dict(group_m=-2), "group_m"),
-    (dict(m=2 ** 31), "32-bit"),
+    (dict(m=2 ** 31), "32-bit"), (dict(flags=32), "unknown flags"), (dict(flags=8 | 16), "exclude each other"),
 ])
 def test_validation_rejects(lib, kw, needle):
     assert lib.mg_gemm_check(C.byref(good_args(**kw))) == L.MG_ERR_ARG

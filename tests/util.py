@@ -23,7 +23,7 @@ def pad_pitch(x, ld, fill):
 
 def run_gemm(dev, a, b, m, n, k, trans_a=False, trans_b=False, dtype="f16", bias=None,
              c_in=None, tile=None, split_k=0, group_m=0, kind="device", poison=True,
-             lda=None, ldb=None, ldc=None, xcd_rotate=False):
+             lda=None, ldb=None, ldc=None, xcd_rotate=None):
     """a, b: stored operands (f16 arrays or bf16 bit patterns).  Returns C (m,n) f32.
     lda/ldb: upload the operand with that row pitch; the padding holds NaN so that
     anything read from it and used shows.  ldc: C has that row pitch; its padding
@@ -66,7 +66,7 @@ def run_gemm(dev, a, b, m, n, k, trans_a=False, trans_b=False, dtype="f16", bias
 
 def check_case(dev, m, n, k, trans_a=False, trans_b=False, dtype="f16", seed=0, bias=False,
                accumulate=False, tile=None, split_k=0, integer=False, group_m=0, lda=None, ldb=None, ldc=None,
-               xcd_rotate=False):
+               xcd_rotate=None):
     """Run one seeded case and compare with the oracle.  Returns metrics dict."""
     a, b = O.make_operands(m, n, k, trans_a, trans_b, dtype, seed, integer=integer)
     rng = np.random.default_rng(seed + 1000)

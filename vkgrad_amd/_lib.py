@@ -15,6 +15,7 @@ MG_FLAG_TIGHT_BUFFERS = 1
 MG_FLAG_SPLITK_ATOMIC = 2
 MG_FLAG_SIDE_STREAM = 4
 MG_FLAG_XCD_ROTATE = 8
+MG_FLAG_XCD_IN_STEP = 16
 MG_STATIC_WS_BYTES = 32 << 20
 MG_STATIC_MAX_TILES = 16384
 

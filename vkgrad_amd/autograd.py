@@ -82,7 +82,7 @@ class Ctx:
                     mm = Matmul(self.dev, trans_a=trans_a, trans_b=trans_b, batched=batched,
                                 tile=e["tile_id"], dtype=self.dtype, split_k=e.get("split_k", 0),
                                 group_m=e.get("group_m", 0), atomic_split=e.get("atomic_split", False),
-                                xcd_rotate=e.get("xcd_rotate", False))
+                                xcd_rotate=e.get("xcd_rotate"))
                 else:
                     mm = Matmul(self.dev, trans_a=trans_a, trans_b=trans_b, batched=batched,
                                 dtype=self.dtype)

@@ -379,7 +379,9 @@ static void finish_plan(const mg_gemm_args &a, int tile, int split, Plan &pl) {
     // a tile count in whole eights, or a grid that is nothing but tiles
     const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n;
     pl.xcd_remap = (tiles % 8 == 0 || (split == 1 && a.nbatch <= 1 && tiles >= 16)) ? 1 : 0;
-    if (pl.xcd_remap && (a.flags & MG_FLAG_XCD_ROTATE)) pl.xcd_remap = 2;
+    // rotated walk unless the caller asks for the in-step one: operands of a training step are
+    // rarely in the last-level cache, and there the rotated walk is worth up to 15 %
+    if (pl.xcd_remap && !(a.flags & MG_FLAG_XCD_IN_STEP)) pl.xcd_remap = 2;
 }
 
 // Heuristic choice of tile, K split and rasterisation band (the reference's
@@ -511,8 +513,10 @@ static int check_args(const mg_gemm_args *a) {
     if (a->tile < -1 || a->tile >= MG_NUM_TILES) return fail(MG_ERR_ARG, "mg_gemm: unknown tile id %d", a->tile);
     if (a->split_k < 0 || a->split_k > 65535) return fail(MG_ERR_ARG, "mg_gemm: split_k %d out of range", a->split_k);
     if (a->group_m < 0) return fail(MG_ERR_ARG, "mg_gemm: group_m %d is negative", a->group_m);
-    if (a->flags & ~(MG_FLAG_TIGHT_BUFFERS | MG_FLAG_SPLITK_ATOMIC | MG_FLAG_SIDE_STREAM | MG_FLAG_XCD_ROTATE))
+    if (a->flags & ~(MG_FLAG_TIGHT_BUFFERS | MG_FLAG_SPLITK_ATOMIC | MG_FLAG_SIDE_STREAM | MG_FLAG_XCD_ROTATE | MG_FLAG_XCD_IN_STEP))
         return fail(MG_ERR_ARG, "mg_gemm: unknown flags 0x%x", a->flags);
+    if ((a->flags & MG_FLAG_XCD_ROTATE) && (a->flags & MG_FLAG_XCD_IN_STEP))
+        return fail(MG_ERR_ARG, "mg_gemm: MG_FLAG_XCD_ROTATE and MG_FLAG_XCD_IN_STEP exclude each other");
     return MG_OK;
 }
 
@@ -893,7 +897,8 @@ static int lane_of(mg_ctx *ctx, const mg_gemm_args &a, Lane &ln) {
 static int64_t tail_rows(const Lane &ln, const mg_gemm_args &a, const Plan &pl, const TileDesc &t, int *slices) {
     if (!t.pingpong || pl.split_k != 1 || a.nbatch != 1 || a.tri != MG_TRI_NONE) return 0;
     if (!a.c || a.y16 || a.z || a.colsum || a.res || a.p16) return 0;
-    const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n, cus = ln.cus;
+    // (cus: workgroups resident at once)
+    const int64_t tiles = (int64_t)pl.grid_m * pl.grid_n, cus = (int64_t)ln.cus * wgs_per_cu(t, a.layout);
     if (cus < 8 || tiles <= cus || tiles % cus == 0) return 0;
     const int64_t rows1 = (tiles / cus) * cus / pl.grid_n;            // tile rows of the whole rounds
     const int64_t rest = (pl.grid_m - rows1) * pl.grid_n;             // tiles left over
@@ -1030,9 +1035,10 @@ static int enqueue_gemm(const Lane &lane, const mg_gemm_args *args, const Plan &
         // starts of the first round over one K loop (2048 MFMA clocks a K-block)
         const int64_t wgs = (int64_t)pl.grid_m * pl.grid_n * a.nbatch * pl.split_k;
         const int64_t nkb = cdiv(pl.split_k > 1 ? pl.k_per_split : a.k, t.bk);
-        if (wgs > ln.cus && nkb <= 16) {
+        const int64_t resident = (int64_t)ln.cus * wgs_per_cu(t, a.layout);
+        if (wgs > resident && nkb <= 16) {
             p.stagger_clk = (int)nkb * 2048;
-            p.stagger_blocks = ln.cus;
+            p.stagger_blocks = (int)resident;
         }
     }
     p.sk_full_rounds = p.sk_rem_tiles = 0;

@@ -63,7 +63,7 @@ class Matmul:
 
     def __init__(self, dev, sg=None, wm=None, wn=None, trans_a=False, trans_b=False,
                  capture_stats=False, lds=True, bk=64, batched=False, acc16=False,
-                 group_m=0, *, tile=None, dtype="f16", split_k=0, atomic_split=False, xcd_rotate=False):
+                 group_m=0, *, tile=None, dtype="f16", split_k=0, atomic_split=False, xcd_rotate=None):
         if acc16:
             raise VkError("acc16 (f16 output) is not provided: no call site of the path uses it")
         if dtype not in L.DTYPES:
@@ -78,7 +78,8 @@ class Matmul:
         self.dtype = dtype
         self.split_k = int(split_k)
         self.atomic_split = bool(atomic_split)   # K slices add into C with atomics, not via the workspace
-        self.xcd_rotate = bool(xcd_rotate)       # every XCD starts elsewhere in its share of the tiles
+        # walk of the XCDs over their shares of the tiles: True rotated, False in step, None the library's choice
+        self.xcd_rotate = None if xcd_rotate is None else bool(xcd_rotate)
         if tile is None and sg is not None:
             tile = _nearest_tile(sg * (wm or 1) * 16, (wn or 1) * 16)
         if tile is not None and not 0 <= tile < len(CONFIGS):
@@ -94,7 +95,7 @@ class Matmul:
         self.name = (f"{base}_{dtype}{'_ta' if trans_a else ''}{'_tb' if trans_b else ''}"
                      f"{'_bat' if batched else ''}{'_g' + str(group_m) if group_m else ''}"
                      f"{'_s' + str(split_k) if split_k > 1 else ''}{'_at' if atomic_split else ''}"
-                     f"{'_rot' if xcd_rotate else ''}")
+                     f"{'' if xcd_rotate is None else ('_rot' if xcd_rotate else '_ins')}")
         self._keep = []
 
     def fits(self, m, n, k):
@@ -140,8 +141,8 @@ class Matmul:
             ga.flags |= L.MG_FLAG_SPLITK_ATOMIC
         if side:
             ga.flags |= L.MG_FLAG_SIDE_STREAM
-        if self.xcd_rotate:
-            ga.flags |= L.MG_FLAG_XCD_ROTATE
+        if self.xcd_rotate is not None:
+            ga.flags |= L.MG_FLAG_XCD_ROTATE if self.xcd_rotate else L.MG_FLAG_XCD_IN_STEP
         if act not in L.ACTS:
             raise VkError(f"{self.name}: unknown activation {act!r}; use None, 'gelu', 'relu', "
                           f"'gelu_grad', 'relu_grad' or 'softmax_grad'")
@@ -434,7 +435,7 @@ def tuned_matmul(dev, m, n, k, trans_a=False, trans_b=False, dtype="f16", batche
         return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, dtype=dtype), "picker"
     return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, dtype=dtype, tile=e["tile_id"],
                   split_k=e.get("split_k", 0), group_m=e.get("group_m", 0),
-                  atomic_split=e.get("atomic_split", False), xcd_rotate=e.get("xcd_rotate", False)), "tuned table"
+                  atomic_split=e.get("atomic_split", False), xcd_rotate=e.get("xcd_rotate")), "tuned table"
 
 
 _WARMED = set()
@@ -493,6 +494,13 @@ def buffer_sets_for(read_bytes):
     if read_bytes >= 2 * LAST_LEVEL_CACHE_BYTES:
         return 1
     return max(3, min(MAX_OPERAND_SETS, -(-2 * LAST_LEVEL_CACHE_BYTES // max(1, read_bytes)) + 1))
+
+
+def walk_matters(tile_id):
+    """Whether a tile's kernel walks the tile order per XCD (MG_FLAG_XCD_ROTATE / _IN_STEP mean
+    something to it): the one-tile-per-workgroup kernels do, the persistent, stream-K and
+    skinny ones place their work themselves."""
+    return CONFIGS[tile_id]["name"].split("_")[0] in ("mm", "mmd", "mmq")
 
 
 def skinny_stream_fits(m, k, layout):
@@ -565,7 +573,7 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
         if e is not None:
             return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=e["tile_id"],
                           dtype=dtype, split_k=e.get("split_k", 0), group_m=e.get("group_m", 0),
-                          atomic_split=e.get("atomic_split", False), xcd_rotate=e.get("xcd_rotate", False)), e
+                          atomic_split=e.get("atomic_split", False), xcd_rotate=e.get("xcd_rotate")), e
 
     nb = nbatch if batched else 1
     pa = int(lda) if lda is not None else (m if trans_a else k)      # row pitches
@@ -651,7 +659,7 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
         variants = [Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=best["tile_id"],
                            dtype=dtype, split_k=best["split_k"], group_m=g, atomic_split=best["atomic_split"],
                            xcd_rotate=rot)
-                    for g in (0, 1, 2, 4, 16) for rot in (True, False)]
+                    for g in (0, 1, 2, 4, 16) for rot in ((True, False) if walk_matters(best["tile_id"]) else (False,))]
         gt = measure(variants)
         scored = sorted(((v.flops(m, n, k) * nb / gt[id(v)] / 1e12, v.group_m, v.xcd_rotate) for v in variants),
                         reverse=True)
