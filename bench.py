@@ -7,10 +7,13 @@ proj 768->768, MLP 768->3072->768, plus the tied LM head 768->50257; for every
 linear the forward, dX and dW products (147 GEMMs, 6.07 TFLOP), bf16 inputs,
 fp32 accumulate and fp32 outputs, synthetic operands already resident in HBM.
 Weights are stored out x in (the tied-head convention), so the kernel layouts
-are NT forward, NN dX, TN dW.  Every GEMM runs behind the previous one;
---overlap-dw runs the forward pass first and then the backward pass with the dW
-GEMMs on the library's second stream beside the dX chain (measured 1-2 % slower
-for the whole step).
+are NT forward, NN dX, TN dW.  The step is given to the device as forward, dX,
+dW of each linear in turn; the dW GEMMs go to the library's second stream, which
+is forked once at the start of the step and joined once at its end (a weight
+gradient is needed by nothing before the optimiser), so they fill the compute
+units the forward / dX chain leaves idle in its partial rounds.  `in_order` in
+the line is the same step with every GEMM behind the previous one on one stream;
+--schedule names the other orders that were measured.
 
 Prints ONE JSON line: whole-step TFLOP/s, the MFMA roofline of the dominant
 GEMM measured with HIP events on the library's stream, and the numpy oracle
@@ -47,6 +50,17 @@ def gemm_list():
     return out
 
 
+SCHEDULES = {
+    "dw-stream": "forward, dX, dW per linear; the dW GEMMs on a second stream, forked once at the start of the "
+                 "step and joined once at its end",
+    "in-order": "forward, dX, dW per linear, every GEMM behind the previous one on one stream",
+    "dw-stream-waits": "forward, dX, dW per linear; the dW GEMMs on a second stream that waits before each for what "
+                       "the main stream has been given so far, joined at the end of the step",
+    "pairs": "forward, then dX and dW of the linear side by side on two streams, forked and joined per pair",
+    "passes": "forward pass, then backward pass with a layer's dW GEMMs on a second stream beside the next "
+              "layer's dX chain, joined at the end of the step",
+}
+
 LAYOUT_FLAGS = {"NN": (False, False), "NT": (False, True), "TN": (True, False)}
 
 
@@ -65,13 +79,21 @@ def pitches_for(name, vpitch):
     return {"ldc": vpitch} if name.endswith(".fwd") else {"lda": vpitch}
 
 
-def plan_for(dev, name, layout, m, n, k, vpitch):
+def plan_for(dev, name, layout, m, n, k, vpitch, context=None):
     """(Matmul, pitches) exactly as the timed step builds them: the tuned table's plan for
-    the shape (tile, K split, band, split mode), the library's picker where it has none."""
+    the shape (tile, K split, band, split mode, walk) - the one chosen inside the step of the
+    named schedule when the table holds one (kernels.tune_in_context), else the one chosen
+    alone - and the library's picker where the table has none."""
     from vkgrad_amd.kernels import tuned_matmul
     ta, tb = LAYOUT_FLAGS[layout]
     kw = pitches_for(name, vpitch)
-    return tuned_matmul(dev, m, n, k, ta, tb, DTYPE, **kw)[0], kw
+    return tuned_matmul(dev, m, n, k, ta, tb, DTYPE, context=context, **kw)[0], kw
+
+
+def context_of(schedule):
+    """Name under which plans tuned inside a step of this schedule are kept (None: a GEMM has the
+    chip to itself, the plans tuned alone apply)."""
+    return None if schedule == "in-order" else "gpt2s-" + schedule
 
 # HBM-side bytes per launch (L2 fetches + L2 write-backs) of each GEMM of the step,
 # measured on MI355X with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over
@@ -240,6 +262,54 @@ def other_workloads(dev):
     return out
 
 
+def tune_step(dev, args, vpitch, context, step_calls, record):
+    """Plans for the step's GEMMs as they run under args.schedule, by coordinate descent on the
+    time of the whole replayed step; the picks go to the tuner's cache under `context`."""
+    import statistics
+    from vkgrad_amd import kernels as K
+    if context is None:
+        sys.exit("bench.py --tune-step: the in-order schedule uses the plans tuned alone (kernels.autotune_matmul)")
+    fields = ("tile_id", "split_k", "atomic_split", "group_m", "xcd_rotate")
+    slots, meta = {}, {}
+    for name, layout, m, n, k, _ in gemm_list():
+        ta, tb = LAYOUT_FLAGS[layout]
+        kw = pitches_for(name, vpitch)
+        cur = K.lookup_tuned(dev.name, m, n, k, ta, tb, DTYPE, context=context, **kw)
+        cands = []
+        for c in K.plan_candidates(m, n, k, K.layout_of(ta, tb), dev.compute_units):
+            mm = K.matmul_from_entry(dev, c, ta, tb, DTYPE)
+            tile, split, _ = mm.plan(m, n, k, **kw)          # what the library would really run
+            mm.destroy()
+            if (tile, split) == (c["tile_id"], c["split_k"]):
+                cands.append(c)
+        first = dict(cands[0]) if cur is None else dict(cands[0], **{f: cur.get(f, cands[0][f]) for f in fields},
+                                                       tile=cur["tile"], config=cur["config"])
+        slots[name] = [first] + [c for c in cands if any(c[f] != first[f] for f in fields)]
+        meta[name] = (m, n, k, ta, tb, kw)
+        print(f"{name}: {len(slots[name])} candidates, held tile {first['tile_id']} split {first['split_k']}", flush=True)
+
+    def measure(assign):
+        graph = record(step_calls(vpitch, context, assign), "tune_step", args.schedule)
+        for _ in range(2):
+            graph.enqueue()
+        dev.sync()
+        each = graph.time(6)
+        graph.destroy()
+        return statistics.median(each)
+
+    assign, best, log = K.tune_in_context(slots, measure, verbose=True)
+    for what, plan, t in log:
+        print(f"  {what}: {plan} -> {t * 1e3:.4f} ms", flush=True)
+    cache = K._load_cache()
+    for name, e in assign.items():
+        m, n, k, ta, tb, kw = meta[name]
+        cache[K.tune_key(dev.name, m, n, k, ta, tb, DTYPE, context=context, **kw)] = dict(
+            e, context=context, step_ms=round(best * 1e3, 4))
+    K._save_cache(cache)
+    print(json.dumps({"context": context, "ms_per_step": round(best * 1e3, 4),
+                      "plans": {nm: [e[f] for f in fields] for nm, e in assign.items()}}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -251,14 +321,21 @@ def main():
     ap.add_argument("--warm-seconds", type=float, default=2.0,
                     help="sustained GEMM load before anything is timed (kernels.py:353-381)")
     ap.add_argument("--eager", action="store_true", help="enqueue GEMMs one by one instead of replaying a graph")
-    ap.add_argument("--overlap-dw", action="store_true",
-                    help="forward pass, then the backward pass with the dW GEMMs of the layers on the library's "
-                         "second stream beside the dX chain; default: every GEMM behind the previous one on one "
-                         "stream (forward, dX, dW per linear), which measured 1-2 %% faster for the whole step")
-    ap.add_argument("--pair-dw", action="store_true",
-                    help="default order, but dX and dW of a linear side by side: dW on the library's second "
-                         "stream, forked before the pair and joined behind it (measured 3-5 %% slower for the "
-                         "whole step: the fork and join of every pair cost more than the overlap gains)")
+    ap.add_argument("--schedule", default="dw-stream",
+                    choices=("dw-stream", "in-order", "dw-stream-waits", "pairs", "passes"),
+                    help="how the step's GEMMs are given to the device.  dw-stream (default): forward, dX, dW "
+                         "of each linear in turn, every dW GEMM on the library's second stream, which is forked "
+                         "once at the start of the step and joined once at its end - a weight gradient is "
+                         "needed by nothing before the optimiser (autograd.py:218-227).  in-order: every GEMM "
+                         "behind the previous one on one stream.  dw-stream-waits: like dw-stream, but the second "
+                         "stream waits, before every dW GEMM, for what the main stream has been given up to "
+                         "there.  pairs: dX and dW of a linear side by side, forked and joined per pair.  passes: "
+                         "the forward pass, then the backward pass with a layer's dW GEMMs on the second stream "
+                         "beside the next layer's dX chain")
+    ap.add_argument("--tune-step", action="store_true",
+                    help="no benchmark line: choose the plan of every GEMM of the step by what the whole step "
+                         "takes under --schedule (kernels.tune_in_context) and write the picks to the tuner's "
+                         "cache (VKGRAD_AMD_TUNE_CACHE) under the schedule's context")
     ap.add_argument("--dense-head", action="store_true",
                     help="row pitch of logits/dlogits = 50257 exactly (rows then start at odd addresses) instead of "
                          "the next multiple of 64")
@@ -305,33 +382,44 @@ def main():
 
     mms = {}
 
-    def mm_for(name, layout, m, n, k, vp):
+    def mm_for(name, layout, m, n, k, vp, context, entry=None):
+        """The step's Matmul for one GEMM: the table's plan for the context, or the plan `entry`
+        names (the step tuner's candidates)."""
         kw = pitches_for(name, vp)
-        key = (layout, m, n, k, tuple(sorted(kw.items())))
+        tag = None if entry is None else (entry["tile_id"], entry["split_k"], entry["atomic_split"],
+                                          entry["group_m"], entry["xcd_rotate"])
+        key = (layout, m, n, k, tuple(sorted(kw.items())), context, tag)
         if key not in mms:
-            mms[key] = plan_for(dev, name, layout, m, n, k, vp)[0]
+            if entry is None:
+                mms[key] = plan_for(dev, name, layout, m, n, k, vp, context)[0]
+            else:
+                from vkgrad_amd.kernels import matmul_from_entry
+                mms[key] = matmul_from_entry(dev, entry, *LAYOUT_FLAGS[layout], DTYPE)
         return mms[key], kw
 
     role_bufs = {"fwd": ("x", "w", "y"), "dX": ("dy", "w", "dx"), "dW": ("dy", "x", "dw")}
 
-    def step_calls(vp):
-        """Every GEMM of one step in order: (mm, a, b, c, m, n, k, pitches)."""
+    def step_calls(vp, context, plans=None):
+        """Every GEMM of one step in order: (mm, a, b, c, m, n, k, pitches); plans: {GEMM name:
+        table entry} overrides the table."""
         shapes = {nm: (lay, m, n, k) for nm, lay, m, n, k, _ in gemm_list()}
+        plans = plans or {}
         calls = []
         for layer in range(LAYERS):
             b = sets[layer % NSET]
             for name, _, _ in LINEARS:
                 for role in ("fwd", "dX", "dW"):
                     lay, m, n, k = shapes[f"{name}.{role}"]
-                    mm, kw = mm_for(f"{name}.{role}", lay, m, n, k, vp)
+                    mm, kw = mm_for(f"{name}.{role}", lay, m, n, k, vp, context, plans.get(f"{name}.{role}"))
                     calls.append((mm,) + tuple(b[name][x] for x in role_bufs[role]) + (m, n, k, kw))
         for role in ("fwd", "dX", "dW"):
             lay, m, n, k = shapes[f"head.{role}"]
-            mm, kw = mm_for(f"head.{role}", lay, m, n, k, vp)
+            mm, kw = mm_for(f"head.{role}", lay, m, n, k, vp, context, plans.get(f"head.{role}"))
             calls.append((mm,) + tuple(head[x] for x in role_bufs[role]) + (m, n, k, kw))
         return calls
 
-    calls = step_calls(vpitch)
+    context = context_of(args.schedule)
+    calls = step_calls(vpitch, context)
     step_flops = sum(2.0 * c[4] * c[5] * c[6] for c in calls)
 
     if args.pmc_pass:
@@ -366,37 +454,43 @@ def main():
         dev.destroy()
         return
 
-    def schedule_of(calls):
-        """Order of one step.  Default: forward, dX, dW of each linear in turn, every GEMM
-        behind the previous one.  --overlap-dw: the forward pass (layer 0 .. 11, LM head), then
-        the backward pass from the head down; dW of a linear depends on nothing that follows it
-        (autograd.py:218-227), so the dW GEMMs of a layer go to the library's second stream once
-        that layer's dX chain is done and overlap the next layer's dX chain; the streams join at
-        the end of the step.  Entries: ("gemm", call, on_side_stream) | ("fork",) | ("join",)"""
-        if args.pair_dw:
+    def schedule_of(calls, schedule):
+        """One step as a list of ("gemm", call, on_side_stream) | ("fork",) | ("join",): fork lets
+        the library's second stream wait for what the main stream has been given so far, join
+        lets the main stream wait for the second.  calls holds (fwd, dX, dW) per linear, the LM
+        head last."""
+        triples = [calls[i:i + 3] for i in range(0, len(calls), 3)]
+        if schedule == "in-order":
+            return [("gemm", c, False) for c in calls]
+        if schedule in ("dw-stream", "dw-stream-waits"):
+            out = [("fork",)] if schedule == "dw-stream" else []
+            for fwd, dx, dw in triples:
+                out += [("gemm", fwd, False), ("gemm", dx, False)]
+                if schedule == "dw-stream-waits":
+                    out.append(("fork",))
+                out.append(("gemm", dw, True))
+            return out + [("join",)]
+        if schedule == "pairs":
             out = []
-            for i in range(0, len(calls), 3):
-                fwd, dx, dw = calls[i:i + 3]
+            for fwd, dx, dw in triples:
                 out += [("gemm", fwd, False), ("fork",), ("gemm", dx, False), ("gemm", dw, True), ("join",)]
             return out
-        if not args.overlap_dw:
-            return [("gemm", c, False) for c in calls]
-        per_linear = [calls[i:i + 3] for i in range(0, len(calls), 3)]     # (fwd, dX, dW) per linear, head last
-        schedule = [("gemm", fwd, False) for fwd, _, _ in per_linear]
-        # (the LM head's two backward products stay on the main stream: each fills the chip with
-        # resident workgroups and two such kernels only take CUs from each other)
-        schedule += [("gemm", per_linear[-1][1], False), ("gemm", per_linear[-1][2], False)]
-        groups = [per_linear[l * len(LINEARS):(l + 1) * len(LINEARS)][::-1] for l in reversed(range(LAYERS))]
-        for g in groups:
-            schedule += [("gemm", dx, False) for _, dx, _ in g]
-            schedule.append(("fork",))
-            schedule += [("gemm", dw, True) for _, _, dw in g]
-        schedule.append(("join",))
-        return schedule
+        # passes: forward of layer 0 .. 11 and the head, then backward from the head down; the dW
+        # GEMMs of a layer go to the second stream once that layer's dX chain has been given to
+        # the main stream.  (The head's two backward products stay on the main stream: each fills
+        # the chip with resident workgroups and two such kernels only take CUs from each other.)
+        out = [("gemm", fwd, False) for fwd, _, _ in triples]
+        out += [("gemm", triples[-1][1], False), ("gemm", triples[-1][2], False)]
+        for l in reversed(range(LAYERS)):
+            g = triples[l * len(LINEARS):(l + 1) * len(LINEARS)][::-1]
+            out += [("gemm", dx, False) for _, dx, _ in g]
+            out.append(("fork",))
+            out += [("gemm", dw, True) for _, _, dw in g]
+        return out + [("join",)]
 
-    def record(calls, name):
+    def record(calls, name, schedule):
         graph = dev.graph(name)
-        for item in schedule_of(calls):
+        for item in schedule_of(calls, schedule):
             if item[0] == "fork":
                 graph.fork()
             elif item[0] == "join":
@@ -406,8 +500,8 @@ def main():
                 mm(a, b, c, m, n, k, graph=graph, side=item[2], **kw)
         return graph.finish()
 
-    def run_eager(calls):
-        for item in schedule_of(calls):
+    def run_eager(calls, schedule):
+        for item in schedule_of(calls, schedule):
             if item[0] == "fork":
                 dev.side_fork()
             elif item[0] == "join":
@@ -416,19 +510,19 @@ def main():
                 mm, a, b, c, m, n, k, kw = item[1]
                 mm.enqueue(a, b, c, m, n, k, side=item[2], **kw)
 
-    def time_steps(calls, name, steps, nwarm):
+    def time_steps(calls, name, steps, nwarm, schedule):
         """nwarm untimed steps, then `steps` timed ones: host wall clock around all of them
         (synchronised on both sides) and, for a graph, device time of each replay."""
         if args.eager:
             for _ in range(nwarm):
-                run_eager(calls)
+                run_eager(calls, schedule)
             dev.sync()
             t0 = time.perf_counter()
             for _ in range(steps):
-                run_eager(calls)
+                run_eager(calls, schedule)
             dev.sync()
             return time.perf_counter() - t0, None
-        graph = record(calls, name)
+        graph = record(calls, name, schedule)
         for _ in range(nwarm):
             graph.enqueue()
         dev.sync()
@@ -442,7 +536,11 @@ def main():
     # Sustained load first: the chip's clock under matrix load settles over milliseconds, and the
     # first kernels after an idle period run at a different clock than a training loop sees.
     warm_s = warmup(dev, args.warm_seconds, force=True) if args.warm_seconds > 0 else 0.0
-    dt, each = time_steps(calls, "gpt2_small_gemms", args.steps, args.warmup)
+    if args.tune_step:
+        tune_step(dev, args, vpitch, context, step_calls, record)
+        dev.destroy()
+        return
+    dt, each = time_steps(calls, "gpt2_small_gemms", args.steps, args.warmup, args.schedule)
     ms_per_step = dt / args.steps * 1e3
     tflops = step_flops / (dt / args.steps) / 1e12
 
@@ -452,7 +550,7 @@ def main():
     # it does inside the step.
     per_shape = []
     for name, layout, m, n, k, count in gemm_list():
-        mm, kw = mm_for(name, layout, m, n, k, vpitch)
+        mm, kw = mm_for(name, layout, m, n, k, vpitch, context)
         is_head = name.startswith("head")
         lin, role = name.split(".")
         groups = [head] if is_head else [s[lin] for s in sets]
@@ -507,9 +605,7 @@ def main():
                                "QKV/proj/MLP + tied head 50257, fwd+dX+dW, 147 GEMMs, 6.07 TFLOP per step",
                    "rows": ROWS, "d_model": D, "layers": LAYERS, "vocab": VOCAB, "logits_row_pitch": vpitch,
                    "launch": "eager" if args.eager else "hip-graph replay",
-                   "order": "forward, dX, dW per linear, one stream" if not args.overlap_dw else
-                            "forward pass, then backward pass with the layers' dW GEMMs on a second stream "
-                            "beside the next layer's dX chain (joined at the end)"},
+                   "schedule": SCHEDULES[args.schedule]},
         "frac_of_mfma_peak": round(tflops / PEAK_TFLOPS, 4),
         "sustained_warmup_s": round(warm_s, 2),
         "sum_of_event_timed_gemms_ms": round(events_ms, 4),
@@ -519,6 +615,11 @@ def main():
                    "derived_peak_tflops": round(dev.compute_units * 4 * 1024 * dev.clock_khz * 1e3 / 1e12, 1)},
         "per_shape": per_shape,
     }
+    if args.schedule != "in-order":
+        # the same step with every GEMM behind the previous one on one stream
+        idt, _ = time_steps(step_calls(vpitch, None), "gpt2_small_gemms_in_order", args.steps, args.warmup, "in-order")
+        out["in_order"] = {"schedule": SCHEDULES["in-order"], "value": round(step_flops / (idt / args.steps) / 1e12, 2),
+                           "unit": "TFLOP/s", "ms_per_step": round(idt / args.steps * 1e3, 4)}
     if each is not None:
         ev = sorted(x * 1e3 for x in each)
         out["ms_per_step_events"] = {"median": round(ev[len(ev) // 2], 4), "min": round(ev[0], 4), "max": round(ev[-1], 4),
@@ -526,8 +627,8 @@ def main():
     if not args.no_extra:
         if not args.dense_head and not args.eager:
             # the same step with logits / dlogits rows exactly 50257 elements apart
-            dcalls = step_calls(VOCAB)
-            ddt, deach = time_steps(dcalls, "gpt2_small_gemms_dense_head", args.steps, args.warmup)
+            dcalls = step_calls(VOCAB, context)
+            ddt, deach = time_steps(dcalls, "gpt2_small_gemms_dense_head", args.steps, args.warmup, args.schedule)
             out["dense_head"] = {"logits_row_pitch": VOCAB, "value": round(step_flops / (ddt / args.steps) / 1e12, 2),
                                  "unit": "TFLOP/s", "ms_per_step": round(ddt / args.steps * 1e3, 4)}
         out["other_workloads"] = other_workloads(dev)

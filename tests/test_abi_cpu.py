@@ -288,6 +288,60 @@ def test_autotuner_logic_with_fake_timer(tmp_path, monkeypatch):
     assert K.tune_key("d", 1, 2, 3, False, True) != K.tune_key("d", 1, 2, 3, True, False)
 
 
+def test_plans_tuned_in_context(tmp_path, monkeypatch):
+    """kernels.tune_in_context against a deterministic cost: coordinate descent finds plans whose
+    merit only shows in the sum (a GEMM that is slower alone but leaves room for its neighbour),
+    differences below the noise threshold change nothing, the refinement sweep picks band and
+    walk, every kept change is confirmed by a second measurement; a plan tuned in a context is
+    found under that context only, and a context without its own plan falls back to the one
+    tuned alone."""
+    import vkgrad_amd.kernels as K
+    monkeypatch.setattr(K, "_TUNE_CACHE", str(tmp_path / "tune.json"))
+    monkeypatch.setattr(K, "_SHIPPED_CACHE", str(tmp_path / "none.json"))
+    cands = K.plan_candidates(3072, 768, 8192, K.L.MG_TN)
+    assert len(cands) > 20 and cands[0]["split_k"] == 1
+    names = {K.CONFIGS[c["tile_id"]]["name"] for c in cands}
+    assert "mmq_256x256x64_w2x4_s2" in names and "mmd_128x128x64_w2x2_s2" in names and "mm_64x64x64_w2x2" in names
+    assert all(c["split_k"] == 1 or 8192 // (4 * c["config"][2]) >= c["split_k"] for c in cands)
+    assert {c["atomic_split"] for c in cands if c["split_k"] > 1} == {False, True}
+    assert not any(c["atomic_split"] for c in cands if c["split_k"] == 1)
+    big = K.plan_candidates(8192, 50257, 768, K.L.MG_NT)
+    assert all(c["split_k"] == 1 for c in big)          # 12 K-blocks: nothing to split
+    pp = next(t["id"] for t in K.CONFIGS if t["name"].startswith("mmq_"))
+    calls = []
+
+    def measure(assign):
+        calls.append({k: dict(v) for k, v in assign.items()})
+        t = 10.0
+        # the ping-pong tile for "dw" is worth 1.0, but only while "fwd" keeps its first plan
+        if assign["dw"]["tile_id"] == pp and assign["dw"]["split_k"] == 2 and assign["fwd"] == slots["fwd"][0]:
+            t -= 1.0
+        if assign["fwd"]["tile_id"] == pp:
+            t -= 0.01                                   # below min_gain: noise
+        if assign["dw"]["group_m"] == 4 and assign["dw"]["xcd_rotate"] is True:
+            t -= 0.2
+        return t
+
+    slots = {"fwd": K.plan_candidates(8192, 3072, 768, K.L.MG_NT), "dw": cands}
+    assign, best, log = K.tune_in_context(slots, measure, passes=3, min_gain=0.003)
+    assert assign["dw"]["tile_id"] == pp and assign["dw"]["split_k"] == 2
+    assert assign["dw"]["group_m"] == 4 and assign["dw"]["xcd_rotate"] is True
+    assert assign["fwd"] == slots["fwd"][0] and abs(best - 8.8) < 1e-9
+    assert [x[0] for x in log] == ["start", "dw", "dw"]
+    # a kept change was measured twice in a row with the same assignment
+    i = next(i for i, c in enumerate(calls) if c["dw"]["tile_id"] == pp and c["dw"]["split_k"] == 2)
+    assert calls[i] == calls[i + 1]
+    # keys: the context is part of the key, and lookup falls back to the plan tuned alone
+    k0 = K.tune_key("d", 8, 9, 10, True, False, "bf16")
+    k1 = K.tune_key("d", 8, 9, 10, True, False, "bf16", context="gpt2s-dw-stream")
+    assert k1 == k0 + "|in:gpt2s-dw-stream"
+    K._save_cache({k0: dict(cands[0], tile_id=3), k1: dict(cands[0], tile_id=pp)})
+    assert K.lookup_tuned("d", 8, 9, 10, True, False, "bf16")["tile_id"] == 3
+    assert K.lookup_tuned("d", 8, 9, 10, True, False, "bf16", context="gpt2s-dw-stream")["tile_id"] == pp
+    assert K.lookup_tuned("d", 8, 9, 10, True, False, "bf16", context="another")["tile_id"] == 3
+    assert K.lookup_tuned("d", 8, 9, 11, True, False, "bf16", context="gpt2s-dw-stream") is None
+
+
 def test_graph_state_errors():
     from vkgrad_amd.vk import Graph, VkError
     g = Graph(FakeDev(), "g")

@@ -94,19 +94,23 @@ def _run_mm(dev, mm, a, b, m, n, k, lda=None, ldb=None, ldc=None, c_in=None, nba
 # ---------------------------------------------------------------------------
 
 def _bench_cases():
-    """Every GEMM of the benchmark step, and the three LM-head GEMMs once more with logits
-    rows exactly 50257 elements apart (the step bench.py reports as `dense_head`)."""
+    """Every GEMM of the benchmark step with the plan chosen alone (the in-order schedule and
+    the fallback of every other) and with the plan chosen inside the step of the default
+    schedule, and the three LM-head GEMMs once more with logits rows exactly 50257 elements
+    apart (the step bench.py reports as `dense_head`)."""
     import bench
-    cases = [(name, layout, m, n, k, False) for name, layout, m, n, k, _ in bench.gemm_list()]
-    return cases + [c[:5] + (True,) for c in cases if c[0].startswith("head")]
+    cases = [(name, layout, m, n, k, False, None) for name, layout, m, n, k, _ in bench.gemm_list()]
+    ctx = bench.context_of("dw-stream")
+    return (cases + [c[:6] + (ctx,) for c in cases] +
+            [c[:5] + (True, x) for c in cases if c[0].startswith("head") for x in (None, ctx)])
 
 
-@pytest.mark.parametrize("name,layout,m,n,k,dense", _bench_cases(),
-                         ids=[c[0] + (".dense" if c[5] else "") for c in _bench_cases()])
-def test_benchmark_plan_at_full_size(dev, name, layout, m, n, k, dense):
+@pytest.mark.parametrize("name,layout,m,n,k,dense,context", _bench_cases(),
+                         ids=[c[0] + (".dense" if c[5] else "") + ("@" + c[6] if c[6] else "") for c in _bench_cases()])
+def test_benchmark_plan_at_full_size(dev, name, layout, m, n, k, dense, context):
     import bench
     vpitch = bench.head_pitch(dense)
-    mm, kw = bench.plan_for(dev, name, layout, m, n, k, vpitch)
+    mm, kw = bench.plan_for(dev, name, layout, m, n, k, vpitch, context)
     assert (kw == {}) == (dense or not name.startswith("head"))
     if os.path.exists(os.path.join(ROOT, "vkgrad_amd", "tuned_mi355x.json")) and dev.name.startswith("gfx950"):
         assert mm.tile >= 0, f"{name}: the tuned table has no plan for this shape (the benchmark would run the picker)"
@@ -129,7 +133,8 @@ def test_benchmark_plan_at_full_size(dev, name, layout, m, n, k, dense):
 # ---------------------------------------------------------------------------
 
 _KEY = re.compile(r"^(?P<dev>.*)\|(?P<m>\d+)x(?P<n>\d+)x(?P<k>\d+)\|ta(?P<ta>[01])tb(?P<tb>[01])\|(?P<dt>f16|bf16)"
-                  r"(?P<acc>\|acc)?(?:\|bat(?P<bat>\d+))?(?:\|ld(?P<lda>\d+),(?P<ldb>\d+),(?P<ldc>\d+))?$")
+                  r"(?P<acc>\|acc)?(?:\|bat(?P<bat>\d+))?(?:\|ld(?P<lda>\d+),(?P<ldb>\d+),(?P<ldc>\d+))?"
+                  r"(?:\|in:(?P<ctx>[\w-]+))?$")
 
 
 def _table():
@@ -143,7 +148,7 @@ def _table_ids():
 
 @pytest.mark.parametrize("key", list(_table()), ids=_table_ids())
 def test_tuned_table_entry_is_exact_at_its_shape(dev, key):
-    from vkgrad_amd.kernels import Matmul
+    from vkgrad_amd.kernels import matmul_from_entry
     e = _table()[key]
     g = _KEY.match(key)
     assert g, f"unparsable tuned-table key {key!r}"
@@ -154,8 +159,7 @@ def test_tuned_table_entry_is_exact_at_its_shape(dev, key):
     # a pitch equal to the default says nothing
     dflt = dict(lda=m if ta else k, ldb=k if tb else n, ldc=n)
     pitch = {x: v for x, v in pitch.items() if v != dflt[x]}
-    mm = Matmul(dev, trans_a=ta, trans_b=tb, batched=nbatch > 1, dtype=dtype, tile=e["tile_id"],
-                split_k=e.get("split_k", 0), group_m=e.get("group_m", 0), atomic_split=e.get("atomic_split", False))
+    mm = matmul_from_entry(dev, e, ta, tb, dtype, nbatch > 1)
     rng = np.random.default_rng(len(key) * 7919 + m + 3 * n + 5 * k)
     sa, sb = _stored(m, n, k, ta, tb)
     if nbatch > 1:

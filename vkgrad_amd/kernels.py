@@ -405,37 +405,125 @@ def _pitch_tag(m, n, k, trans_a, trans_b, lda, ldb, ldc):
 
 
 def tune_key(dev_name, m, n, k, trans_a, trans_b, dtype="f16", batched=False, nbatch=1,
-             accumulate=False, lda=None, ldb=None, ldc=None):
-    """Cache key; the reference's shape (kernels.py:459-460) plus dtype, beta and pitches."""
+             accumulate=False, lda=None, ldb=None, ldc=None, context=None):
+    """Cache key; the reference's shape (kernels.py:459-460) plus dtype, beta and pitches, and the
+    context a plan was tuned in when that is not "alone" (see tune_in_context)."""
     return (f"{dev_name}|{m}x{n}x{k}|ta{int(trans_a)}tb{int(trans_b)}|{dtype}"
             f"{'|acc' if accumulate else ''}{'|bat' + str(nbatch) if batched else ''}"
-            f"{_pitch_tag(m, n, k, trans_a, trans_b, lda, ldb, ldc)}")
+            f"{_pitch_tag(m, n, k, trans_a, trans_b, lda, ldb, ldc)}{'|in:' + context if context else ''}")
 
 
 def lookup_tuned(dev_name, m, n, k, trans_a, trans_b, dtype="f16", batched=False, nbatch=1,
-                 accumulate=False, lda=None, ldb=None, ldc=None):
-    """Cached pick for a shape, user cache first, then the shipped table."""
-    key = tune_key(dev_name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate, lda, ldb, ldc)
-    for path in (_TUNE_CACHE, _SHIPPED_CACHE):
-        e = _load_cache(path).get(key)
-        if e is not None:
-            return e
+                 accumulate=False, lda=None, ldb=None, ldc=None, context=None):
+    """Cached pick for a shape, user cache first, then the shipped table; with a context, the
+    pick made in that context if there is one, else the one made alone."""
+    for ctx in ((context, None) if context else (None,)):
+        key = tune_key(dev_name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate, lda, ldb, ldc, ctx)
+        for path in (_TUNE_CACHE, _SHIPPED_CACHE):
+            e = _load_cache(path).get(key)
+            if e is not None:
+                return e
     return None
 
 
+def matmul_from_entry(dev, e, trans_a=False, trans_b=False, dtype="f16", batched=False):
+    """The Matmul a cache entry (or a candidate of tune_in_context) describes."""
+    return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, dtype=dtype, tile=e["tile_id"],
+                  split_k=e.get("split_k", 0), group_m=e.get("group_m", 0),
+                  atomic_split=e.get("atomic_split", False), xcd_rotate=e.get("xcd_rotate"))
+
+
 def tuned_matmul(dev, m, n, k, trans_a=False, trans_b=False, dtype="f16", batched=False, nbatch=1,
-                 accumulate=False, lda=None, ldb=None, ldc=None):
+                 accumulate=False, lda=None, ldb=None, ldc=None, context=None):
     """(Matmul, how) for one shape as the benchmarks run it: the cached pick (tile,
-    K split, rasterisation band, split mode) when a cache holds the shape, else a
+    K split, rasterisation band, split mode, walk) when a cache holds the shape, else a
     Matmul that leaves the choice to the library's picker.  how is 'tuned table' or
     'picker'.  The parity tests build their GEMMs through this same function, so what
     is timed is what is checked."""
-    e = lookup_tuned(dev.name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate, lda, ldb, ldc)
+    e = lookup_tuned(dev.name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate, lda, ldb, ldc, context)
     if e is None:
         return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, dtype=dtype), "picker"
-    return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, dtype=dtype, tile=e["tile_id"],
-                  split_k=e.get("split_k", 0), group_m=e.get("group_m", 0),
-                  atomic_split=e.get("atomic_split", False), xcd_rotate=e.get("xcd_rotate")), "tuned table"
+    return matmul_from_entry(dev, e, trans_a, trans_b, dtype, batched), "tuned table"
+
+
+def plan_candidates(m, n, k, layout, cus=256, splits=(1, 2, 3, 4, 6, 8)):
+    """Candidate plans for tune_in_context: one tile of every family and size (64 x 64
+    register-staged, the direct-to-LDS 128 x 128 with 64- and 32-wide K-blocks, 128 x 256,
+    256 x 128, the persistent 128 x 128, the ping-pong 256 x 256) with K splits from none up to
+    where a slice has fewer than four K-blocks or the grid has more than twice the resident
+    workgroups - beside another stream's kernels a GEMM is often better off with few, large
+    workgroups than with the grid that fills the chip by itself - each split both through
+    the workspace and with atomics."""
+    fams = [t for t in CONFIGS if t["name"] in ("mm_64x64x64_w2x2", "mmd_128x128x64_w2x2_s2", "mmd_128x128x32_w2x2_s3",
+                                                "mmd_128x256x32_w2x2_s3", "mmd_256x128x32_w2x2_s3",
+                                                "mmp_128x128x64_w2x2_s2", "mmq_256x256x64_w2x4_s2")]
+    out = []
+    for t in fams:
+        tiles = -(-m // t["bm"]) * -(-n // t["bn"])
+        if tiles * t["bm"] * t["bn"] > 2.0 * m * n:
+            continue                                    # more padding than matrix
+        for sp in splits:
+            if sp > 1 and (k // (4 * t["bk"]) < sp or tiles * sp > 4 * cus):
+                continue
+            for at in ((False, True) if sp > 1 else (False,)):
+                out.append({"tile_id": t["id"], "split_k": sp, "atomic_split": at, "group_m": 0, "xcd_rotate": None,
+                            "tile": [t["bm"], t["bn"]], "config": [t["bm"], t["bn"], t["bk"]], "lds": True})
+    return out
+
+
+def tune_in_context(slots, measure, passes=2, min_gain=0.003, refine=True, verbose=False):
+    """Plans for GEMMs that run beside each other, chosen by what the whole sequence takes.
+
+    The per-shape tuner times a GEMM alone; a GEMM that shares the chip with another stream's
+    kernels wants a different plan (a weight-gradient GEMM beside the forward / dX chain of a
+    training step: fewer, larger workgroups than the grid that is fastest alone).  slots maps
+    a name to its candidate plans (dicts with tile_id, split_k, atomic_split, group_m,
+    xcd_rotate), the first being the current one; measure(assignment) returns the seconds the
+    sequence takes with {name: plan}.  Coordinate descent: for one slot after the other every
+    candidate is measured with the others held, and kept when it beats the held plan by more
+    than min_gain (relative; below that a difference is noise); `passes` sweeps or until a
+    sweep changes nothing.  With refine, a last sweep tries the rasterisation band and the walk
+    of the XCDs on each kept plan.  Returns (assignment, seconds, log); no counterpart in the
+    reference, whose steps run on one queue (vk.py:848-851)."""
+    cur = {name: dict(c[0]) for name, c in slots.items()}
+    best = measure(cur)
+    log = [("start", None, best)]
+
+    def sweep(options_of):
+        nonlocal best
+        changed = False
+        for name in slots:
+            held, held_t = cur[name], best
+            for cand in options_of(name):
+                if cand == held:
+                    continue
+                cur[name] = cand
+                t = measure(cur)
+                if verbose:
+                    print(f"    {name}: tile {cand['tile_id']} split {cand['split_k']}{' at' if cand['atomic_split'] else ''} "
+                          f"g{cand['group_m']} walk {cand['xcd_rotate']}: {t * 1e3:.4f} ms (held {held_t * 1e3:.4f})", flush=True)
+                if t < held_t * (1.0 - min_gain):
+                    # confirm: a second measurement must agree before a plan is replaced
+                    t2 = measure(cur)
+                    if t2 < held_t * (1.0 - min_gain):
+                        held, held_t = cand, max(t, t2)
+            cur[name] = held
+            if held_t < best:
+                changed = True
+                log.append((name, dict(held), held_t))
+            best = held_t
+        return changed
+
+    for _ in range(passes):
+        if not sweep(lambda name: [dict(c) for c in slots[name]]):
+            break
+    if refine:
+        def variants(name):
+            base = cur[name]
+            walks = (True, False) if walk_matters(base["tile_id"]) else (base["xcd_rotate"],)
+            return [dict(base, group_m=g, xcd_rotate=w) for g in (0, 1, 2, 4, 16) for w in walks]
+        sweep(variants)
+    return cur, best, log
 
 
 _WARMED = set()
@@ -571,9 +659,7 @@ def autotune_matmul(dev, m, n, k, trans_a=False, trans_b=False, reps=3, verbose=
     if use_cache:
         e = lookup_tuned(dev.name, m, n, k, trans_a, trans_b, dtype, batched, nbatch, accumulate, lda, ldb, ldc)
         if e is not None:
-            return Matmul(dev, trans_a=trans_a, trans_b=trans_b, batched=batched, tile=e["tile_id"],
-                          dtype=dtype, split_k=e.get("split_k", 0), group_m=e.get("group_m", 0),
-                          atomic_split=e.get("atomic_split", False), xcd_rotate=e.get("xcd_rotate")), e
+            return matmul_from_entry(dev, e, trans_a, trans_b, dtype, batched), e
 
     nb = nbatch if batched else 1
     pa = int(lda) if lda is not None else (m if trans_a else k)      # row pitches
