@@ -102,12 +102,13 @@ def context_of(schedule):
 # only valid for the (tile, split_k) it was measured with; for another plan the
 # bench line reports null.  gemm -> (tile, split_k, fetch bytes, write bytes)
 MEASURED_TRAFFIC = {
-    "qkv.fwd": (21, 1, 46.5e6, 75.5e6), "qkv.dX": (11, 1, 66.2e6, 25.2e6), "qkv.dW": (17, 4, 95.7e6, 35.4e6),
-    "proj.fwd": (11, 1, 22.2e6, 25.2e6), "proj.dX": (11, 1, 22.2e6, 25.2e6),
-    "proj.dW": (4, 5, 106.3e6, 14.2e6), "fc1.fwd": (21, 1, 63.1e6, 100.8e6), "fc1.dX": (11, 1, 91.5e6, 25.2e6),
-    "fc1.dW": (11, 3, 227.0e6, 37.8e6), "fc2.fwd": (3, 1, 106.2e6, 25.2e6), "fc2.dX": (21, 1, 63.4e6, 100.7e6),
-    "fc2.dW": (17, 3, 122.0e6, 37.8e6), "head.fwd": (21, 1, 769.2e6, 1649.1e6),
-    "head.dX": (21, 8, 1650.1e6, 226.5e6), "head.dW": (21, 1, 1261.7e6, 218.1e6),
+    "qkv.fwd": (21, 1, 52.1e6, 75.5e6), "qkv.dX": (11, 1, 66.2e6, 25.2e6), "qkv.dW": (21, 1, 151.2e6, 7.1e6),
+    "proj.fwd": (11, 1, 22.2e6, 25.2e6), "proj.dX": (14, 1, 22.2e6, 25.2e6),
+    "proj.dW": (17, 4, 47.4e6, 11.8e6), "fc1.fwd": (21, 1, 76.9e6, 100.7e6),
+    "fc1.dX": (21, 1, 126.1e6, 25.2e6), "fc1.dW": (11, 2, 260.1e6, 28.3e6), "fc2.fwd": (11, 1, 90.8e6, 25.2e6),
+    "fc2.dX": (21, 1, 77.8e6, 100.7e6), "fc2.dW": (11, 3, 192.0e6, 37.8e6),
+    "head.fwd": (21, 1, 733.4e6, 1647.6e6), "head.dX": (21, 8, 1662.6e6, 226.5e6),
+    "head.dW": (21, 1, 1464.0e6, 218.1e6),
 }
 
 
@@ -583,7 +584,9 @@ def main():
         ts = sorted(seen[r["gemm"]])
         r["us_in_step"] = round(ts[len(ts) // 2] * 1e6, 2)
     in_step_ms = sorted(passes)[2] * 1e3
-    dom = max(per_shape, key=lambda r: r["us"] * r["count"])
+    # the dominant kernel: the GEMM with the largest share of the step's arithmetic (the LM-head
+    # forward; under the two-stream schedule the time of a GEMM alone says nothing about its share)
+    dom = max(per_shape, key=lambda r: 2.0 * r["m"] * r["n"] * r["k"] * r["count"])
     mt = MEASURED_TRAFFIC.get(dom["gemm"])
     traffic = None
     if mt and (mt[0], mt[1]) == (dom["tile"], dom["split_k"]) and not args.dense_head:
