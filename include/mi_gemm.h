@@ -456,6 +456,19 @@ int mg_tk_attn_rowdot(mg_ctx *ctx, const void *a16, const float *b32, float *out
 int mg_tk_attn_p_supported(int64_t hd, int64_t T);
 int mg_tk_attn_p(mg_ctx *ctx, const void *q16, const void *k16, const uint32_t *seg, void *p16, int64_t nbh, int64_t T,
                  int64_t H, int64_t hd, float scale, int causal, int dtype);
+/* Attention forward in one kernel: mg_tk_attn_p and the Out = P V product over the heads after it
+ * (transformer.py:153-159; attn_softmax / attn_softmax_doc tkernels.py:105-165), so that P is written
+ * (the backward pass reads it) but not read back: p16 as from mg_tk_attn_p, and
+ *   out32[b][i][d] = sum_j p16[b][i][j] * v16[b][j][d]      (nbh, T, hd) f32, head-side,
+ * the 16-bit P as stored times V with f32 sums (a GEMM over the stored P gives the same up to the
+ * order of the sums).  out16 (or NULL): the same values narrowed, in the merged (B*T, H*hd) layout
+ * of merge_heads (tkernels.py:274-286).  hd in {32, 64, 128}, T a multiple of 8 up to 1024
+ * (mg_tk_attn_fwd_supported); q16, k16, v16 (nbh, T, hd) and p16 16-byte aligned.  causal != 0:
+ * blocks of 32 queries x 256 keys wholly beyond the diagonal are not written - keep p16 zero there. */
+int mg_tk_attn_fwd_supported(int64_t hd, int64_t T);
+int mg_tk_attn_fwd(mg_ctx *ctx, const void *q16, const void *k16, const void *v16, const uint32_t *seg, void *p16,
+                   float *out32, void *out16, int64_t nbh, int64_t T, int64_t H, int64_t hd, float scale, int causal,
+                   int dtype);
 /* dS of attention in one kernel: the dP = dOut V^T product over the heads (transformer.py:171-173)
  * and attn_softmax_bwd (tkernels.py:167-187) after it, without the f32 dP in between:
  *   ds16[b][i][j] = narrow(scale * p16[b][i][j] * (sum_d dout16[b][i][d] * v16[b][j][d] - rowsub[b][i]))

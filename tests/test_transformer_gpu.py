@@ -201,6 +201,69 @@ def test_scores_and_softmax_in_one_kernel(dev, tk):
     assert not dev._lib.mg_tk_attn_p_supported(64, 100)
 
 
+def test_attention_forward_in_one_kernel(dev, tk):
+    """attn_fwd: P as attn_p writes it (bit for bit: the same arithmetic) and Out = P V behind
+    it in the same kernel.  Out is checked against the product of the 16-bit P the kernel stored
+    with V, summed in float64 (tolerance: f32 sums of up to 1024 terms, 2e-5 of the largest
+    entry plus 1e-5 relative), and P against the oracle's softmax as in the test above; the
+    optional 16-bit output must be Out narrowed, in the merged (B*T, H*hd) layout.  Head widths
+    32 / 64 / 128; T of one block of queries, of a ragged last block, beyond one wavefront's 256
+    keys and of all four; plain causal and packed samples (seg), with and without the causal
+    skipping; what the kernel does not take is refused."""
+    dtype, TK = tk
+    rng = np.random.default_rng(21)
+    lib = dev._lib
+    for B, H, T, hd in ((1, 2, 72, 64), (2, 3, 264, 32), (1, 1, 1024, 64), (1, 2, 520, 128), (2, 1, 136, 64),
+                        (1, 2, 8, 32), (1, 1, 1024, 128), (2, 2, 1024, 32), (1, 3, 264, 128), (1, 1, 776, 64)):
+        nbh, rows, D = B * H, B * H * T, H * hd
+        scale = 1.0 / np.sqrt(hd)
+        assert lib.mg_tk_attn_fwd_supported(hd, T)
+        q16 = O.round_to((rng.standard_normal((nbh, T, hd)) * 1.5).astype(np.float32), dtype)
+        k16 = O.round_to((rng.standard_normal((nbh, T, hd)) * 1.5).astype(np.float32), dtype)
+        v16 = O.round_to((rng.standard_normal((nbh, T, hd)) * 2.0 + 0.25).astype(np.float32), dtype)
+        sc = np.einsum("bid,bjd->bij", O.widen(q16, dtype), O.widen(k16, dtype)).astype(np.float32).reshape(rows, T)
+        seg = np.zeros(B * T, np.uint32)
+        for b in range(B):
+            cut = 1 + (7 * b + T // 3) % (T - 1)
+            seg[b * T + cut:(b + 1) * T] = cut
+        bq, bk, bv, bseg = up(dev, q16), up(dev, k16), up(dev, v16), up(dev, seg)
+        bp, bp2 = dev.buffer(rows * T * 2, "device"), dev.buffer(rows * T * 2, "device")
+        bo, bo16 = dev.buffer(rows * hd * 4, "device"), dev.buffer(rows * hd * 2, "device")
+        try:
+            for use_seg in (False, True):
+                want = RT.attn_softmax(sc, T, scale, dtype, seg=seg if use_seg else None, H=H)
+                for causal in (False, True):
+                    for with16 in (False, True):
+                        for x in (bp, bp2):
+                            x.upload(np.zeros(rows * T, np.uint16))
+                        bo.upload(np.full(rows * hd, np.nan, np.float32))
+                        bo16.upload(np.full(rows * hd, 0x7FFF, np.uint16))
+                        sg = bseg if use_seg else None
+                        TK["attn_p"]([bq, bk, sg, bp2], nbh, T, H, hd, scale, causal)
+                        TK["attn_fwd"]([bq, bk, bv, sg, bp, bo, bo16 if with16 else None], nbh, T, H, hd, scale, causal)
+                        got = stored(bp, dtype, (rows, T))
+                        case = (B, H, T, hd, use_seg, causal, with16)
+                        assert np.array_equal(np.asarray(got).view(np.uint16), np.asarray(stored(bp2, dtype, (rows, T))).view(np.uint16)), case
+                        assert close16(got, want, dtype, slack=2e-5), case
+                        out = bo.download(np.float32, (nbh, T, hd))
+                        ref = np.einsum("bij,bjd->bid", O.widen(got, dtype).reshape(nbh, T, T).astype(np.float64),
+                                        O.widen(v16, dtype).astype(np.float64))
+                        assert np.isfinite(out).all(), case
+                        tol = 2e-5 * np.abs(ref).max() + 1e-5 * np.abs(ref)
+                        assert np.all(np.abs(out - ref) <= tol), (case, float(np.abs(out - ref).max()))
+                        raw16 = bo16.download(np.uint16, (B, T, H, hd))
+                        if with16:
+                            merged = out.reshape(B, H, T, hd).transpose(0, 2, 1, 3)
+                            assert np.array_equal(raw16, np.asarray(O.round_to(np.ascontiguousarray(merged), dtype)).view(np.uint16)), case
+                        else:
+                            assert np.all(raw16 == 0x7FFF), case
+        finally:
+            for t in (bq, bk, bv, bseg, bp, bp2, bo, bo16):
+                t.destroy()
+    assert not lib.mg_tk_attn_fwd_supported(64, 1032) and not lib.mg_tk_attn_fwd_supported(40, 64)
+    assert not lib.mg_tk_attn_fwd_supported(64, 100) and lib.mg_tk_attn_fwd_supported(128, 1024)
+
+
 def test_head_permutes(dev, tk):
     dtype, TK = tk
     rng = np.random.default_rng(2)

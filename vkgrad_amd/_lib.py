@@ -138,6 +138,8 @@ SIGNATURES = {
     "mg_tk_attn_rowdot": (C.c_int, [_P, _P, _P, _P, _I, _I, C.c_int]),
     "mg_tk_attn_p_supported": (C.c_int, [_I, _I]),
     "mg_tk_attn_p": (C.c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, C.c_float, C.c_int, C.c_int]),
+    "mg_tk_attn_fwd_supported": (C.c_int, [_I, _I]),
+    "mg_tk_attn_fwd": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, C.c_float, C.c_int, C.c_int]),
     "mg_tk_attn_ds_supported": (C.c_int, [_I, _I]),
     "mg_tk_attn_ds": (C.c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, C.c_float, C.c_int, C.c_int]),
     "mg_tk_split_qkv": (C.c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, C.c_int]),

@@ -37,6 +37,17 @@ typedef _Float16 ak_half8 __attribute__((ext_vector_type(8)));
 typedef __bf16 ak_bf8 __attribute__((ext_vector_type(8)));
 typedef float ak_f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t ak_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t ak_u32x2 __attribute__((ext_vector_type(2)));
+typedef short ak_short4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) ak_short4 ak_lds_short4;
+
+// Transposing LDS read (ds_read_b64_tr_b16): within each group of 16 lanes the 16 x 8-byte pieces
+// addressed by the lanes form a 4 x 16 matrix of 16-bit elements (lane j supplies row j / 4,
+// columns 4 (j % 4) .. + 3); lane j receives column j.
+__device__ __forceinline__ ak_u32x2 ak_read_tr(const uint16_t *p) {
+    ak_short4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((ak_lds_short4 *)p);
+    return __builtin_bit_cast(ak_u32x2, v);
+}
 
 template <int DT>
 __device__ __forceinline__ ak_f32x16 ak_mfma(ak_u32x4 a, ak_u32x4 b, ak_f32x16 c) {
@@ -253,6 +264,181 @@ k_attn_p(const uint16_t *q16, const uint16_t *k16, const uint32_t *seg, uint16_t
         }
 }
 
+// Attention forward in one kernel: the one-walk P kernel above with the Out = P V product of
+// every head (reference call site transformer.py:157-159) behind it, so that P is written (the
+// backward pass reads it, transformer.py:165-176) but not read back.  P leaves the softmax in
+// accumulator layout with the keys along the rows and one query per lane, 16 neighbouring keys
+// per lane and block: narrowed, the eight keys of a 16-byte store are exactly what a lane holds
+// of the B operand of v_mfma_f32_32x32x16 for the product Out^T = V^T P^T (k = keys, columns =
+// queries), so the same 16-bit values that go to memory go to the matrix cores and the result
+// is what a GEMM over the stored P gives, up to the order of the f32 sums.  The A operand, V^T,
+// is 8 keys of one column of V per lane: every wavefront passes the 32 rows of V of a key block
+// through a buffer of its own in LDS (rows padded so that the four rows and two column groups
+// of a transposing read fall on different banks) and reads them back with ds_read_b64_tr_b16;
+// the rows of the next block are requested before the current one is multiplied.  Key blocks
+// wholly beyond the workgroup's queries hold P = 0 and are not multiplied.  The four
+// wavefronts (256 keys each) then meet in LDS with their partial Out (32 queries x HD floats
+// each) and the workgroup adds them in wavefront order and writes Out in f32 (head-side, the
+// row term of the softmax backward reads it, autograd of transformer.py:171-176) and, if asked,
+// narrowed in the merged (B*T, D) layout the projection reads (merge_heads, tkernels.py:274-286).
+template <int HD>
+constexpr int fwd_pitch() { return HD == 32 ? 64 : HD * 2 + 64; }   // bytes per row of V in LDS
+
+// (heads 128 wide need 270 registers: one workgroup per CU there, two otherwise)
+template <int DT, int HD>
+__global__ void __launch_bounds__(256, (HD == 128 ? 1 : 2))
+k_attn_fwd(const uint16_t *q16, const uint16_t *k16, const uint16_t *v16, const uint32_t *seg, uint16_t *p16,
+           float *out32, uint16_t *out16, int T, int H, float scale, int causal) {
+    constexpr int KK = HD / 16, NB = 8, MB = HD / 32;
+    constexpr int PITCH = fwd_pitch<HD>(), VBUF = 32 * PITCH;
+    constexpr int OPITCH = HD + 1;                       // floats per query of a partial Out
+    constexpr int LDS_V = 4 * VBUF, LDS_O = 4 * 32 * OPITCH * 4;
+    constexpr int CPR = HD / 8, RPI = 64 / CPR, NLD = 32 / RPI;   // staging of a key block: 16-byte chunks per row, rows per load, loads
+    __shared__ __attribute__((aligned(16))) char smem[LDS_V > LDS_O ? LDS_V : LDS_O];
+    __shared__ float part_m[4][32], part_l[4][32];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t b = blockIdx.y;
+    const int i0 = blockIdx.x * 32;      // the workgroup's first query
+    const int j0 = wave * 256;           // this wavefront's first key
+    const int n = lane & 31, half = lane >> 5, fk = half * 8;
+    const int q = i0 + n;                // this lane's query
+    // keys that no query of this block sees hold P = 0: not written with `causal`, never multiplied
+    const bool beyond = j0 >= T || j0 > i0 + 31;
+    const bool idle = j0 >= T || (causal && j0 > i0 + 31);
+    ak_f32x16 acc[NB];
+    float m = -1e30f, l = 0.f;
+    if (!idle) {
+        const uint16_t *qb = q16 + b * (int64_t)T * HD + (int64_t)min(q, T - 1) * HD + fk;
+        const uint16_t *kb = k16 + b * (int64_t)T * HD;
+        ak_u32x4 bf[KK];                 // B operand: the queries
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) bf[kk] = *reinterpret_cast<const ak_u32x4 *>(qb + kk * 16);
+        const int first = seg ? (int)seg[(b / H) * T + min(q, T - 1)] : 0;
+        // A operand row n = 8g + 4h' + e of block t is key j0 + 32 t + 16 h' + 4 g + e
+        const int arow = 16 * ((n >> 2) & 1) + 4 * (n >> 3) + (n & 3);
+#pragma unroll
+        for (int t = 0; t < NB; t++) {
+            const uint16_t *ap = kb + (int64_t)min(j0 + 32 * t + arow, T - 1) * HD + fk;
+            ak_u32x4 af[KK];
+#pragma unroll
+            for (int kk = 0; kk < KK; kk++) af[kk] = *reinterpret_cast<const ak_u32x4 *>(ap + kk * 16);
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < KK; kk++) acc[t] = ak_mfma<DT>(af[kk], bf[kk], acc[t]);
+        }
+        // base-2 domain, masked keys at -1e30 (see k_attn_p)
+        const float c2 = scale * 1.4426950408889634f;
+        const int k0 = j0 + 16 * half;   // register r of block t: key k0 + 32 t + r
+#pragma unroll
+        for (int t = 0; t < NB; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int key = k0 + 32 * t + r;
+                acc[t][r] = (key >= first && key <= q) ? acc[t][r] * c2 : -1e30f;
+                m = fmaxf(m, acc[t][r]);
+            }
+        m = fmaxf(m, __shfl_xor(m, 32, 64));
+#pragma unroll
+        for (int t = 0; t < NB; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float e = __builtin_amdgcn_exp2f(acc[t][r] - m);
+                acc[t][r] = e;
+                l += e;
+            }
+        l += __shfl_xor(l, 32, 64);
+    }
+    if (half == 0) {
+        part_m[wave][n] = m;
+        part_l[wave][n] = l;
+    }
+    __syncthreads();
+    ak_f32x16 oacc[MB];
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[i][r] = 0.f;
+    if (!idle) {
+        const float m0 = part_m[0][n], m1 = part_m[1][n], m2 = part_m[2][n], m3 = part_m[3][n];
+        const float mx = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
+        const float sum = part_l[0][n] * __builtin_amdgcn_exp2f(m0 - mx) + part_l[1][n] * __builtin_amdgcn_exp2f(m1 - mx) +
+                          part_l[2][n] * __builtin_amdgcn_exp2f(m2 - mx) + part_l[3][n] * __builtin_amdgcn_exp2f(m3 - mx);
+        const float f = __builtin_amdgcn_exp2f(m - mx) / sum;
+        uint16_t *pq = p16 + b * (int64_t)T * T + (int64_t)min(q, T - 1) * T + j0 + 16 * half;
+        // key blocks of this wavefront that some query of the workgroup sees (0 when all lie beyond)
+        const int kend = min(min(T, j0 + 256), i0 + 32);
+        const int nblk = beyond ? 0 : (kend - j0 + 31) / 32;
+        // staging of V: lane l fetches chunk l % CPR of row l / CPR + RPI i of the block
+        const uint16_t *vbase = v16 + b * (int64_t)T * HD;
+        const int lrow = lane / CPR, lch = lane % CPR;
+        char *vb = smem + wave * VBUF;
+        char *vdst = vb + lrow * PITCH + lch * 16;
+        // transposing read: lane (j = l % 16, g = l / 16) supplies the 8-byte piece of row 16 (g / 2) + j / 4
+        // (+ 8 u, + 4 for the second read), columns 16 (g % 2) + 4 (j % 4) .. + 3, and receives column l % 32
+        const int j = lane & 15, g4 = lane >> 4;
+        const char *vsrc = vb + ((g4 >> 1) * 16 + (j >> 2)) * PITCH + ((g4 & 1) * 16 + (j & 3) * 4) * 2;
+        ak_u32x4 vreg[NLD];
+        auto load_v = [&](int t) {
+#pragma unroll
+            for (int i = 0; i < NLD; i++)
+                vreg[i] = *reinterpret_cast<const ak_u32x4 *>(vbase + (int64_t)min(j0 + 32 * t + lrow + RPI * i, T - 1) * HD + lch * 8);
+        };
+        if (nblk > 0) load_v(0);
+#pragma unroll
+        for (int t = 0; t < NB; t++) {
+            const bool mul = t < nblk;       // uniform over the wavefront
+            if (mul) {
+#pragma unroll
+                for (int i = 0; i < NLD; i++) *reinterpret_cast<ak_u32x4 *>(vdst + RPI * i * PITCH) = vreg[i];
+                if (t + 1 < nblk) load_v(t + 1);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the block is in LDS before it is read back
+            }
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                ak_u32x4 o;
+#pragma unroll
+                for (int w = 0; w < 4; w++)
+                    o[w] = ak_narrow<DT>(acc[t][8 * u + 2 * w] * f) | (ak_narrow<DT>(acc[t][8 * u + 2 * w + 1] * f) << 16);
+                // T is a multiple of 8: the eight keys of a store exist or none does
+                if (q < T && j0 + 16 * half + 32 * t + 8 * u < T) *reinterpret_cast<ak_u32x4 *>(pq + 32 * t + 8 * u) = o;
+                if (mul) {
+#pragma unroll
+                    for (int i = 0; i < MB; i++) {
+                        const uint16_t *vp = reinterpret_cast<const uint16_t *>(vsrc + 8 * u * PITCH + i * 64);
+                        const ak_u32x2 lo = ak_read_tr(vp);
+                        const ak_u32x2 hi = ak_read_tr(reinterpret_cast<const uint16_t *>(reinterpret_cast<const char *>(vp) + 4 * PITCH));
+                        oacc[i] = ak_mfma<DT>(ak_u32x4{lo[0], lo[1], hi[0], hi[1]}, o, oacc[i]);
+                    }
+                }
+            }
+            if (mul) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // read back before the next block overwrites it
+        }
+    }
+    __syncthreads();                         // every wavefront is done with its V buffer
+    float *po = reinterpret_cast<float *>(smem);
+    if (!beyond) {
+#pragma unroll
+        for (int i = 0; i < MB; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                po[(wave * 32 + n) * OPITCH + 32 * i + (r >> 2) * 8 + half * 4 + (r & 3)] = oacc[i][r];
+    }
+    __syncthreads();
+    // wavefronts with keys to add: 0 .. nw - 1
+    const int nw = min(4, min((T + 255) / 256, (i0 + 31) / 256 + 1));
+    const int64_t bb = b / H, hh = b % H;
+    for (int e = threadIdx.x; e < 32 * HD; e += 256) {
+        const int qq = e / HD, d = e % HD;
+        if (i0 + qq >= T) break;
+        float sacc = 0.f;
+        for (int w = 0; w < nw; w++) sacc += po[(w * 32 + qq) * OPITCH + d];
+        out32[b * (int64_t)T * HD + (int64_t)(i0 + qq) * HD + d] = sacc;
+        if (out16) out16[(bb * T + i0 + qq) * ((int64_t)H * HD) + hh * HD + d] = (uint16_t)ak_narrow<DT>(sacc);
+    }
+}
+
 // The same for heads up to 64 wide and any T (a multiple of 8), for rows longer than the 1024 keys
 // the kernel above can hold: a workgroup is four blocks of 32 queries (queries along the
 // accumulator rows here, as in k_attn_ds) that walk the key tiles of 256 together, the K rows of
@@ -406,6 +592,14 @@ static void launch_attn_p(hipStream_t s, const void *q, const void *k, const uin
 }
 
 template <int DT, int HD>
+static void launch_attn_fwd(hipStream_t s, const void *q, const void *k, const void *v, const uint32_t *seg, void *p16,
+                            float *out32, void *out16, int64_t nbh, int T, int H, float scale, int causal) {
+    const dim3 grid((unsigned)((T + 31) / 32), (unsigned)nbh);
+    hipLaunchKernelGGL((k_attn_fwd<DT, HD>), grid, dim3(256), 0, s, (const uint16_t *)q, (const uint16_t *)k,
+                       (const uint16_t *)v, seg, (uint16_t *)p16, out32, (uint16_t *)out16, T, H, scale, causal);
+}
+
+template <int DT, int HD>
 static void launch_attn_ds(hipStream_t s, const void *dout, const void *v, const void *p16, const float *rowsub, void *ds16,
                            int64_t nbh, int T, float scale, int causal) {
     const dim3 grid((unsigned)((T + DS_BN - 1) / DS_BN), (unsigned)((T + DS_BM - 1) / DS_BM), (unsigned)nbh);
@@ -442,6 +636,32 @@ int mg_tk_attn_p(mg_ctx *ctx, const void *q16, const void *k16, const uint32_t *
         else launch_attn_p<MG_BF16, 128>(s, q16, k16, seg, p16, nbh, t, h, scale, c);
     }
     EW_POSTCHECK("mg_tk_attn_p");
+}
+
+int mg_tk_attn_fwd_supported(int64_t hd, int64_t T) {
+    return (hd == 32 || hd == 64 || hd == 128) && T > 0 && T % 8 == 0 && T <= 1024;
+}
+
+int mg_tk_attn_fwd(mg_ctx *ctx, const void *q16, const void *k16, const void *v16, const uint32_t *seg, void *p16,
+                   float *out32, void *out16, int64_t nbh, int64_t T, int64_t H, int64_t hd, float scale, int causal,
+                   int dtype) {
+    EW_PRECHECK("mg_tk_attn_fwd", q16 && k16 && v16 && p16 && out32 && nbh > 0 && nbh <= 65535 &&
+                                      mg_tk_attn_fwd_supported(hd, T) && H > 0 && nbh % H == 0 && dtype_ok(dtype) &&
+                                      scale == scale &&
+                                      (((uintptr_t)q16 | (uintptr_t)k16 | (uintptr_t)v16 | (uintptr_t)p16) & 15) == 0 &&
+                                      ((uintptr_t)out32 & 3) == 0 && ((uintptr_t)out16 & 1) == 0 && ((uintptr_t)seg & 3) == 0);
+    hipStream_t s = ctx_stream(ctx);
+    const int t = (int)T, c = causal ? 1 : 0, h = (int)H;
+    if (dtype == MG_F16) {
+        if (hd == 32) launch_attn_fwd<MG_F16, 32>(s, q16, k16, v16, seg, p16, out32, out16, nbh, t, h, scale, c);
+        else if (hd == 64) launch_attn_fwd<MG_F16, 64>(s, q16, k16, v16, seg, p16, out32, out16, nbh, t, h, scale, c);
+        else launch_attn_fwd<MG_F16, 128>(s, q16, k16, v16, seg, p16, out32, out16, nbh, t, h, scale, c);
+    } else {
+        if (hd == 32) launch_attn_fwd<MG_BF16, 32>(s, q16, k16, v16, seg, p16, out32, out16, nbh, t, h, scale, c);
+        else if (hd == 64) launch_attn_fwd<MG_BF16, 64>(s, q16, k16, v16, seg, p16, out32, out16, nbh, t, h, scale, c);
+        else launch_attn_fwd<MG_BF16, 128>(s, q16, k16, v16, seg, p16, out32, out16, nbh, t, h, scale, c);
+    }
+    EW_POSTCHECK("mg_tk_attn_fwd");
 }
 
 int mg_tk_attn_ds(mg_ctx *ctx, const void *dout16, const void *v16, const void *p16, const float *rowsub, void *ds16,

@@ -78,6 +78,10 @@ def make_transformer_kernels(dev, dtype="f16"):
     # buffers: q16, k16, seg (or None), p16 ; n = heads ; args: T, H, hd, scale, causal
     add("attn_p", lambda lib, ctx, p, n, T, H, hd, scale, causal:
         lib.mg_tk_attn_p(ctx, p[0], p[1], p[2], p[3], int(n), int(T), int(H), int(hd), float(scale), int(bool(causal)), dt))
+    # buffers: q16, k16, v16, seg (or None), p16, out32, out16 merged (or None) ; n = heads ; args: T, H, hd, scale, causal
+    add("attn_fwd", lambda lib, ctx, p, n, T, H, hd, scale, causal:
+        lib.mg_tk_attn_fwd(ctx, p[0], p[1], p[2], p[3], p[4], p[5], p[6], int(n), int(T), int(H), int(hd), float(scale),
+                           int(bool(causal)), dt))
     # buffers: dout16, v16, p16, rowsub, ds16 ; n = heads ; args: T, hd, scale, causal
     add("attn_ds", lambda lib, ctx, p, n, T, hd, scale, causal:
         lib.mg_tk_attn_ds(ctx, p[0], p[1], p[2], p[3], p[4], int(n), int(T), int(hd), float(scale), int(bool(causal)), dt))

@@ -180,6 +180,11 @@ class Attention:
         self.q16, self.k16, self.v16 = (_h16(ctx, nbh, T_, hd) for _ in range(3))
         lib = ctx.dev._lib
         self._one_kernel_p = bool(ctx.fuse and lib.mg_tk_attn_p_supported(self.hd, T))
+        # P, Out = P V and the merged 16-bit copy of Out from one kernel (P is written, not read back).
+        # For heads up to 64 wide: 96 heads x 1024 x 64 take 115 us against 77 + 39 + 8 for P, the
+        # P V GEMM and merge_heads, 32 wide 62 against 103; 128 wide the kernel needs the registers
+        # of a whole SIMD lane and loses (167 against 133 us).
+        self._one_kernel_fwd = bool(ctx.fuse and self.hd <= 64 and lib.mg_tk_attn_fwd_supported(self.hd, T))
         self._one_kernel_ds = bool(ctx.fuse and lib.mg_tk_attn_ds_supported(self.hd, T))
         if self._one_kernel_p:
             # P comes out of one kernel (scores + softmax): no f32 scores.  Wavefronts whose keys all
@@ -231,6 +236,12 @@ class Attention:
         fused = ctx.fuse
         qkv = self.qkv.forward(x16, graph=graph, bias=fused)
         self._permute("split_qkv", [qkv, None if fused else self.qkv.b.w32, self.q16, self.k16, self.v16], graph)
+        if self._one_kernel_fwd:
+            ctx.TK["attn_fwd"]([self.q16, self.k16, self.v16, seg, self.p16, self.ao32, self.ao16], self.nbh, self.T,
+                               self.H, self.hd, self.scale, ctx.causal_gemms, graph=graph)
+            if fused and res is not None:
+                return self.proj.forward(self.ao16, graph=graph, bias=True, res=res, out=out)
+            return self.proj.forward(self.ao16, graph=graph)
         if self._one_kernel_p:
             ctx.TK["attn_p"]([self.q16, self.k16, seg, self.p16], self.nbh, self.T, self.H, self.hd, self.scale,
                              ctx.causal_gemms, graph=graph)
