@@ -393,7 +393,9 @@ k_attn_fwd(const uint16_t *q16, const uint16_t *k16, const uint16_t *v16, const 
 #pragma unroll
                 for (int i = 0; i < NLD; i++) *reinterpret_cast<ak_u32x4 *>(vdst + RPI * i * PITCH) = vreg[i];
                 if (t + 1 < nblk) load_v(t + 1);
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the block is in LDS before it is read back
+                // a wavefront's LDS operations execute in order: the reads below see the block, and the next
+                // block's writes come after them; the compiler only has to keep that order
+                asm volatile("" ::: "memory");
             }
 #pragma unroll
             for (int u = 0; u < 2; u++) {
@@ -413,7 +415,7 @@ k_attn_fwd(const uint16_t *q16, const uint16_t *k16, const uint16_t *v16, const 
                     }
                 }
             }
-            if (mul) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // read back before the next block overwrites it
+            if (mul) asm volatile("" ::: "memory");
         }
     }
     __syncthreads();                         // every wavefront is done with its V buffer
