@@ -298,6 +298,12 @@ def test_plans_tuned_in_context(tmp_path, monkeypatch):
     import vkgrad_amd.kernels as K
     monkeypatch.setattr(K, "_TUNE_CACHE", str(tmp_path / "tune.json"))
     monkeypatch.setattr(K, "_SHIPPED_CACHE", str(tmp_path / "none.json"))
+    # operand sets of a timing loop: sized by what a launch reads, so that a rotation's reads are twice the cache
+    mb = 1 << 20
+    assert K.buffer_sets_for(600 * mb) == 1 and K.buffer_sets_for(512 * mb) == 1
+    assert K.buffer_sets_for(17 * mb) == 32 and K.buffer_sets_for(1) == 32
+    assert K.buffer_sets_for(90 * mb) == 7 and K.buffer_sets_for(268 * mb) == 3 and K.buffer_sets_for(300 * mb) == 3
+    assert all(K.buffer_sets_for(r * mb) * r >= 512 for r in (20, 50, 64, 100, 128, 200, 255))
     cands = K.plan_candidates(3072, 768, 8192, K.L.MG_TN)
     assert len(cands) > 20 and cands[0]["split_k"] == 1
     names = {K.CONFIGS[c["tile_id"]]["name"] for c in cands}
