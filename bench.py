@@ -91,9 +91,9 @@ def plan_for(dev, name, layout, m, n, k, vpitch, context=None):
 
 
 def context_of(schedule):
-    """Name under which plans tuned inside a step of this schedule are kept (None: a GEMM has the
-    chip to itself, the plans tuned alone apply)."""
-    return None if schedule == "in-order" else "gpt2s-" + schedule
+    """Name under which plans tuned inside a step of this schedule are kept (where the table has
+    none for it, the plans tuned alone apply)."""
+    return "gpt2s-" + schedule
 
 # HBM-side bytes per launch (L2 fetches + L2 write-backs) of each GEMM of the step,
 # measured on MI355X with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over
@@ -268,8 +268,6 @@ def tune_step(dev, args, vpitch, context, step_calls, record):
     time of the whole replayed step; the picks go to the tuner's cache under `context`."""
     import statistics
     from vkgrad_amd import kernels as K
-    if context is None:
-        sys.exit("bench.py --tune-step: the in-order schedule uses the plans tuned alone (kernels.autotune_matmul)")
     fields = ("tile_id", "split_k", "atomic_split", "group_m", "xcd_rotate")
     slots, meta = {}, {}
     for name, layout, m, n, k, _ in gemm_list():
@@ -620,7 +618,8 @@ def main():
     }
     if args.schedule != "in-order":
         # the same step with every GEMM behind the previous one on one stream
-        idt, _ = time_steps(step_calls(vpitch, None), "gpt2_small_gemms_in_order", args.steps, args.warmup, "in-order")
+        idt, _ = time_steps(step_calls(vpitch, context_of("in-order")), "gpt2_small_gemms_in_order", args.steps, args.warmup,
+                            "in-order")
         out["in_order"] = {"schedule": SCHEDULES["in-order"], "value": round(step_flops / (idt / args.steps) / 1e12, 2),
                            "unit": "TFLOP/s", "ms_per_step": round(idt / args.steps * 1e3, 4)}
     if each is not None:
