@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the training-GEMM path on one MI355X.
 
-One step = every GEMM of one GPT-2-small training step (BASELINE.json configs[2]):
+One step = every GEMM of one GPT-2-small training step (the GPT-2-small configuration of the workload list):
 d_model 768, 12 layers, 8 x 1024 = 8192 token rows, per layer QKV 768->2304,
 proj 768->768, MLP 768->3072->768, plus the tied LM head 768->50257; for every
 linear the forward, dX and dW products (147 GEMMs, 6.07 TFLOP), bf16 inputs,
@@ -175,7 +175,7 @@ MLP_SIZES, MLP_BATCH, MLP_CLASSES = (784, 512, 512), 128, 10
 
 
 def mlp_step_device(dev, steps=300):
-    """BASELINE configs[0] on the device: the synthetic-MNIST MLP train step (batch 128, 784 ->
+    """The MLP configuration on the device: the synthetic-MNIST MLP train step (batch 128, 784 ->
     512 -> 512 -> 10, ReLU, He-normal weights, f16, fwd + dX + dW + bias gradients + AdamW)
     recorded once and replayed as one HIP graph; microseconds per step including the read-back
     of the loss, as the reference's TrainStep measures it (bench/mnist-repro.json:5-24)."""

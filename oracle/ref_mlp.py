@@ -151,7 +151,7 @@ def he_init(sizes_full, seed):
 
 
 def synthetic_batch(batch, n_in, n_classes, seed=0, dtype="f16"):
-    """BASELINE config 1 inputs: x uniform[0,1) rounded to the 16-bit type,
+    """Inputs of the MLP configuration: x uniform[0,1) rounded to the 16-bit type,
     integer labels uniform over the classes."""
     rng = np.random.default_rng(seed)
     x = rng.random((batch, n_in), dtype=np.float32)

@@ -1,4 +1,4 @@
-"""Parity at BASELINE.json's full sizes, through size-independent properties.
+"""Parity at the full sizes of the workload configurations, through size-independent properties.
 
 The numpy oracle needs seconds to minutes at these sizes, so the full result is
 checked by (a) a random sample of output entries recomputed exactly in float64
@@ -55,7 +55,7 @@ def _checksum_check(got, a, b, ta, tb, dtype):
 @pytest.mark.parametrize("layout", list(LAY))
 @pytest.mark.parametrize("n", [1024, 4096])
 def test_square_sweep_sizes(dev, layout, n):
-    """BASELINE configs[1] (seed 7, f16, ~N(0,1)); 8192^3 runs in the benchmark."""
+    """The square configuration (seed 7, f16, ~N(0,1)); 8192^3 runs in the benchmark."""
     ta, tb = LAY[layout]
     a, b = O.make_operands(n, n, n, ta, tb, "f16", seed=7)
     got = _run(dev, a, b, n, n, n, ta, tb, "f16")
@@ -71,7 +71,7 @@ GPT2 = [("qkv", 768, 2304), ("proj", 768, 768), ("fc1", 768, 3072), ("fc2", 3072
 
 @pytest.mark.parametrize("name,fin,fout", GPT2)
 def test_gpt2_small_linears(dev, name, fin, fout):
-    """BASELINE configs[2]: R=8192, bf16, X~N(0,1), W~N(0,0.02), dY~N(0,1); the
+    """The GPT-2-small configuration: R=8192, bf16, X~N(0,1), W~N(0,0.02), dY~N(0,1); the
     three GEMMs of each linear with W stored out x in (NT fwd, NN dX, TN dW)."""
     R = 8192
     rng = np.random.default_rng(1)
@@ -115,7 +115,7 @@ def test_lm_head_unpadded_vocab(dev):
 @pytest.mark.parametrize("m", [1, 7, 63, 129, 4097])
 @pytest.mark.parametrize("n", [96, 2304, 50257])
 def test_skinny_and_ragged_with_bias(dev, m, n):
-    """BASELINE configs[4]: M x 768 x N, NT, f16, fused bias, non-tile-multiples."""
+    """The skinny configuration: M x 768 x N, NT, f16, fused bias, non-tile-multiples."""
     k = 768
     a, b = O.make_operands(m, n, k, False, True, "f16", seed=3)
     bias = (np.random.default_rng(3).standard_normal(n) * 2 + 1).astype(np.float32)
@@ -126,7 +126,7 @@ def test_skinny_and_ragged_with_bias(dev, m, n):
 
 
 def test_charlm_shapes(dev):
-    """BASELINE configs[4]: char-LM d_model 256, vocab 96, 64 x 256 rows."""
+    """The char-LM configuration: d_model 256, vocab 96, 64 x 256 rows."""
     R = 16384
     for fin, fout in [(256, 768), (256, 256), (256, 1024), (1024, 256), (256, 96)]:
         rng = np.random.default_rng(3)

@@ -1,4 +1,4 @@
-"""GPU parity of the MLP train step (BASELINE config 1) against the numpy model.
+"""GPU parity of the MLP train step (the MLP configuration) against the numpy model.
 
 Protocols follow /root/reference/test_autograd.py: loss within 2e-3 and gradients
 within 2e-2 relative of an independent float32 model (:78-103), AdamW overfits one

@@ -5,7 +5,7 @@ rasterisation band, split mode) from the shipped tuned table.  These tests build
 through the same functions (bench.plan_for, kernels.tuned_matmul) and check it against the
 oracle at full size:
 
-  * every GEMM of the benchmark step (BASELINE configs[2]) with the benchmark's operand
+  * every GEMM of the benchmark step (the GPT-2-small configuration) with the benchmark's operand
     statistics and the LM head's padded logits pitch: sampled exact recomputation in float64
     plus the column-checksum identity (tests/test_fullsize_gpu.py explains both);
   * every entry of the tuned table at the shape, layout, dtype, pitches and batch count it is
