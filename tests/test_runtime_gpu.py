@@ -252,6 +252,48 @@ def test_graph_with_parallel_branches_replays(dev):
                 b.destroy()
 
 
+def test_graph_with_a_free_running_side_chain_replays_back_to_back(dev):
+    """The benchmark's default schedule in small: one fork at the start of the recorded step,
+    the dW GEMMs of several linears queued behind each other on the side stream - an unsplit
+    ping-pong tile, a K split through the side stream's half of the workspace, a persistent
+    tile with a split, an atomic split - beside the dX chain on the main stream (one of them
+    split through the main half), one join at the end.  Replays are enqueued back to back
+    without a synchronisation in between, as the benchmark times them; afterwards every
+    product must be exact (integer data), and again after a second burst."""
+    from vkgrad_amd.kernels import Matmul
+    rows = 2048
+    dims = [(512, 768), (768, 256), (256, 1024), (1024, 512)]
+    cases = [_linear_backward_case(dev, rows, fin, fout, 51 + 2 * i) for i, (fin, fout) in enumerate(dims)]
+    dw_plans = [dict(tile=21), dict(tile=11, split_k=2), dict(tile=17, split_k=4), dict(tile=14, split_k=3, atomic_split=True)]
+    dx_plans = [dict(tile=11), dict(tile=21), dict(tile=11, split_k=2), dict(tile=14)]
+    mm_dw = [Matmul(dev, trans_a=True, dtype="bf16", **kw) for kw in dw_plans]
+    mm_dx = [Matmul(dev, dtype="bf16", **kw) for kw in dx_plans]
+    g = dev.graph("free_side_chain")
+    g.fork()
+    for (bufs, _, _), (fin, fout), dx, dw in zip(cases, dims, mm_dx, mm_dw):
+        dx(bufs["dy"], bufs["w"], bufs["dx"], rows, fin, fout, graph=g)
+        dw(bufs["dy2"], bufs["x"], bufs["dw"], fout, fin, rows, graph=g, side=True)
+    g.finish()
+    try:
+        for burst in range(2):
+            for (bufs, _, _), (fin, fout) in zip(cases, dims):
+                bufs["dx"].upload(np.full((rows, fin), np.nan, np.float32))
+                bufs["dw"].upload(np.full((fout, fin), np.nan, np.float32))
+            for _ in range(6):
+                g.enqueue()
+            dev.sync()
+            for j, ((bufs, ref_dx, ref_dw), (fin, fout)) in enumerate(zip(cases, dims)):
+                assert np.array_equal(bufs["dx"].download(np.float32, (rows, fin)), ref_dx), f"burst {burst} dX {j}"
+                assert np.array_equal(bufs["dw"].download(np.float32, (fout, fin)), ref_dw), f"burst {burst} dW {j}"
+    finally:
+        g.destroy()
+        for m in mm_dw + mm_dx:
+            m.destroy()
+        for bufs, _, _ in cases:
+            for b in bufs.values():
+                b.destroy()
+
+
 def test_elementwise_kernels(dev):
     from vkgrad_amd.kernels import make_kernels
     from oracle import ref_mlp as RM
